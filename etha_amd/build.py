@@ -1,0 +1,51 @@
+"""Build recipe for the HIP library (gfx950 only).
+
+``python -m etha_amd.build`` compiles ``csrc/etha_reshard.hip`` into
+``etha_amd/libetha_reshard.so`` next to this file.  hipcc cross-compiles, so no GPU is needed.
+"""
+
+from __future__ import annotations
+
+import os
+import shutil
+import subprocess
+import sys
+
+PKG_DIR = os.path.dirname(os.path.abspath(__file__))
+REPO_DIR = os.path.dirname(PKG_DIR)
+SOURCE = os.path.join(PKG_DIR, "csrc", "etha_reshard.hip")
+INCLUDE_DIR = os.path.join(REPO_DIR, "include")
+LIB_PATH = os.path.join(PKG_DIR, "libetha_reshard.so")
+
+HIPCC_FLAGS = [
+    "-O3",
+    "--offload-arch=gfx950",
+    # keep the compiler from forming packed fp32 instructions
+    "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
+    "-fPIC",
+    "-shared",
+    "-std=c++17",
+]
+
+
+def hipcc_path() -> str:
+    path = shutil.which("hipcc") or "/opt/rocm/bin/hipcc"
+    if not os.path.exists(path):
+        raise RuntimeError("hipcc not found; the ROCm toolchain is required to build etha_amd")
+    return path
+
+
+def build_library(verbose: bool = False) -> str:
+    """Compile the shared library (always recompiles) and return its path."""
+    cmd = [hipcc_path(), *HIPCC_FLAGS, f"-I{INCLUDE_DIR}", "-o", LIB_PATH + ".tmp", SOURCE]
+    proc = subprocess.run(cmd, capture_output=True, text=True)
+    if proc.returncode != 0:
+        raise RuntimeError(f"hipcc failed ({proc.returncode}):\n{' '.join(cmd)}\n{proc.stdout}\n{proc.stderr}")
+    if verbose and proc.stderr:
+        sys.stderr.write(proc.stderr)
+    os.replace(LIB_PATH + ".tmp", LIB_PATH)
+    return LIB_PATH
+
+
+if __name__ == "__main__":
+    print(build_library(verbose=True))

@@ -1,0 +1,175 @@
+"""Executor: run planned buckets on the GPU.
+
+Counterpart of ``bucket_comm`` (``src/etha/comm/comm_methods.py:53-119``).  The reference walks
+per-key channels through prepare -> launch -> complete -> finalize with one ATen launch per chunk.
+Here a bucket list is compiled once into tile programs and a call enqueues, in bucket-list order:
+
+* source buckets:  one pack (or reduce-pack) launch each - ``Bucket.prepare``;
+* the wire step:   nothing to do, the consumer reads the producer's pool slot;
+* target buckets:  one unpack launch each - ``Bucket.finalize``;
+* LOCAL buckets:   one direct self-copy launch each, or pack + unpack through a private slot when
+                   source and destination bytes may overlap;
+* NONE buckets:    nothing - the primary's reduce-pack already read this member's partial.
+
+Consecutive buckets of the same kind can be merged into one launch (``merge_launches=True``).
+All work goes to one stream, so per-channel FIFO order and "pack before unpack" hold by stream
+order; the call returns after synchronising that stream, like the reference's final
+``torch.cuda.synchronize()`` (``comm_methods.py:119``).
+"""
+
+from __future__ import annotations
+
+import torch
+
+from .device_plan import DescBuilder, SelfCopyBuilder, local_bucket_needs_staging
+from .ir import Bucket
+from .transfer import Transport
+
+__all__ = ["bucket_comm", "TransferPlan"]
+
+_PACK, _REDUCE, _UNPACK, _SELF = "pack", "reduce_pack", "unpack", "selfcopy"
+
+
+class TransferPlan:
+    """Compiled form of one rank's bucket list."""
+
+    def __init__(self, wire, buckets: list[Bucket]):
+        self.wire = wire
+        self.buckets = buckets
+        self.device: torch.device | None = None
+        send, recv, local = DescBuilder(), DescBuilder(), SelfCopyBuilder()
+        # steps: (kind, first_chunk, n_chunks, slot or None), in execution order
+        self.steps: list[tuple[str, int, int, object]] = []
+        send_index: dict[tuple, int] = {}
+        recv_index: dict[tuple, int] = {}
+        from .loopback import wire_key
+
+        for bucket in buckets:
+            if not bucket.chunks:
+                continue
+            first_tensor = bucket.chunks[0].tensor
+            if first_tensor is None:
+                raise ValueError(f"{bucket}: chunks without a tensor cannot be executed")
+            device = first_tensor.device
+            if device.type != "cuda":
+                raise RuntimeError(
+                    f"{bucket}: tensors live on {device}; this executor only runs on a GPU (there is no CPU path)"
+                )
+            if self.device is None:
+                self.device = device
+            elif device != self.device:
+                raise RuntimeError("all buckets of one call must live on the same GPU")
+            transport = bucket.transport
+            if transport == Transport.NONE:
+                continue
+            if transport == Transport.LOCAL:
+                if local_bucket_needs_staging(bucket):
+                    slot = wire.private_slot(bucket.total_bytes, device)
+                    f_send, f_recv = len(send), len(recv)
+                    for off, c in zip(bucket.offsets, bucket.chunks):
+                        src_t = c.src_tensor if c.src_tensor is not None else c.tensor
+                        send.add_chunk(c, src_t, c.src_slice, slot, off, reduce=False)
+                        recv.add_chunk(c, c.tensor, c.dst_slice, slot, off, reduce=False)
+                    self.steps.append((_PACK, f_send, len(bucket.chunks), slot))
+                    self.steps.append((_UNPACK, f_recv, len(bucket.chunks), slot))
+                else:
+                    first = len(local)
+                    for c in bucket.chunks:
+                        local.add_chunk(c)
+                    self.steps.append((_SELF, first, len(bucket.chunks), None))
+                continue
+            key = wire_key(bucket)
+            if bucket.is_source:
+                idx = send_index.get(key, 0)
+                send_index[key] = idx + 1
+                slot = wire.slot_for_send(bucket, idx, device)
+                first = len(send)
+                reduce = bool(bucket.chunks[0].source_partial_groups)
+                for off, c in zip(bucket.offsets, bucket.chunks):
+                    send.add_chunk(c, c.tensor, c.src_slice, slot, off, reduce=reduce)
+                self.steps.append((_REDUCE if reduce else _PACK, first, len(bucket.chunks), slot))
+            elif bucket.is_target:
+                idx = recv_index.get(key, 0)
+                recv_index[key] = idx + 1
+                slot = wire.slot_for_recv(bucket, idx)
+                first = len(recv)
+                for off, c in zip(bucket.offsets, bucket.chunks):
+                    recv.add_chunk(c, c.tensor, c.dst_slice, slot, off, reduce=False)
+                self.steps.append((_UNPACK, first, len(bucket.chunks), slot))
+        self._keepalive = send.keepalive + recv.keepalive + local.keepalive
+        self.send_table = send.build()
+        self.recv_table = recv.build()
+        self.local_table = local.build()
+        self.merged_steps = self._merge(self.steps)
+
+    @staticmethod
+    def _merge(steps):
+        merged: list[list] = []
+        for kind, first, count, slot in steps:
+            if merged and merged[-1][0] == kind and merged[-1][1] + merged[-1][2] == first:
+                merged[-1][2] += count
+                merged[-1][3].append(slot)
+            else:
+                merged.append([kind, first, count, [slot]])
+        return [(k, f, c, tuple(s)) for k, f, c, s in merged]
+
+    def run(self, stream: int | None = None, merge_launches: bool = False) -> None:
+        if self.device is None:
+            return
+        if stream is None:
+            stream = torch.cuda.current_stream(self.device).cuda_stream
+        steps = self.merged_steps if merge_launches else [(k, f, c, (s,)) for k, f, c, s in self.steps]
+        with torch.cuda.device(self.device):
+            for kind, first, count, slots in steps:
+                if kind == _PACK:
+                    self.send_table.pack(first, count, stream)
+                elif kind == _REDUCE:
+                    self.send_table.reduce_pack(first, count, stream)
+                elif kind == _UNPACK:
+                    for s in slots:
+                        if s is not None and s.filled == 0:
+                            raise RuntimeError(
+                                "recv bucket runs before its send bucket was ever packed "
+                                "(a real wire would block here)"
+                            )
+                    self.recv_table.unpack(first, count, stream)
+                else:
+                    self.local_table.selfcopy(first, count, stream)
+                if kind in (_PACK, _REDUCE):
+                    for s in slots:
+                        if s is not None:
+                            s.filled += 1
+
+    def payload_bytes(self) -> dict[str, int]:
+        out = {}
+        for name, table in (("send", self.send_table), ("recv", self.recv_table), ("local", self.local_table)):
+            out[name] = table.info().payload_bytes if table is not None else 0
+        return out
+
+
+def bucket_comm(
+    buckets: list[Bucket],
+    max_in_flight: int = 2,
+    *,
+    wire=None,
+    merge_launches: bool = False,
+    synchronize: bool = True,
+) -> None:
+    """Run the bucket pipeline for one rank's buckets.
+
+    ``max_in_flight`` is accepted for compatibility; every bucket owns a persistent pool slot, so
+    there is nothing to throttle.  The keyword-only arguments are additions: ``wire`` selects the
+    loopback wire (default: the process-wide one), ``merge_launches`` fuses consecutive buckets of
+    one kind into a single launch, ``synchronize=False`` leaves the stream un-synchronised.
+    """
+    del max_in_flight
+    if wire is None:
+        from .loopback import default_wire
+
+        wire = default_wire()
+    if not buckets:
+        return
+    plan = wire.plan(buckets)
+    plan.run(merge_launches=merge_launches)
+    if synchronize and plan.device is not None:
+        torch.cuda.current_stream(plan.device).synchronize()

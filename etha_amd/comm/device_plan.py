@@ -1,0 +1,198 @@
+"""From planner objects to the flat chunk-descriptor table the HIP library consumes.
+
+Everything here runs once per registered batch ("plan once, transfer N times"): chunks are
+turned into ``EthaChunkDesc`` rows (``include/etha_reshard.h``), the library compiles them into a
+device-resident tile program, and a transfer is then a handful of kernel launches.  This is the
+replacement for the per-transfer Python loops of ``Bucket.prepare`` / ``Bucket.finalize``
+(``src/etha/comm/ir.py:246-259,306-308``).
+"""
+
+from __future__ import annotations
+
+from dataclasses import dataclass
+
+import numpy as np
+import torch
+
+from .. import _native as nat
+from .ir import Bucket, Chunk
+
+_FLOAT_CODES = {
+    torch.float16: nat.F16,
+    torch.bfloat16: nat.BF16,
+    torch.float32: nat.F32,
+    torch.float64: nat.F64,
+}
+_OPAQUE_CODES = {1: nat.B8, 2: nat.B16, 4: nat.B32, 8: nat.B64}
+
+
+def dtype_code(dtype: torch.dtype) -> int:
+    if dtype in _FLOAT_CODES:
+        return _FLOAT_CODES[dtype]
+    code = _OPAQUE_CODES.get(dtype.itemsize)
+    if code is None:
+        raise NotImplementedError(f"dtype {dtype} (itemsize {dtype.itemsize}) is not supported")
+    return code
+
+
+def check_cast(src: torch.dtype, dst: torch.dtype) -> None:
+    """Same dtype is a byte move; otherwise both must be floating (fp16/bf16/fp32/fp64)."""
+    if src != dst and not (src in _FLOAT_CODES and dst in _FLOAT_CODES):
+        raise NotImplementedError(f"conversion {src} -> {dst} is only implemented between floating dtypes")
+
+
+def _storage_range(t: torch.Tensor) -> tuple[int, int]:
+    st = t.untyped_storage()
+    lo = st.data_ptr()
+    return lo, lo + st.nbytes()
+
+
+def fill_region(row, tensor: torch.Tensor, slices: tuple, chunk_shape: tuple) -> None:
+    """Tensor-side fields of one descriptor row: pointer, strides, slice starts, chunk shape."""
+    nd = tensor.dim()
+    if nd > nat.ETHA_MAX_NDIM:
+        raise NotImplementedError(f"tensors of more than {nat.ETHA_MAX_NDIM} dims are not supported")
+    if len(slices) > nd:
+        raise ValueError(f"slice of rank {len(slices)} on a tensor of rank {nd}")
+    shape = tuple(tensor.shape)
+    starts, extents = [], []
+    for d in range(nd):
+        if d < len(slices):
+            s = slices[d]
+            if s.step not in (None, 1):
+                raise NotImplementedError("chunk slices must have unit step")
+            lo, hi, _ = s.indices(shape[d])
+            starts.append(lo)
+            extents.append(max(hi - lo, 0))
+        else:
+            starts.append(0)
+            extents.append(shape[d])
+    cs = tuple(chunk_shape)
+    if nd == 0:
+        if int(np.prod(cs, dtype=np.int64)) != 1:
+            raise ValueError(f"chunk_shape {cs} does not match a scalar tensor")
+    elif tuple(extents) != cs:
+        raise ValueError(f"chunk_shape {cs} does not match the slice extents {tuple(extents)} of tensor {shape}")
+    row["tensor_ptr"] = tensor.data_ptr()
+    lo, hi = _storage_range(tensor)
+    row["tensor_lo"], row["tensor_hi"] = lo, hi
+    row["ndim"] = nd
+    row["start"][:nd] = starts
+    row["shape"][:nd] = extents
+    row["stride"][:nd] = tensor.stride()
+    row["tensor_dtype"] = dtype_code(tensor.dtype)
+
+
+@dataclass
+class Slot:
+    """A bucket buffer inside the pool."""
+
+    ptr: int
+    nbytes: int
+    lo: int  # bounds of the allocation holding the slot
+    hi: int
+    filled: int = 0  # number of times a pack has been enqueued into this slot
+    drained: int = 0  # number of unpacks enqueued from it (per consumer bookkeeping is the wire's job)
+
+
+class DescBuilder:
+    """Accumulates descriptor rows bucket by bucket and remembers each bucket's chunk range."""
+
+    def __init__(self) -> None:
+        self.rows: list[np.ndarray] = []
+        self.partial_ptrs: list[int] = []
+        self.keepalive: list[torch.Tensor] = []
+
+    def __len__(self) -> int:
+        return len(self.rows)
+
+    def add_chunk(self, chunk: Chunk, tensor: torch.Tensor, slices: tuple, slot: Slot, offset: int,
+                  reduce: bool) -> None:
+        row = np.zeros((), dtype=nat.CHUNK_DESC)
+        fill_region(row, tensor, slices, chunk.chunk_shape)
+        wire = chunk.transfer_dtype or tensor.dtype
+        check_cast(tensor.dtype, wire)
+        row["wire_dtype"] = dtype_code(wire)
+        row["bucket_ptr"] = slot.ptr + offset
+        row["bucket_lo"], row["bucket_hi"] = slot.ptr, slot.ptr + slot.nbytes
+        peers = chunk.partial_peers() if reduce else None
+        if peers is not None:
+            tensors, op = peers
+            for t in tensors:
+                if t.dtype != tensor.dtype or tuple(t.shape) != tuple(tensor.shape) or t.stride() != tensor.stride():
+                    raise NotImplementedError("Partial peers must share dtype, shape and strides")
+                if t.device != tensor.device:
+                    raise NotImplementedError("Partial peers must live on the same GPU")
+            row["n_partials"] = len(tensors)
+            row["partial_first"] = len(self.partial_ptrs)
+            row["reduce_op"] = nat.REDUCE_OPS[op]
+            self.partial_ptrs.extend(t.data_ptr() for t in tensors)
+            self.keepalive.extend(tensors)
+        self.keepalive.append(tensor)
+        self.rows.append(row)
+
+    def build(self) -> nat.Table | None:
+        if not self.rows:
+            return None
+        descs = np.stack(self.rows)
+        ptrs = np.asarray(self.partial_ptrs, dtype=np.uint64) if self.partial_ptrs else None
+        return nat.Table.create(descs, ptrs, upload=True)
+
+
+class SelfCopyBuilder:
+    def __init__(self) -> None:
+        self.src: list[np.ndarray] = []
+        self.dst: list[np.ndarray] = []
+        self.keepalive: list[torch.Tensor] = []
+
+    def __len__(self) -> int:
+        return len(self.src)
+
+    def add_chunk(self, chunk: Chunk) -> None:
+        src_t = chunk.src_tensor if chunk.src_tensor is not None else chunk.tensor
+        a = np.zeros((), dtype=nat.CHUNK_DESC)
+        b = np.zeros((), dtype=nat.CHUNK_DESC)
+        fill_region(a, src_t, chunk.src_slice, chunk.chunk_shape)
+        fill_region(b, chunk.tensor, chunk.dst_slice, chunk.chunk_shape)
+        check_cast(src_t.dtype, chunk.tensor.dtype)
+        a["wire_dtype"] = a["tensor_dtype"]
+        b["wire_dtype"] = b["tensor_dtype"]
+        self.src.append(a)
+        self.dst.append(b)
+        self.keepalive += [src_t, chunk.tensor]
+
+    def build(self) -> nat.Table | None:
+        if not self.src:
+            return None
+        return nat.Table.create_selfcopy(np.stack(self.src), np.stack(self.dst), upload=True)
+
+
+def region_hull(tensor: torch.Tensor, slices: tuple) -> tuple[int, int]:
+    """Smallest byte interval covering ``tensor[slices]`` (empty regions give lo == hi)."""
+    view = tensor[slices] if slices else tensor
+    if view.numel() == 0:
+        return view.data_ptr(), view.data_ptr()
+    span = sum((n - 1) * s for n, s in zip(view.shape, view.stride()))
+    lo = view.data_ptr()
+    return lo, lo + (span + 1) * view.element_size()
+
+
+def local_bucket_needs_staging(bucket: Bucket) -> bool:
+    """True when some chunk's source bytes may overlap some chunk's destination bytes.
+
+    The reference stages a bundled self-copy bucket through the bucket buffer - all reads happen
+    before all writes (``ir.py:246-259,306-308``).  A direct copy gives the same result exactly
+    when no source region overlaps a destination region, which is the common case.
+    """
+    srcs, dsts = [], []
+    for c in bucket.chunks:
+        src_t = c.src_tensor if c.src_tensor is not None else c.tensor
+        srcs.append(region_hull(src_t, c.src_slice))
+        dsts.append(region_hull(c.tensor, c.dst_slice))
+    if len(bucket.chunks) == 1:
+        return False  # single-entry path of the reference copies directly (ir.py:238-244)
+    for s_lo, s_hi in srcs:
+        for d_lo, d_hi in dsts:
+            if s_lo < d_hi and d_lo < s_hi:
+                return True
+    return False

@@ -1,0 +1,230 @@
+"""Plan objects of the redistribute path: routes, chunks, buckets.
+
+Same names, fields and meaning as the reference's IR (``src/etha/comm/ir.py``): ``Endpoint``,
+``Route`` and ``M2MMap`` (``ir.py:16-48``) describe the shape-free mesh-to-mesh topology,
+``Chunk`` (``ir.py:60-169``) one strided tensor region and its role, ``Bucket``
+(``ir.py:172-310``) a group of chunks that travel as one contiguous buffer.
+
+Differences, all additive:
+
+* the byte work of ``Chunk.prepare/finalize`` and ``Bucket.prepare/finalize`` is not done here
+  with per-chunk tensor ops; buckets are compiled into a device tile program
+  (:mod:`etha_amd.comm.device_plan`) and run as batched HIP launches;
+* a Partial source is described by :class:`PartialGroup` objects (the peers' tensors, all resident
+  on this GPU) instead of ``ProcessGroup`` handles;
+* ``Chunk.rank`` records the rank the chunk was built for, and ``Chunk.src_tensor`` lets a LOCAL
+  chunk read a source tensor that is a different object than its target tensor.
+"""
+
+from __future__ import annotations
+
+import math
+from dataclasses import dataclass, field
+from typing import Any
+
+import torch
+
+from .transfer import Transport
+
+REDUCE_OPS = ("sum", "avg", "max", "min", "product")  # ir.py:51-57
+
+
+@dataclass(frozen=True)
+class Endpoint:
+    """A chunk location: a rank and its cell (multi-index) in the transfer grid."""
+
+    rank: int
+    cell: tuple[int, ...]
+
+
+@dataclass(frozen=True)
+class Route:
+    """Delivery plan of one source cell: ``src`` to every endpoint in ``dsts``.
+
+    ``kind`` is NONE for a reduce-only entry (no dsts), P2P for one dst, BROADCAST for several.
+    """
+
+    src: Endpoint
+    dsts: tuple[Endpoint, ...]
+    kind: Transport
+
+
+@dataclass
+class M2MMap:
+    """Mesh-to-mesh topology; independent of tensor shapes and reusable across batches.
+
+    The first four fields are the reference's (``ir.py:36-48``).  The remaining ones record the
+    two layouts so that chunk building can treat unevenly sharded dims.
+    """
+
+    routes: list[Route] | None = None
+    source_num_slicers: list[int] | None = None
+    target_num_slicers: list[int] | None = None
+    source_partial_reductions: list[tuple[int, str]] = field(default_factory=list)
+    source_mesh: Any = None  # nested list of ranks
+    source_placements: tuple = ()
+    target_mesh: Any = None
+    target_placements: tuple = ()
+
+
+@dataclass(eq=False)
+class PartialGroup:
+    """The members of one Partial reduction as seen from one GPU.
+
+    ``ranks`` are in ascending order; ``tensors[i]`` is rank ``ranks[i]``'s local partial
+    tensor.  Stands in for the ``ProcessGroup`` of ``Chunk.source_partial_groups`` (``ir.py:84``):
+    the reduce kernel reads the peers directly instead of running a collective.
+    """
+
+    ranks: tuple[int, ...]
+    tensors: tuple[torch.Tensor, ...]
+
+    def __post_init__(self) -> None:
+        self.ranks = tuple(self.ranks)
+        self.tensors = tuple(self.tensors)
+        if len(self.ranks) != len(self.tensors):
+            raise ValueError("PartialGroup needs one tensor per rank")
+        if list(self.ranks) != sorted(self.ranks):
+            raise ValueError("PartialGroup ranks must be ascending (reduction order is rank order)")
+
+
+@dataclass(kw_only=True, eq=False)
+class Chunk:
+    """A shape-dependent transfer descriptor: one tensor region plus its role."""
+
+    transport: Transport
+    is_source: bool
+    is_target: bool
+    src_rank: int
+    dst_ranks: tuple[int, ...]
+    chunk_shape: tuple[int, ...]
+    tensor: torch.Tensor | None = None
+    src_slice: tuple[slice, ...] = ()  # read here when is_source
+    dst_slice: tuple[slice, ...] = ()  # written here when is_target
+    transfer_dtype: torch.dtype | None = None  # wire dtype; None = tensor.dtype
+    src_idx: tuple = ()
+    dst_idx: tuple | None = None
+    source_partial_groups: list[tuple[PartialGroup, str]] | None = None
+    buffer: torch.Tensor | None = None
+    # additions
+    rank: int | None = None  # rank this chunk was materialised for
+    src_tensor: torch.Tensor | None = None  # LOCAL chunks: tensor that src_slice indexes (default: tensor)
+
+    def __post_init__(self) -> None:
+        if self.transfer_dtype is None and self.tensor is not None:
+            self.transfer_dtype = self.tensor.dtype
+        self.chunk_shape = tuple(int(n) for n in self.chunk_shape)
+        self.dst_ranks = tuple(self.dst_ranks)
+
+    def __repr__(self) -> str:
+        role = ("S" if self.is_source else "") + ("T" if self.is_target else "") or "-"
+        return f"Chunk({self.transport.name[:3]}/{role}, src={self.src_rank}->{self.dst_ranks}, shape={self.chunk_shape})"
+
+    @property
+    def partial_signature(self) -> tuple:
+        if not self.source_partial_groups:
+            return ()
+        return tuple((g.ranks, op) for g, op in self.source_partial_groups)
+
+    @property
+    def bucket_key(self) -> tuple:
+        """Grouping key, as ``ir.py:143-164``.
+
+        ``(src_rank, dst_ranks, partial signature, cell key, transport)``; the cell key is only
+        set for reduce-only chunks so that they never bundle across cells.  The partial signature
+        is built from the group's ranks and op (the reference uses ``id(group)``; equal for
+        equal groups either way).
+        """
+        cell_key: tuple = ()
+        if self.source_partial_groups and not self.dst_ranks:
+            cell_key = tuple(self.src_idx)
+        return (self.src_rank, self.dst_ranks, self.partial_signature, cell_key, self.transport)
+
+    @property
+    def nbytes(self) -> int:
+        """Byte size on the wire (``ir.py:166-169``)."""
+        return math.prod(self.chunk_shape) * self.transfer_dtype.itemsize
+
+    # -- reduction description used by the device plan ------------------------------------
+    def partial_peers(self) -> tuple[tuple[torch.Tensor, ...], str] | None:
+        """Peers (rank order) and op of this chunk's Partial collapse, or None.
+
+        The reference runs one in-place all-reduce per group in sequence (``ir.py:123-124``); with
+        one op that equals a single reduction over the union of the groups' members, which is
+        what is returned here.  Different ops on different mesh dims are not supported.
+        """
+        if not self.source_partial_groups:
+            return None
+        ops = {op for _, op in self.source_partial_groups}
+        if len(ops) != 1:
+            raise NotImplementedError(f"Partial dims with different reduce ops {sorted(ops)} are not supported")
+        op = ops.pop()
+        if op not in REDUCE_OPS:
+            raise ValueError(f"unknown reduce op {op!r}")
+        members: dict[int, torch.Tensor] = {}
+        for group, _ in self.source_partial_groups:
+            for r, t in zip(group.ranks, group.tensors):
+                members[r] = t
+        ranks = sorted(members)
+        return tuple(members[r] for r in ranks), op
+
+
+@dataclass(kw_only=True, eq=False)
+class Bucket:
+    """A transfer unit: one contiguous buffer holding its chunks back to back.
+
+    Identity (transport, role, ranks, key) is uniform over the chunks and read from the first
+    one; ``offsets`` is the un-padded prefix sum of ``chunk.nbytes`` (``ir.py:189-194``).
+    """
+
+    chunks: list[Chunk]
+    device: torch.device | None = None
+    buffer: torch.Tensor | None = None
+    offsets: list[int] = field(init=False)
+
+    def __post_init__(self) -> None:
+        cursor, offsets = 0, []
+        for chunk in self.chunks:
+            offsets.append(cursor)
+            cursor += chunk.nbytes
+        self.offsets = offsets
+        self._total = cursor
+
+    @property
+    def transport(self) -> Transport:
+        return self.chunks[0].transport
+
+    @property
+    def is_source(self) -> bool:
+        return self.chunks[0].is_source
+
+    @property
+    def is_target(self) -> bool:
+        return self.chunks[0].is_target
+
+    @property
+    def src_rank(self) -> int:
+        return self.chunks[0].src_rank
+
+    @property
+    def dst_ranks(self) -> tuple[int, ...]:
+        return self.chunks[0].dst_ranks
+
+    @property
+    def key(self) -> tuple:
+        return self.chunks[0].bucket_key
+
+    @property
+    def rank(self) -> int | None:
+        return self.chunks[0].rank
+
+    @property
+    def total_bytes(self) -> int:
+        return self._total
+
+    def __repr__(self) -> str:
+        role = ("S" if self.is_source else "") + ("T" if self.is_target else "") or "-"
+        return (
+            f"Bucket({self.transport.name[:3]}/{role}, n={len(self.chunks)}, bytes={self.total_bytes}, "
+            f"src={self.src_rank}->{self.dst_ranks})"
+        )

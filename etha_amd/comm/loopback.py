@@ -1,0 +1,148 @@
+"""The wire step of this build: a same-GPU loopback.
+
+In the reference a prepared bucket crosses ranks with ``dist.isend/irecv`` or a sub-group
+``dist.broadcast`` (``src/etha/comm/transfer.py:20-41``).  Here every rank's shards live on one
+GPU, so "sending" a bucket means handing its buffer over in HBM: the producer packs into a slot
+of a persistent bucket pool, the consumer unpacks from the very same slot (zero copy).  Slots are
+assigned when a bucket list is first planned and reused by every later transfer, so the
+consumer's tile program can hold absolute addresses.
+
+Matching follows the point-to-point rule of the reference's transports: the k-th bucket a rank
+sends on a wire key ``(src_rank, dst_ranks, transport)`` is the k-th bucket its peers receive on
+that key.
+"""
+
+from __future__ import annotations
+
+from collections import defaultdict
+
+import torch
+
+from .device_plan import Slot
+from .ir import Bucket
+
+_SLOT_ALIGN = 256
+
+
+class BucketPool:
+    """Persistent device memory for bucket buffers, carved from < 2 GiB segments.
+
+    Segments stay below 2 GiB so that each one can be shared with another process through
+    ``hipIpcGetMemHandle`` (larger shared allocations are not reliable on this platform).
+    """
+
+    def __init__(self, device: torch.device, segment_bytes: int = 1 << 30):
+        self.device = device
+        self.segment_bytes = segment_bytes
+        self.segments: list[torch.Tensor] = []
+        self._cursor = 0  # offset inside the last segment
+
+    def alloc(self, nbytes: int) -> Slot:
+        need = max(nbytes, 1)
+        if need > self.segment_bytes or not self.segments or self._cursor + need > self.segments[-1].numel():
+            size = max(self.segment_bytes, need)
+            self.segments.append(torch.empty(size, dtype=torch.uint8, device=self.device))
+            self._cursor = 0
+        seg = self.segments[-1]
+        ptr = seg.data_ptr() + self._cursor
+        self._cursor = -(-(self._cursor + need) // _SLOT_ALIGN) * _SLOT_ALIGN
+        return Slot(ptr=ptr, nbytes=nbytes, lo=seg.data_ptr(), hi=seg.data_ptr() + seg.numel())
+
+    def view(self, slot: Slot) -> torch.Tensor:
+        """uint8 tensor aliasing a slot (for inspection and tests)."""
+        for seg in self.segments:
+            base = seg.data_ptr()
+            if base <= slot.ptr and slot.ptr + slot.nbytes <= base + seg.numel():
+                return seg[slot.ptr - base : slot.ptr - base + slot.nbytes]
+        raise ValueError("slot does not belong to this pool")
+
+    @property
+    def reserved_bytes(self) -> int:
+        return sum(s.numel() for s in self.segments)
+
+
+def wire_key(bucket: Bucket) -> tuple:
+    return (bucket.src_rank, tuple(bucket.dst_ranks), bucket.transport.value)
+
+
+class LoopbackWire:
+    """Process-wide stand-in for the process groups of the reference's executor."""
+
+    def __init__(self, device: torch.device | str | None = None, segment_bytes: int = 1 << 30):
+        self.device = torch.device(device) if device is not None else None
+        self.segment_bytes = segment_bytes
+        self.pool: BucketPool | None = None
+        self._sent: dict[tuple, list[tuple[Slot, tuple[int, ...]]]] = defaultdict(list)
+        self._plans: dict[tuple, object] = {}
+
+    def _pool_for(self, device: torch.device) -> BucketPool:
+        if self.pool is None:
+            self.device = self.device or device
+            self.pool = BucketPool(self.device, self.segment_bytes)
+        if device != self.pool.device:
+            raise RuntimeError(f"loopback wire is bound to {self.pool.device}, got a bucket on {device}")
+        return self.pool
+
+    # -- plan-time rendezvous -------------------------------------------------------------------
+    def slot_for_send(self, bucket: Bucket, index: int, device: torch.device) -> Slot:
+        """Slot of the ``index``-th bucket sent on this bucket's wire key (allocated on first use)."""
+        sent = self._sent[wire_key(bucket)]
+        sizes = tuple(c.nbytes for c in bucket.chunks)
+        if index < len(sent):
+            slot, known = sent[index]
+            if known != sizes:
+                raise RuntimeError(f"{bucket}: re-planned with a different chunk layout")
+            return slot
+        if index != len(sent):
+            raise RuntimeError(f"{bucket}: send buckets must be planned in order")
+        slot = self._pool_for(device).alloc(bucket.total_bytes)
+        sent.append((slot, sizes))
+        return slot
+
+    def slot_for_recv(self, bucket: Bucket, index: int) -> Slot:
+        sent = self._sent.get(wire_key(bucket), [])
+        if index >= len(sent):
+            raise RuntimeError(
+                f"{bucket}: no matching send bucket #{index} has been planned on this wire "
+                "(plan/run the source side first; a real wire would deadlock here)"
+            )
+        slot, sizes = sent[index]
+        if sizes != tuple(c.nbytes for c in bucket.chunks):
+            raise RuntimeError(f"{bucket}: chunk layout differs from the matching send bucket")
+        return slot
+
+    def private_slot(self, nbytes: int, device: torch.device) -> Slot:
+        return self._pool_for(device).alloc(nbytes)
+
+    # -- plan cache -----------------------------------------------------------------------------
+    def plan(self, buckets: list[Bucket]):
+        from .comm_methods import TransferPlan
+
+        key = tuple(id(b) for b in buckets)
+        plan = self._plans.get(key)
+        if plan is None:
+            plan = TransferPlan(self, list(buckets))
+            self._plans[key] = plan
+        return plan
+
+    def reset(self) -> None:
+        self._plans.clear()
+        self._sent.clear()
+        self.pool = None
+
+
+_default_wire: LoopbackWire | None = None
+
+
+def default_wire() -> LoopbackWire:
+    global _default_wire
+    if _default_wire is None:
+        _default_wire = LoopbackWire()
+    return _default_wire
+
+
+def reset_default_wire() -> None:
+    global _default_wire
+    if _default_wire is not None:
+        _default_wire.reset()
+    _default_wire = None

@@ -1,0 +1,931 @@
+// MI355X (gfx950) redistribute hot path: pack / unpack / self-copy / Partial reduce-pack.
+//
+// Design.  These are HBM-bound byte movers.  On MI355X a plain copy runs fastest when every
+// work-item moves exactly one 16-byte vector, workgroups are small (256 work-items = 4 KiB),
+// the grid is huge and ordered by address, and both sides use nontemporal accesses; loops and
+// several vectors per work-item lose 10-30 %.  So all chunk geometry (slices, strides, bucket
+// offsets, dtype pairs, alignment classes) is resolved once on the host into a flat
+// device-resident *tile program*: one entry per workgroup holding absolute addresses.  A
+// workgroup does one scalar table load, each work-item one vector load and one vector store.
+//
+// What it replaces in the reference: the per-chunk ATen launches of Chunk.prepare /
+// Bucket.prepare / Chunk.finalize / Bucket.finalize (src/etha/comm/ir.py:101-141, 229-264,
+// 300-310) - slice, contiguous(), all_reduce, to(dtype), narrow/view/copy_.
+#include <hip/hip_runtime.h>
+
+#include <cstdarg>
+#include <cstdio>
+#include <cstring>
+#include <map>
+#include <mutex>
+#include <new>
+#include <string>
+#include <vector>
+
+#include "etha_reshard.h"
+
+namespace {
+
+constexpr uint32_t kTileThreads = 256;  // work-items per tile = units per tile
+
+// ---- tile program entries (device-visible, also read back by host-side checkers) -------------
+// A "unit" is what one work-item moves: 2^ua bytes on the a side and 2^ub bytes on the b side
+// (equal for byte moves; different for converting moves).  a = tensor side, b = bucket side
+// (for self-copy tables a = source region, b = destination region).
+struct RunTile {  // one contiguous run on both sides
+  uint64_t a;     // address of the tile's first unit, a side
+  uint64_t b;     // address of the tile's first unit, b side
+  uint32_t n;     // active units (<= kTileThreads)
+  uint32_t meta;
+};
+static_assert(sizeof(RunTile) == 24, "RunTile layout");
+
+struct RowTile {     // walks rows of `run` units; covers units [c0, c0+n) counted from row r0
+  uint64_t a;        // address of (row r0, unit 0) on the a side; for reduce tiles: byte offset from each peer base
+  uint64_t b;        // address of (row r0, unit 0) on the b side
+  int64_t a_pitch;   // bytes between consecutive rows
+  int64_t b_pitch;
+  uint32_t n;        // active units (<= kTileThreads)
+  uint32_t meta;
+  uint32_t run;      // units per row
+  uint32_t c0;       // first unit's column inside row r0 (< run)
+  uint32_t peer_first;  // reduce tiles: index of the first peer base in the peers array
+  uint32_t n_peers;     // 0 = plain tile
+  uint32_t reduce_op;
+  uint32_t pad;
+};
+static_assert(sizeof(RowTile) == 64, "RowTile layout");
+
+// meta bits
+constexpr uint32_t kMetaUaShift = 0;    // 4 bits: log2 bytes per unit, a side
+constexpr uint32_t kMetaUbShift = 4;    // 4 bits: log2 bytes per unit, b side
+constexpr uint32_t kMetaDtaShift = 8;   // 4 bits: ETHA_* dtype, a side
+constexpr uint32_t kMetaDtbShift = 12;  // 4 bits: ETHA_* dtype, b side
+constexpr uint32_t kMetaCvt = 1u << 16; // converting move (else byte move)
+constexpr uint32_t kMetaVec = 1u << 17; // converting move handles the full vector (else 1 element)
+
+// ---- typed vector access ----------------------------------------------------------------------
+typedef uint32_t u32x2 __attribute__((ext_vector_type(2)));
+typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
+
+template <typename V>
+__device__ __forceinline__ V ld_stream(uint64_t addr) {
+  return __builtin_nontemporal_load(reinterpret_cast<const V*>(addr));
+}
+template <typename V>
+__device__ __forceinline__ void st_stream(uint64_t addr, V v) {
+  __builtin_nontemporal_store(v, reinterpret_cast<V*>(addr));
+}
+template <typename V>
+__device__ __forceinline__ void copy_as(uint64_t src, uint64_t dst) {
+  st_stream<V>(dst, ld_stream<V>(src));
+}
+
+// N elements of storage type T as one naturally aligned vector.
+template <typename T, int N>
+struct Pack {
+  typedef T vec __attribute__((ext_vector_type(N)));
+  vec v;
+  __device__ __forceinline__ void load(uint64_t addr) { v = ld_stream<vec>(addr); }
+  __device__ __forceinline__ void store(uint64_t addr) const { st_stream<vec>(addr, v); }
+  __device__ __forceinline__ T get(int i) const { return v[i]; }
+  __device__ __forceinline__ void set(int i, T x) { v[i] = x; }
+};
+template <typename T>
+struct Pack<T, 1> {
+  T v;
+  __device__ __forceinline__ void load(uint64_t addr) { v = ld_stream<T>(addr); }
+  __device__ __forceinline__ void store(uint64_t addr) const { st_stream<T>(addr, v); }
+  __device__ __forceinline__ T get(int) const { return v; }
+  __device__ __forceinline__ void set(int, T x) { v = x; }
+};
+
+// ---- element conversions (all go through fp32, as c10::Half/BFloat16 constructors do) ----------
+struct TagF16 { typedef uint16_t bits; };
+struct TagBF16 { typedef uint16_t bits; };
+struct TagF32 { typedef uint32_t bits; };
+struct TagF64 { typedef uint64_t bits; };
+
+__device__ __forceinline__ float to_f32(TagF16, uint16_t x) { return (float)__builtin_bit_cast(_Float16, x); }
+__device__ __forceinline__ float to_f32(TagBF16, uint16_t x) { return __builtin_bit_cast(float, (uint32_t)x << 16); }
+__device__ __forceinline__ float to_f32(TagF32, uint32_t x) { return __builtin_bit_cast(float, x); }
+__device__ __forceinline__ float to_f32(TagF64, uint64_t x) { return (float)__builtin_bit_cast(double, x); }
+
+__device__ __forceinline__ uint16_t from_f32(TagF16, float f) { return __builtin_bit_cast(uint16_t, (_Float16)f); }
+// round-to-nearest-even on the bit pattern; every NaN becomes the canonical quiet NaN 0x7FC0
+__device__ __forceinline__ uint16_t from_f32(TagBF16, float f) {
+  uint32_t u = __builtin_bit_cast(uint32_t, f);
+  if ((u & 0x7fffffffu) > 0x7f800000u) return 0x7fc0;
+  u += 0x7fffu + ((u >> 16) & 1u);
+  return (uint16_t)(u >> 16);
+}
+__device__ __forceinline__ uint32_t from_f32(TagF32, float f) { return __builtin_bit_cast(uint32_t, f); }
+__device__ __forceinline__ uint64_t from_f32(TagF64, float f) { return __builtin_bit_cast(uint64_t, (double)f); }
+
+template <typename S, typename D, int N>
+__device__ __forceinline__ void cvt_n(uint64_t src, uint64_t dst) {
+  Pack<typename S::bits, N> in;
+  Pack<typename D::bits, N> out;
+  in.load(src);
+#pragma unroll
+  for (int i = 0; i < N; i++) out.set(i, from_f32(D(), to_f32(S(), in.get(i))));
+  out.store(dst);
+}
+
+template <typename S, typename D>
+__device__ __forceinline__ void cvt_pair(bool vec, uint64_t src, uint64_t dst) {
+  constexpr int kMaxBytes = sizeof(typename S::bits) > sizeof(typename D::bits) ? sizeof(typename S::bits)
+                                                                                  : sizeof(typename D::bits);
+  constexpr int kN = 16 / kMaxBytes;
+  if (vec)
+    cvt_n<S, D, kN>(src, dst);
+  else
+    cvt_n<S, D, 1>(src, dst);
+}
+
+template <typename S>
+__device__ __forceinline__ void cvt_from(uint32_t dd, bool vec, uint64_t src, uint64_t dst) {
+  switch (dd) {
+    case ETHA_F16: cvt_pair<S, TagF16>(vec, src, dst); break;
+    case ETHA_BF16: cvt_pair<S, TagBF16>(vec, src, dst); break;
+    case ETHA_F32: cvt_pair<S, TagF32>(vec, src, dst); break;
+    default: cvt_pair<S, TagF64>(vec, src, dst); break;
+  }
+}
+
+template <bool REV>
+__device__ __forceinline__ void move_unit(uint32_t meta, uint64_t a, uint64_t b) {
+  const uint64_t src = REV ? b : a, dst = REV ? a : b;
+  if (!(meta & kMetaCvt)) {
+    switch (meta & 15u) {
+      case 4: copy_as<u32x4>(src, dst); break;
+      case 3: copy_as<u32x2>(src, dst); break;
+      case 2: copy_as<uint32_t>(src, dst); break;
+      case 1: copy_as<uint16_t>(src, dst); break;
+      default: copy_as<uint8_t>(src, dst); break;
+    }
+    return;
+  }
+  const uint32_t dta = (meta >> kMetaDtaShift) & 15u, dtb = (meta >> kMetaDtbShift) & 15u;
+  const uint32_t sd = REV ? dtb : dta, dd = REV ? dta : dtb;
+  const bool vec = (meta & kMetaVec) != 0;
+  switch (sd) {
+    case ETHA_F16: cvt_from<TagF16>(dd, vec, src, dst); break;
+    case ETHA_BF16: cvt_from<TagBF16>(dd, vec, src, dst); break;
+    case ETHA_F32: cvt_from<TagF32>(dd, vec, src, dst); break;
+    default: cvt_from<TagF64>(dd, vec, src, dst); break;
+  }
+}
+
+__device__ __forceinline__ void row_position(const RowTile& t, uint32_t tid, uint32_t& r, uint32_t& c) {
+  const uint32_t q = t.c0 + tid;  // c0 < run and tid < 256, so q < 2*run whenever run >= 256
+  if (t.run >= kTileThreads) {
+    r = q >= t.run ? 1u : 0u;
+    c = q - (r ? t.run : 0u);
+  } else {
+    r = q / t.run;
+    c = q - r * t.run;
+  }
+}
+
+// pack (REV = false): a -> b.   unpack (REV = true): b -> a.
+template <bool REV>
+__global__ __launch_bounds__(256) void etha_tile_kernel(const RunTile* __restrict__ run_tiles, uint32_t n_run,
+                                                         const RowTile* __restrict__ row_tiles) {
+  const uint32_t bid = blockIdx.x, tid = threadIdx.x;
+  uint64_t a, b;
+  uint32_t n, meta;
+  if (bid < n_run) {
+    const RunTile t = run_tiles[bid];
+    n = t.n;
+    meta = t.meta;
+    a = t.a + ((uint64_t)tid << ((meta >> kMetaUaShift) & 15u));
+    b = t.b + ((uint64_t)tid << ((meta >> kMetaUbShift) & 15u));
+  } else {
+    const RowTile t = row_tiles[bid - n_run];
+    n = t.n;
+    meta = t.meta;
+    uint32_t r, c;
+    row_position(t, tid, r, c);
+    a = t.a + (uint64_t)((int64_t)r * t.a_pitch) + ((uint64_t)c << ((meta >> kMetaUaShift) & 15u));
+    b = t.b + (uint64_t)((int64_t)r * t.b_pitch) + ((uint64_t)c << ((meta >> kMetaUbShift) & 15u));
+  }
+  if (tid >= n) return;
+  move_unit<REV>(meta, a, b);
+}
+
+// ---- Partial reduce-pack ------------------------------------------------------------------------
+template <typename ACC>
+__device__ __forceinline__ ACC combine(uint32_t op, ACC x, ACC y) {
+  switch (op) {
+    case ETHA_MAX: return x > y ? x : (y > x ? y : (x == x ? x : y));
+    case ETHA_MIN: return x < y ? x : (y < x ? y : (x == x ? x : y));
+    case ETHA_PRODUCT: return x * y;
+    default: return x + y;  // SUM, AVG
+  }
+}
+
+template <typename S, int N>
+struct LoadF32 {
+  __device__ static __forceinline__ void run(uint64_t addr, float* out) {
+    Pack<typename S::bits, N> in;
+    in.load(addr);
+#pragma unroll
+    for (int i = 0; i < N; i++) out[i] = to_f32(S(), in.get(i));
+  }
+};
+
+// f16/bf16/f32 partials: fp32 accumulation, peers combined strictly in list (= rank) order.
+template <typename S, typename D, int N>
+__device__ __forceinline__ void reduce_f32(const uint64_t* __restrict__ peers, uint32_t np, uint32_t op, uint64_t a_off,
+                                           uint64_t dst) {
+  float acc[N];
+  LoadF32<S, N>::run(peers[0] + a_off, acc);
+  uint32_t p = 1;
+  for (; p + 3 <= np; p += 3) {  // three peers' loads in flight, then combine in order
+    float v0[N], v1[N], v2[N];
+    LoadF32<S, N>::run(peers[p] + a_off, v0);
+    LoadF32<S, N>::run(peers[p + 1] + a_off, v1);
+    LoadF32<S, N>::run(peers[p + 2] + a_off, v2);
+#pragma unroll
+    for (int i = 0; i < N; i++) acc[i] = combine(op, combine(op, combine(op, acc[i], v0[i]), v1[i]), v2[i]);
+  }
+  for (; p < np; p++) {
+    float v[N];
+    LoadF32<S, N>::run(peers[p] + a_off, v);
+#pragma unroll
+    for (int i = 0; i < N; i++) acc[i] = combine(op, acc[i], v[i]);
+  }
+  Pack<typename D::bits, N> out;
+  const float cnt = (float)np;
+#pragma unroll
+  for (int i = 0; i < N; i++) {
+    float r = acc[i];
+    if (op == ETHA_AVG) r = r / cnt;
+    out.set(i, from_f32(D(), r));
+  }
+  out.store(dst);
+}
+
+// f64 partials: f64 accumulation; result converted like a plain f64 -> D move.
+template <typename D, int N>
+__device__ __forceinline__ void reduce_f64(const uint64_t* __restrict__ peers, uint32_t np, uint32_t op, uint64_t a_off,
+                                           uint64_t dst) {
+  double acc[N];
+  {
+    Pack<uint64_t, N> in;
+    in.load(peers[0] + a_off);
+#pragma unroll
+    for (int i = 0; i < N; i++) acc[i] = __builtin_bit_cast(double, in.get(i));
+  }
+  for (uint32_t p = 1; p < np; p++) {
+    Pack<uint64_t, N> in;
+    in.load(peers[p] + a_off);
+#pragma unroll
+    for (int i = 0; i < N; i++) acc[i] = combine(op, acc[i], __builtin_bit_cast(double, in.get(i)));
+  }
+  Pack<typename D::bits, N> out;
+#pragma unroll
+  for (int i = 0; i < N; i++) {
+    double r = acc[i];
+    if (op == ETHA_AVG) r = r / (double)np;
+    if (sizeof(typename D::bits) == 8)
+      out.set(i, (typename D::bits)__builtin_bit_cast(uint64_t, r));
+    else
+      out.set(i, from_f32(D(), (float)r));
+  }
+  out.store(dst);
+}
+
+template <typename S, typename D>
+__device__ __forceinline__ void reduce_pair(bool vec, const uint64_t* peers, uint32_t np, uint32_t op, uint64_t a_off,
+                                            uint64_t dst) {
+  constexpr int kMaxBytes = sizeof(typename S::bits) > sizeof(typename D::bits) ? sizeof(typename S::bits)
+                                                                                  : sizeof(typename D::bits);
+  constexpr int kN = 16 / kMaxBytes;
+  if (sizeof(typename S::bits) == 8) {
+    if (vec)
+      reduce_f64<D, kN>(peers, np, op, a_off, dst);
+    else
+      reduce_f64<D, 1>(peers, np, op, a_off, dst);
+  } else {
+    if (vec)
+      reduce_f32<S, D, kN>(peers, np, op, a_off, dst);
+    else
+      reduce_f32<S, D, 1>(peers, np, op, a_off, dst);
+  }
+}
+
+template <typename S>
+__device__ __forceinline__ void reduce_from(uint32_t dd, bool vec, const uint64_t* peers, uint32_t np, uint32_t op,
+                                            uint64_t a_off, uint64_t dst) {
+  switch (dd) {
+    case ETHA_F16: reduce_pair<S, TagF16>(vec, peers, np, op, a_off, dst); break;
+    case ETHA_BF16: reduce_pair<S, TagBF16>(vec, peers, np, op, a_off, dst); break;
+    case ETHA_F32: reduce_pair<S, TagF32>(vec, peers, np, op, a_off, dst); break;
+    default: reduce_pair<S, TagF64>(vec, peers, np, op, a_off, dst); break;
+  }
+}
+
+__global__ __launch_bounds__(256) void etha_reduce_kernel(const RowTile* __restrict__ row_tiles,
+                                                           const uint64_t* __restrict__ peer_bases) {
+  const uint32_t tid = threadIdx.x;
+  const RowTile t = row_tiles[blockIdx.x];
+  if (tid >= t.n) return;
+  uint32_t r, c;
+  row_position(t, tid, r, c);
+  const uint32_t meta = t.meta;
+  const uint64_t a_off = t.a + (uint64_t)((int64_t)r * t.a_pitch) + ((uint64_t)c << ((meta >> kMetaUaShift) & 15u));
+  const uint64_t dst = t.b + (uint64_t)((int64_t)r * t.b_pitch) + ((uint64_t)c << ((meta >> kMetaUbShift) & 15u));
+  const uint64_t* peers = peer_bases + t.peer_first;
+  const bool vec = (meta & kMetaVec) != 0;
+  const uint32_t dd = (meta >> kMetaDtbShift) & 15u;
+  switch ((meta >> kMetaDtaShift) & 15u) {
+    case ETHA_F16: reduce_from<TagF16>(dd, vec, peers, t.n_peers, t.reduce_op, a_off, dst); break;
+    case ETHA_BF16: reduce_from<TagBF16>(dd, vec, peers, t.n_peers, t.reduce_op, a_off, dst); break;
+    case ETHA_F32: reduce_from<TagF32>(dd, vec, peers, t.n_peers, t.reduce_op, a_off, dst); break;
+    default: reduce_from<TagF64>(dd, vec, peers, t.n_peers, t.reduce_op, a_off, dst); break;
+  }
+}
+
+// =================================================================================================
+// Host side: validation and the tile compiler.
+// =================================================================================================
+thread_local std::string g_err;
+std::mutex g_ipc_mutex;
+std::map<void*, void*> g_ipc_bases;  // pointer handed out by etha_ipc_open -> mapping base
+
+int fail(int code, const char* fmt, ...) {
+  char buf[512];
+  va_list ap;
+  va_start(ap, fmt);
+  vsnprintf(buf, sizeof(buf), fmt, ap);
+  va_end(ap);
+  g_err = buf;
+  return code;
+}
+
+#define HIP_TRY(expr)                                                                      \
+  do {                                                                                     \
+    hipError_t e_ = (expr);                                                                \
+    if (e_ != hipSuccess) return fail(ETHA_ERR_HIP, "%s: %s", #expr, hipGetErrorString(e_)); \
+  } while (0)
+
+int dtype_size(uint32_t dt) {
+  switch (dt) {
+    case ETHA_F16: case ETHA_BF16: case ETHA_B16: return 2;
+    case ETHA_F32: case ETHA_B32: return 4;
+    case ETHA_F64: case ETHA_B64: return 8;
+    case ETHA_B8: return 1;
+    default: return 0;
+  }
+}
+bool is_float(uint32_t dt) { return dt <= ETHA_F64; }
+int log2u(uint64_t x) {
+  int l = 0;
+  while ((1ull << (l + 1)) <= x) l++;
+  return l;
+}
+
+struct Region {  // strided region; strides in bytes
+  uint64_t base = 0;
+  int nd = 0;
+  int64_t shape[ETHA_MAX_NDIM];
+  int64_t stride[ETHA_MAX_NDIM];
+};
+
+// region of the tensor side of a descriptor + byte range check
+int tensor_region(const EthaChunkDesc& d, uint32_t idx, uint64_t base_ptr, bool relative, Region* out) {
+  const int es = dtype_size(d.tensor_dtype);
+  if (es == 0) return fail(ETHA_ERR_INVALID, "chunk %u: unknown tensor_dtype %u", idx, d.tensor_dtype);
+  if (d.ndim > ETHA_MAX_NDIM) return fail(ETHA_ERR_INVALID, "chunk %u: ndim %u > %d", idx, d.ndim, ETHA_MAX_NDIM);
+  if (base_ptr == 0 && !relative) return fail(ETHA_ERR_INVALID, "chunk %u: null tensor pointer", idx);
+  Region r;
+  r.nd = (int)d.ndim;
+  __int128 off = 0, lo = 0, hi = 0;
+  bool empty = false;
+  for (int i = 0; i < r.nd; i++) {
+    if (d.shape[i] < 0 || d.start[i] < 0)
+      return fail(ETHA_ERR_INVALID, "chunk %u: negative shape/start in dim %d", idx, i);
+    r.shape[i] = d.shape[i];
+    r.stride[i] = d.stride[i] * es;
+    off += (__int128)d.start[i] * d.stride[i] * es;
+    if (d.shape[i] == 0) empty = true;
+    const __int128 ext = (__int128)(d.shape[i] - 1) * d.stride[i] * es;
+    if (d.shape[i] > 0) (ext < 0 ? lo : hi) += ext;
+  }
+  const __int128 first = (__int128)base_ptr + off;
+  if (first < 0 || first > (__int128)UINT64_MAX) return fail(ETHA_ERR_INVALID, "chunk %u: address overflow", idx);
+  r.base = (uint64_t)first;
+  if (!empty && (d.tensor_lo || d.tensor_hi)) {
+    if (first + lo < (__int128)d.tensor_lo || first + hi + es > (__int128)d.tensor_hi)
+      return fail(ETHA_ERR_INVALID, "chunk %u: tensor region [%llx,%llx) leaves the allowed range [%llx,%llx)", idx,
+                  (unsigned long long)(first + lo), (unsigned long long)(first + hi + es),
+                  (unsigned long long)d.tensor_lo, (unsigned long long)d.tensor_hi);
+  }
+  *out = r;
+  return ETHA_OK;
+}
+
+uint64_t region_numel(const Region& r) {
+  uint64_t n = 1;
+  for (int i = 0; i < r.nd; i++) n *= (uint64_t)r.shape[i];
+  return n;
+}
+
+struct Builder {
+  std::vector<RunTile> run;
+  std::vector<RowTile> row;
+  std::vector<uint32_t> run_begin, row_begin;
+  std::vector<uint8_t> is_reduce;
+  uint64_t payload_bytes = 0;
+};
+
+constexpr uint64_t kMaxTiles = 0x7fff0000ull;  // grid.x limit with margin
+
+struct ReduceSpec {
+  uint32_t n_peers = 0, peer_first = 0, op = 0;
+};
+
+// Emit tiles moving region A (dtype dta) to/from region B (dtype dtb); both have the same shape.
+// For reduce chunks A.base is 0 and tile addresses on the a side are offsets from the peer bases;
+// `align_bases` then lists the peers' real bases for the alignment decision.
+int compile_pair(Builder& bld, uint32_t idx, const Region& A0, const Region& B0, uint32_t dta, uint32_t dtb,
+                 const ReduceSpec& red, const std::vector<uint64_t>& align_bases) {
+  const int esa = dtype_size(dta), esb = dtype_size(dtb);
+  if (A0.nd != B0.nd) return fail(ETHA_ERR_INVALID, "chunk %u: rank mismatch", idx);
+  for (int i = 0; i < A0.nd; i++)
+    if (A0.shape[i] != B0.shape[i]) return fail(ETHA_ERR_INVALID, "chunk %u: shape mismatch in dim %d", idx, i);
+  const bool cvt = dta != dtb;
+  if (cvt && !(is_float(dta) && is_float(dtb)))
+    return fail(ETHA_ERR_UNSUPPORTED, "chunk %u: conversion %u -> %u is only implemented between floating types", idx,
+                dta, dtb);
+  if (red.n_peers && !is_float(dta))
+    return fail(ETHA_ERR_UNSUPPORTED, "chunk %u: Partial reduce needs a floating tensor dtype", idx);
+  if (region_numel(A0) == 0) return ETHA_OK;
+
+  // 1. drop size-1 dims, 2. merge dims that are contiguous on both sides
+  int64_t n[ETHA_MAX_NDIM], sa[ETHA_MAX_NDIM], sb[ETHA_MAX_NDIM];
+  int k = 0;
+  for (int i = 0; i < A0.nd; i++) {
+    if (A0.shape[i] == 1) continue;
+    if (k > 0 && sa[k - 1] == A0.shape[i] * A0.stride[i] && sb[k - 1] == A0.shape[i] * B0.stride[i]) {
+      n[k - 1] *= A0.shape[i];
+      sa[k - 1] = A0.stride[i];
+      sb[k - 1] = B0.stride[i];
+    } else {
+      n[k] = A0.shape[i];
+      sa[k] = A0.stride[i];
+      sb[k] = B0.stride[i];
+      k++;
+    }
+  }
+  // 3. innermost contiguous run (in elements)
+  uint64_t run_elems = 1;
+  if (k > 0 && sa[k - 1] == esa && sb[k - 1] == esb) {
+    run_elems = (uint64_t)n[k - 1];
+    k--;
+  }
+  // 4. unit size: the widest vector every row start and the run length allow
+  int ua_log2, ub_log2;
+  uint64_t run_units;
+  uint32_t meta = 0;
+  {
+    uint64_t mask_a = red.n_peers ? 0 : A0.base, mask_b = B0.base;
+    for (uint64_t p : align_bases) mask_a |= p + A0.base;  // reduce: A0.base is an offset from each peer base
+    for (int i = 0; i < k; i++) {
+      mask_a |= (uint64_t)(sa[i] < 0 ? -sa[i] : sa[i]);
+      mask_b |= (uint64_t)(sb[i] < 0 ? -sb[i] : sb[i]);
+    }
+    if (!cvt && !red.n_peers) {
+      const uint64_t run_bytes = run_elems * (uint64_t)esa;
+      uint64_t m = mask_a | mask_b | run_bytes;
+      int v = 4;
+      while (v > 0 && (m & ((1ull << v) - 1))) v--;
+      ua_log2 = ub_log2 = v;
+      run_units = run_bytes >> v;
+    } else {
+      const int big = esa > esb ? esa : esb;
+      int epv = 16 / big;
+      const bool vec_ok = (run_elems % (uint64_t)epv == 0) && (mask_a % (uint64_t)(epv * esa) == 0) &&
+                          (mask_b % (uint64_t)(epv * esb) == 0);
+      if (!vec_ok) {
+        epv = 1;
+        if (mask_a % (uint64_t)esa || mask_b % (uint64_t)esb)
+          return fail(ETHA_ERR_INVALID, "chunk %u: element address not aligned to its dtype", idx);
+      }
+      ua_log2 = log2u((uint64_t)(epv * esa));
+      ub_log2 = log2u((uint64_t)(epv * esb));
+      run_units = run_elems / (uint64_t)epv;
+      meta |= kMetaCvt;
+      if (epv > 1) meta |= kMetaVec;
+    }
+  }
+  meta |= ((uint32_t)ua_log2 << kMetaUaShift) | ((uint32_t)ub_log2 << kMetaUbShift) | (dta << kMetaDtaShift) |
+          (dtb << kMetaDtbShift);
+  const uint64_t ua = 1ull << ua_log2, ub = 1ull << ub_log2;
+
+  // 5. tiles.  Long or 256-multiple rows (and single runs) become run tiles; other shapes become
+  //    row tiles over the innermost remaining dim; dims further out are unrolled here.
+  const bool use_rows = red.n_peers != 0 || (k > 0 && run_units % kTileThreads != 0 && run_units < 4096);
+  if (run_units > 0xffffffffull && use_rows && k > 0)
+    return fail(ETHA_ERR_UNSUPPORTED, "chunk %u: row longer than 2^32 units", idx);
+  const int outer = use_rows && k > 0 ? k - 1 : k;  // dims unrolled on the host
+  int64_t pos[ETHA_MAX_NDIM] = {0};
+  uint64_t off_a = 0, off_b = 0;  // wraps mod 2^64 for negative strides, which is fine
+  while (true) {
+    const uint64_t a0 = A0.base + off_a, b0 = B0.base + off_b;
+    if (!use_rows) {
+      for (uint64_t q = 0; q < run_units; q += kTileThreads) {
+        RunTile t;
+        t.a = a0 + q * ua;
+        t.b = b0 + q * ub;
+        t.n = (uint32_t)(run_units - q < kTileThreads ? run_units - q : kTileThreads);
+        t.meta = meta;
+        bld.run.push_back(t);
+      }
+    } else {
+      const uint64_t rows = k > 0 ? (uint64_t)n[k - 1] : 1;
+      const int64_t pa = k > 0 ? sa[k - 1] : 0, pb = k > 0 ? sb[k - 1] : 0;
+      const uint64_t total = rows * run_units;
+      for (uint64_t q = 0; q < total; q += kTileThreads) {
+        RowTile t;
+        memset(&t, 0, sizeof(t));
+        const uint64_t left = total - q;
+        t.n = (uint32_t)(left < kTileThreads ? left : kTileThreads);
+        t.meta = meta;
+        if (rows == 1) {  // one (possibly very long) run: address the tile directly
+          t.a = a0 + q * ua;
+          t.b = b0 + q * ub;
+          t.run = kTileThreads;
+          t.c0 = 0;
+        } else {
+          const uint64_t r0 = q / run_units, c0 = q % run_units;
+          t.a = a0 + (uint64_t)((int64_t)r0 * pa);
+          t.b = b0 + (uint64_t)((int64_t)r0 * pb);
+          t.a_pitch = pa;
+          t.b_pitch = pb;
+          t.run = (uint32_t)run_units;
+          t.c0 = (uint32_t)c0;
+        }
+        t.peer_first = red.peer_first;
+        t.n_peers = red.n_peers;
+        t.reduce_op = red.op;
+        bld.row.push_back(t);
+      }
+    }
+    if (bld.run.size() + bld.row.size() > kMaxTiles)
+      return fail(ETHA_ERR_UNSUPPORTED, "tile program too large (> %llu tiles)", (unsigned long long)kMaxTiles);
+    int d = outer - 1;
+    for (; d >= 0; d--) {
+      pos[d]++;
+      off_a += (uint64_t)sa[d];
+      off_b += (uint64_t)sb[d];
+      if (pos[d] < n[d]) break;
+      off_a -= (uint64_t)(sa[d] * n[d]);
+      off_b -= (uint64_t)(sb[d] * n[d]);
+      pos[d] = 0;
+    }
+    if (d < 0) break;
+  }
+  return ETHA_OK;
+}
+
+}  // namespace
+
+struct EthaTable {
+  int kind = 0;  // 0 = pack/unpack table, 1 = self-copy table
+  std::vector<RunTile> h_run;
+  std::vector<RowTile> h_row;
+  std::vector<uint32_t> run_begin, row_begin;
+  std::vector<uint32_t> reduce_prefix;  // number of reduce chunks before chunk i
+  std::vector<uint64_t> h_peers;
+  RunTile* d_run = nullptr;
+  RowTile* d_row = nullptr;
+  uint64_t* d_peers = nullptr;
+  uint32_t n_chunks = 0;
+  uint64_t payload_bytes = 0;
+  uint64_t device_bytes = 0;
+  bool uploaded = false;
+};
+
+namespace {
+
+int upload_table(EthaTable* t) {
+  if (!t->h_run.empty()) {
+    const size_t bytes = t->h_run.size() * sizeof(RunTile);
+    HIP_TRY(hipMalloc(&t->d_run, bytes));
+    HIP_TRY(hipMemcpy(t->d_run, t->h_run.data(), bytes, hipMemcpyHostToDevice));
+    t->device_bytes += bytes;
+  }
+  if (!t->h_row.empty()) {
+    const size_t bytes = t->h_row.size() * sizeof(RowTile);
+    HIP_TRY(hipMalloc(&t->d_row, bytes));
+    HIP_TRY(hipMemcpy(t->d_row, t->h_row.data(), bytes, hipMemcpyHostToDevice));
+    t->device_bytes += bytes;
+  }
+  if (!t->h_peers.empty()) {
+    const size_t bytes = t->h_peers.size() * sizeof(uint64_t);
+    HIP_TRY(hipMalloc(&t->d_peers, bytes));
+    HIP_TRY(hipMemcpy(t->d_peers, t->h_peers.data(), bytes, hipMemcpyHostToDevice));
+    t->device_bytes += bytes;
+  }
+  t->uploaded = true;
+  return ETHA_OK;
+}
+
+void free_table(EthaTable* t) {
+  if (!t) return;
+  if (t->d_run) (void)hipFree(t->d_run);
+  if (t->d_row) (void)hipFree(t->d_row);
+  if (t->d_peers) (void)hipFree(t->d_peers);
+  delete t;
+}
+
+int finish_table(Builder& bld, EthaTable* t, int upload, EthaTable** out) {
+  t->h_run.swap(bld.run);
+  t->h_row.swap(bld.row);
+  t->run_begin.swap(bld.run_begin);
+  t->row_begin.swap(bld.row_begin);
+  t->reduce_prefix.assign(t->n_chunks + 1, 0);
+  for (uint32_t i = 0; i < t->n_chunks; i++) t->reduce_prefix[i + 1] = t->reduce_prefix[i] + bld.is_reduce[i];
+  t->payload_bytes = bld.payload_bytes;
+  if (upload) {
+    const int rc = upload_table(t);
+    if (rc != ETHA_OK) {
+      free_table(t);
+      return rc;
+    }
+  }
+  *out = t;
+  return ETHA_OK;
+}
+
+int check_range(const EthaTable* t, uint32_t first, uint32_t count, int kind) {
+  if (!t) return fail(ETHA_ERR_INVALID, "null table");
+  if (t->kind != kind) return fail(ETHA_ERR_INVALID, "wrong table kind for this entry point");
+  if ((uint64_t)first + count > t->n_chunks)
+    return fail(ETHA_ERR_INVALID, "chunk range [%u,%u) exceeds table of %u chunks", first, first + count, t->n_chunks);
+  if (!t->uploaded) return fail(ETHA_ERR_INVALID, "table was created without upload; it cannot be launched");
+  return ETHA_OK;
+}
+
+template <bool REV>
+int launch_tiles(const EthaTable* t, uint32_t first, uint32_t count, void* stream) {
+  const uint32_t r0 = t->run_begin[first], r1 = t->run_begin[first + count];
+  const uint32_t w0 = t->row_begin[first], w1 = t->row_begin[first + count];
+  const uint32_t n_run = r1 - r0, n_row = w1 - w0;
+  if (n_run + n_row == 0) return ETHA_OK;
+  hipLaunchKernelGGL(etha_tile_kernel<REV>, dim3(n_run + n_row), dim3(kTileThreads), 0, (hipStream_t)stream,
+                     t->d_run + r0, n_run, t->d_row + w0);
+  HIP_TRY(hipGetLastError());
+  return ETHA_OK;
+}
+
+}  // namespace
+
+extern "C" {
+
+int etha_abi_version(void) { return ETHA_ABI_VERSION; }
+const char* etha_last_error(void) { return g_err.c_str(); }
+
+int etha_table_create(const EthaChunkDesc* descs, uint32_t n_chunks, const uint64_t* partial_ptrs,
+                      uint32_t n_partial_ptrs, int upload, EthaTable** out) {
+  if (!out) return fail(ETHA_ERR_INVALID, "null out");
+  *out = nullptr;
+  if (n_chunks && !descs) return fail(ETHA_ERR_INVALID, "null descriptor array");
+  Builder bld;
+  bld.run_begin.reserve(n_chunks + 1);
+  bld.row_begin.reserve(n_chunks + 1);
+  bld.is_reduce.assign(n_chunks, 0);
+  for (uint32_t i = 0; i < n_chunks; i++) {
+    const EthaChunkDesc& d = descs[i];
+    bld.run_begin.push_back((uint32_t)bld.run.size());
+    bld.row_begin.push_back((uint32_t)bld.row.size());
+    const int esw = dtype_size(d.wire_dtype);
+    if (esw == 0) return fail(ETHA_ERR_INVALID, "chunk %u: unknown wire_dtype %u", i, d.wire_dtype);
+    ReduceSpec red;
+    std::vector<uint64_t> peer_bases;
+    Region A;
+    if (d.n_partials) {
+      if (d.reduce_op > ETHA_PRODUCT) return fail(ETHA_ERR_INVALID, "chunk %u: unknown reduce_op %u", i, d.reduce_op);
+      if (!partial_ptrs || (uint64_t)d.partial_first + d.n_partials > n_partial_ptrs)
+        return fail(ETHA_ERR_INVALID, "chunk %u: partial pointer range outside partial_ptrs", i);
+      // every peer shares the chunk geometry; validate each peer's range with its own base
+      for (uint32_t p = 0; p < d.n_partials; p++) {
+        Region tmp;
+        EthaChunkDesc dp = d;
+        dp.tensor_lo = dp.tensor_hi = 0;  // the single lo/hi pair cannot describe several peers
+        const int rc = tensor_region(dp, i, partial_ptrs[d.partial_first + p], false, &tmp);
+        if (rc != ETHA_OK) return rc;
+        peer_bases.push_back(partial_ptrs[d.partial_first + p]);
+      }
+      EthaChunkDesc dz = d;
+      dz.tensor_lo = dz.tensor_hi = 0;
+      const int rc = tensor_region(dz, i, 0, true, &A);  // offsets relative to a peer base
+      if (rc != ETHA_OK) return rc;
+      red.n_peers = d.n_partials;
+      red.peer_first = d.partial_first;
+      red.op = d.reduce_op;
+      bld.is_reduce[i] = 1;
+    } else {
+      const int rc = tensor_region(d, i, d.tensor_ptr, false, &A);
+      if (rc != ETHA_OK) return rc;
+    }
+    // bucket side: contiguous, row-major, wire dtype
+    Region B;
+    B.nd = A.nd;
+    B.base = d.bucket_ptr;
+    int64_t acc = esw;
+    for (int j = A.nd - 1; j >= 0; j--) {
+      B.shape[j] = A.shape[j];
+      B.stride[j] = acc;
+      acc *= A.shape[j];
+    }
+    const uint64_t nbytes = region_numel(A) * (uint64_t)esw;
+    if (nbytes) {
+      if (d.bucket_ptr == 0) return fail(ETHA_ERR_INVALID, "chunk %u: null bucket pointer", i);
+      if ((d.bucket_lo || d.bucket_hi) &&
+          (d.bucket_ptr < d.bucket_lo || d.bucket_ptr + nbytes > d.bucket_hi || d.bucket_ptr + nbytes < d.bucket_ptr))
+        return fail(ETHA_ERR_INVALID, "chunk %u: bucket bytes [%llx,%llx) leave the bucket buffer [%llx,%llx)", i,
+                    (unsigned long long)d.bucket_ptr, (unsigned long long)(d.bucket_ptr + nbytes),
+                    (unsigned long long)d.bucket_lo, (unsigned long long)d.bucket_hi);
+    }
+    bld.payload_bytes += nbytes;
+    const int rc = compile_pair(bld, i, A, B, d.tensor_dtype, d.wire_dtype, red, peer_bases);
+    if (rc != ETHA_OK) return rc;
+  }
+  bld.run_begin.push_back((uint32_t)bld.run.size());
+  bld.row_begin.push_back((uint32_t)bld.row.size());
+  EthaTable* t = new (std::nothrow) EthaTable();
+  if (!t) return fail(ETHA_ERR_NOMEM, "out of host memory");
+  t->kind = 0;
+  t->n_chunks = n_chunks;
+  if (partial_ptrs && n_partial_ptrs) t->h_peers.assign(partial_ptrs, partial_ptrs + n_partial_ptrs);
+  return finish_table(bld, t, upload, out);
+}
+
+int etha_selfcopy_table_create(const EthaChunkDesc* src, const EthaChunkDesc* dst, uint32_t n_chunks, int upload,
+                               EthaTable** out) {
+  if (!out) return fail(ETHA_ERR_INVALID, "null out");
+  *out = nullptr;
+  if (n_chunks && (!src || !dst)) return fail(ETHA_ERR_INVALID, "null descriptor array");
+  Builder bld;
+  bld.is_reduce.assign(n_chunks, 0);
+  for (uint32_t i = 0; i < n_chunks; i++) {
+    bld.run_begin.push_back((uint32_t)bld.run.size());
+    bld.row_begin.push_back((uint32_t)bld.row.size());
+    if (src[i].n_partials || dst[i].n_partials)
+      return fail(ETHA_ERR_UNSUPPORTED, "chunk %u: self-copy of a Partial source is not implemented", i);
+    Region A, B;
+    int rc = tensor_region(src[i], i, src[i].tensor_ptr, false, &A);
+    if (rc != ETHA_OK) return rc;
+    rc = tensor_region(dst[i], i, dst[i].tensor_ptr, false, &B);
+    if (rc != ETHA_OK) return rc;
+    bld.payload_bytes += region_numel(A) * (uint64_t)dtype_size(dst[i].tensor_dtype);
+    rc = compile_pair(bld, i, A, B, src[i].tensor_dtype, dst[i].tensor_dtype, ReduceSpec(), {});
+    if (rc != ETHA_OK) return rc;
+  }
+  bld.run_begin.push_back((uint32_t)bld.run.size());
+  bld.row_begin.push_back((uint32_t)bld.row.size());
+  EthaTable* t = new (std::nothrow) EthaTable();
+  if (!t) return fail(ETHA_ERR_NOMEM, "out of host memory");
+  t->kind = 1;
+  t->n_chunks = n_chunks;
+  return finish_table(bld, t, upload, out);
+}
+
+int etha_table_destroy(EthaTable* table) {
+  free_table(table);
+  return ETHA_OK;
+}
+
+int etha_table_info(const EthaTable* t, EthaTableInfo* out) {
+  if (!t || !out) return fail(ETHA_ERR_INVALID, "null argument");
+  out->n_chunks = t->n_chunks;
+  out->n_run_tiles = (uint32_t)t->h_run.size();
+  out->n_row_tiles = (uint32_t)t->h_row.size();
+  out->tile_threads = kTileThreads;
+  out->device_bytes = t->device_bytes;
+  out->payload_bytes = t->payload_bytes;
+  return ETHA_OK;
+}
+
+int etha_table_read_tiles(const EthaTable* t, int which, void* out, uint64_t cap_bytes, uint64_t* need_bytes) {
+  if (!t || !need_bytes) return fail(ETHA_ERR_INVALID, "null argument");
+  const void* src;
+  uint64_t bytes;
+  if (which == 0) {
+    src = t->h_run.data();
+    bytes = t->h_run.size() * sizeof(RunTile);
+  } else if (which == 1) {
+    src = t->h_row.data();
+    bytes = t->h_row.size() * sizeof(RowTile);
+  } else {
+    return fail(ETHA_ERR_INVALID, "which must be 0 or 1");
+  }
+  *need_bytes = bytes;
+  if (out && bytes) memcpy(out, src, bytes < cap_bytes ? bytes : cap_bytes);
+  return ETHA_OK;
+}
+
+int etha_table_read_ranges(const EthaTable* t, uint32_t* run_begin, uint32_t* row_begin) {
+  if (!t || !run_begin || !row_begin) return fail(ETHA_ERR_INVALID, "null argument");
+  memcpy(run_begin, t->run_begin.data(), t->run_begin.size() * sizeof(uint32_t));
+  memcpy(row_begin, t->row_begin.data(), t->row_begin.size() * sizeof(uint32_t));
+  return ETHA_OK;
+}
+
+int etha_pack_bucket(const EthaTable* t, uint32_t first, uint32_t count, void* stream) {
+  const int rc = check_range(t, first, count, 0);
+  if (rc != ETHA_OK) return rc;
+  if (t->reduce_prefix[first + count] != t->reduce_prefix[first])
+    return fail(ETHA_ERR_INVALID, "range holds Partial chunks; use etha_reduce_pack_bucket");
+  return launch_tiles<false>(t, first, count, stream);
+}
+
+int etha_unpack_bucket(const EthaTable* t, uint32_t first, uint32_t count, void* stream) {
+  const int rc = check_range(t, first, count, 0);
+  if (rc != ETHA_OK) return rc;
+  if (t->reduce_prefix[first + count] != t->reduce_prefix[first])
+    return fail(ETHA_ERR_INVALID, "range holds Partial chunks; a Partial placement cannot be a target");
+  return launch_tiles<true>(t, first, count, stream);
+}
+
+int etha_reduce_pack_bucket(const EthaTable* t, uint32_t first, uint32_t count, void* stream) {
+  const int rc = check_range(t, first, count, 0);
+  if (rc != ETHA_OK) return rc;
+  if (t->reduce_prefix[first + count] - t->reduce_prefix[first] != count)
+    return fail(ETHA_ERR_INVALID, "range holds chunks that are not Partial chunks");
+  const uint32_t w0 = t->row_begin[first], w1 = t->row_begin[first + count];
+  if (w1 == w0) return ETHA_OK;
+  hipLaunchKernelGGL(etha_reduce_kernel, dim3(w1 - w0), dim3(kTileThreads), 0, (hipStream_t)stream, t->d_row + w0,
+                     t->d_peers);
+  HIP_TRY(hipGetLastError());
+  return ETHA_OK;
+}
+
+int etha_selfcopy_bucket(const EthaTable* t, uint32_t first, uint32_t count, void* stream) {
+  const int rc = check_range(t, first, count, 1);
+  if (rc != ETHA_OK) return rc;
+  return launch_tiles<false>(t, first, count, stream);
+}
+
+int etha_arena_create(uint64_t nbytes, void** out_ptr) {
+  if (!out_ptr || nbytes == 0) return fail(ETHA_ERR_INVALID, "bad arena request");
+  *out_ptr = nullptr;
+  HIP_TRY(hipMalloc(out_ptr, nbytes));
+  return ETHA_OK;
+}
+
+int etha_arena_destroy(void* ptr) {
+  if (ptr) HIP_TRY(hipFree(ptr));
+  return ETHA_OK;
+}
+
+int etha_ipc_export(const void* dev_ptr, EthaIpcHandle* out) {
+  if (!dev_ptr || !out) return fail(ETHA_ERR_INVALID, "null argument");
+  hipDeviceptr_t base = nullptr;
+  size_t size = 0;
+  HIP_TRY(hipMemGetAddressRange(&base, &size, (hipDeviceptr_t)dev_ptr));
+  hipIpcMemHandle_t h;
+  HIP_TRY(hipIpcGetMemHandle(&h, base));
+  static_assert(sizeof(h) == 64, "hipIpcMemHandle_t size");
+  memcpy(out->handle, &h, 64);
+  out->offset = (uint64_t)((const char*)dev_ptr - (const char*)base);
+  out->size = (uint64_t)size;
+  return ETHA_OK;
+}
+
+int etha_ipc_open(const EthaIpcHandle* handle, void** out_ptr) {
+  if (!handle || !out_ptr) return fail(ETHA_ERR_INVALID, "null argument");
+  *out_ptr = nullptr;
+  // shared allocations of 2 GiB and more have not opened reliably on this platform
+  if (handle->size >= (2ull << 30))
+    return fail(ETHA_ERR_UNSUPPORTED, "IPC allocation of %llu bytes: keep shared allocations under 2 GiB",
+                (unsigned long long)handle->size);
+  hipIpcMemHandle_t h;
+  memcpy(&h, handle->handle, 64);
+  void* base = nullptr;
+  HIP_TRY(hipIpcOpenMemHandle(&base, h, hipIpcMemLazyEnablePeerAccess));
+  *out_ptr = (char*)base + handle->offset;
+  std::lock_guard<std::mutex> lock(g_ipc_mutex);
+  g_ipc_bases[*out_ptr] = base;
+  return ETHA_OK;
+}
+
+int etha_ipc_close(void* opened_ptr) {
+  if (!opened_ptr) return ETHA_OK;
+  void* base = nullptr;
+  {
+    std::lock_guard<std::mutex> lock(g_ipc_mutex);
+    auto it = g_ipc_bases.find(opened_ptr);
+    if (it == g_ipc_bases.end()) return fail(ETHA_ERR_INVALID, "pointer was not returned by etha_ipc_open");
+    base = it->second;
+    g_ipc_bases.erase(it);
+  }
+  HIP_TRY(hipIpcCloseMemHandle(base));
+  return ETHA_OK;
+}
+
+}  // extern "C"

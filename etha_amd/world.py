@@ -1,0 +1,205 @@
+"""All ranks of a redistribute job resident on one GPU.
+
+The reference runs one agent process per rank and moves buckets between them with NCCL.  This
+build shows the part one GPU can show: every source rank's shards and every (selected) target
+rank's shards are tensors on the same device, each rank's chunk/bucket plan is built exactly as
+the per-rank agents would build it (``src/etha/tensor_bus/agent.py:543-687``), and the wire is the
+same-GPU loopback.  :class:`ReshardJob` is the harness the tests, the benchmark and the smoke check
+share.
+"""
+
+from __future__ import annotations
+
+from dataclasses import dataclass, field
+
+import numpy as np
+import torch
+from torch.distributed.tensor.placement_types import Partial
+
+from .comm import LoopbackWire, PartialGroup, bucket_comm, chunk_to_bucket_ops, get_m2m_map, m2m_to_chunks
+from .comm.utils import enumerate_partial_subgroup_ranks
+from .layout import local_shape, local_shard, mesh_coord
+
+
+@dataclass
+class TensorSpec:
+    """One logical tensor and its two layouts."""
+
+    name: str
+    shape: tuple[int, ...]
+    source_mesh: list  # nested list of global ranks
+    source_placements: tuple
+    target_mesh: list
+    target_placements: tuple
+    source_dtype: torch.dtype = torch.bfloat16
+    target_dtype: torch.dtype | None = None  # None = source dtype
+    seed: int = 0
+    std: float = 0.02
+    dist: str = "normal"  # "normal" | "uniform" (uniform(-1, 1))
+
+
+def transfer_dtype_rule(source: torch.dtype, target: torch.dtype) -> torch.dtype:
+    """Wire dtype: the side with the smaller item size; on a tie the source's dtype.
+
+    The reference lets each side pick its own dtype on a tie (``agent.py:635-640``), which makes
+    two equally wide but different dtypes (fp16 vs bf16) reinterpret each other's bits; choosing the
+    source's dtype on both sides turns that case into a real conversion at unpack time.
+    """
+    return source if source.itemsize <= target.itemsize else target
+
+
+def create_partial_groups(mesh, partial_reductions, this_rank: int, tensors_by_rank: dict[int, torch.Tensor]):
+    """Partial sub-groups ``this_rank`` belongs to, as (PartialGroup, op) pairs.
+
+    Same enumeration as ``_create_partial_groups`` (``agent.py:46-70``): for every Partial mesh
+    dim, every line of ranks along that dim that contains this rank.
+    """
+    groups = []
+    for mesh_dim, op in partial_reductions:
+        for sub in enumerate_partial_subgroup_ranks(mesh, mesh_dim):
+            if this_rank in sub:
+                ranks = sorted(sub)
+                groups.append((PartialGroup(ranks=ranks, tensors=[tensors_by_rank[r] for r in ranks]), op))
+    return groups
+
+
+def _flat_ranks(mesh) -> list[int]:
+    return [int(r) for r in np.asarray(mesh).reshape(-1)]
+
+
+def make_global(spec: TensorSpec, device, seed: int | None = None, shape=None) -> torch.Tensor:
+    """Synthetic values of a tensor: seeded normal(0, std) or uniform(-1, 1), generated in fp32."""
+    gen = torch.Generator(device=device)
+    gen.manual_seed(spec.seed if seed is None else seed)
+    shape = tuple(spec.shape if shape is None else shape)
+    if spec.dist == "uniform":
+        g = torch.rand(shape, generator=gen, device=device, dtype=torch.float32) * 2 - 1
+    else:
+        g = torch.randn(shape, generator=gen, device=device, dtype=torch.float32) * spec.std
+    return g.to(spec.source_dtype)
+
+
+@dataclass
+class ReshardJob:
+    """Shards, plans and execution of a batch of tensors on one GPU.
+
+    ``target_ranks`` limits the job to those target ranks' share (None = all); source buckets that
+    serve none of them are dropped, like a run where only those target agents exist.
+    ``fill`` controls source data: "random" (seeded per spec) or a callable ``spec -> global tensor``.
+    """
+
+    specs: list[TensorSpec]
+    device: torch.device | str = "cuda:0"
+    bucket_size: int | None = 64 << 20
+    target_ranks: list[int] | None = None
+    keep_globals: bool = False
+    fill: object = "random"
+    wire: LoopbackWire | None = None
+    source_locals: list[dict[int, torch.Tensor]] = field(default_factory=list, init=False)
+    target_locals: list[dict[int, torch.Tensor]] = field(default_factory=list, init=False)
+    globals_: list[torch.Tensor | None] = field(default_factory=list, init=False)
+    send_buckets: dict[int, list] = field(default_factory=dict, init=False)
+    recv_buckets: dict[int, list] = field(default_factory=dict, init=False)
+
+    def __post_init__(self) -> None:
+        self.device = torch.device(self.device)
+        if self.wire is None:
+            self.wire = LoopbackWire(self.device)
+        send_chunks: dict[int, list] = {}
+        recv_chunks: dict[int, list] = {}
+        m2m_cache: dict[tuple, object] = {}
+        wanted = set(self.target_ranks) if self.target_ranks is not None else None
+        for spec in self.specs:
+            src_mesh, tgt_mesh = np.asarray(spec.source_mesh), np.asarray(spec.target_mesh)
+            src_ranks, tgt_ranks = _flat_ranks(src_mesh), _flat_ranks(tgt_mesh)
+            tgt_dtype = spec.target_dtype or spec.source_dtype
+            partial = any(isinstance(p, Partial) for p in spec.source_placements)
+            # ---- stage the shards
+            src_local: dict[int, torch.Tensor] = {}
+            glob = None
+            if partial:
+                # every member holds a full-shape contribution with its own seed (seed + rank position)
+                for pos, r in enumerate(src_ranks):
+                    shape = local_shape(spec.shape, src_mesh.shape, spec.source_placements, mesh_coord(src_mesh.shape, pos))
+                    src_local[r] = make_global(spec, self.device, seed=spec.seed + pos, shape=shape)
+            else:
+                glob = self.fill(spec).to(self.device) if callable(self.fill) else make_global(spec, self.device)
+                for pos, r in enumerate(src_ranks):
+                    view = local_shard(glob, src_mesh.shape, spec.source_placements, mesh_coord(src_mesh.shape, pos))
+                    src_local[r] = view.clone(memory_format=torch.contiguous_format)
+            tgt_local: dict[int, torch.Tensor] = {}
+            for pos, r in enumerate(tgt_ranks):
+                if wanted is not None and r not in wanted:
+                    continue
+                shape = local_shape(spec.shape, tgt_mesh.shape, spec.target_placements, mesh_coord(tgt_mesh.shape, pos))
+                tgt_local[r] = torch.zeros(shape, dtype=tgt_dtype, device=self.device)
+            self.source_locals.append(src_local)
+            self.target_locals.append(tgt_local)
+            self.globals_.append(glob if self.keep_globals else None)
+            # ---- plan, rank by rank
+            key = (str(spec.source_mesh), spec.source_placements, str(spec.target_mesh), spec.target_placements)
+            if key not in m2m_cache:
+                m2m_cache[key] = get_m2m_map(src_mesh, spec.source_placements, tgt_mesh, spec.target_placements)
+            m2m = m2m_cache[key]
+            wire_dtype = transfer_dtype_rule(spec.source_dtype, tgt_dtype)
+            for r in sorted(set(src_ranks) | set(tgt_local)):
+                s_t = src_local.get(r)
+                t_t = tgt_local.get(r)
+                groups = None
+                if partial and s_t is not None:
+                    groups = create_partial_groups(src_mesh, m2m.source_partial_reductions, r, src_local) or None
+                for c in m2m_to_chunks(m2m, r, source_tensor=s_t, target_tensor=t_t, transfer_dtype=wire_dtype,
+                                       source_partial_groups=groups):
+                    if c.is_source:  # wire source, reduce-only, or LOCAL
+                        if wanted is not None and c.dst_ranks and not (set(c.dst_ranks) & wanted):
+                            continue
+                        if wanted is not None and not c.dst_ranks and not self._cell_wanted(m2m, c, wanted):
+                            continue
+                        send_chunks.setdefault(r, []).append(c)
+                    else:
+                        recv_chunks.setdefault(r, []).append(c)
+        size = self.bucket_size or 1
+        self.send_buckets = {r: chunk_to_bucket_ops(cs, size) for r, cs in sorted(send_chunks.items())}
+        self.recv_buckets = {r: chunk_to_bucket_ops(cs, size) for r, cs in sorted(recv_chunks.items())}
+
+    @staticmethod
+    def _cell_wanted(m2m, chunk, wanted) -> bool:
+        """A reduce-only chunk matters if the primary of its cell ships to a wanted rank."""
+        for route in m2m.routes:
+            if route.src.cell == tuple(chunk.src_idx) and any(d.rank in wanted for d in route.dsts):
+                return True
+        return False
+
+    # ------------------------------------------------------------------------------------------
+    def run_send(self, merge_launches: bool = False) -> None:
+        for buckets in self.send_buckets.values():
+            bucket_comm(buckets, wire=self.wire, merge_launches=merge_launches, synchronize=False)
+
+    def run_recv(self, merge_launches: bool = False) -> None:
+        for buckets in self.recv_buckets.values():
+            bucket_comm(buckets, wire=self.wire, merge_launches=merge_launches, synchronize=False)
+
+    def run(self, merge_launches: bool = False, synchronize: bool = True) -> None:
+        """One transfer: every source rank packs (and self-copies), then every target rank unpacks."""
+        self.run_send(merge_launches)
+        self.run_recv(merge_launches)
+        if synchronize:
+            torch.cuda.current_stream(self.device).synchronize()
+
+    def payload_bytes(self) -> int:
+        """Bytes the measured target ranks end up holding, in wire dtype (the reference's
+        effective-throughput numerator, ``bench/transfer_benchmark.py:339-360``)."""
+        total = 0
+        for buckets in self.recv_buckets.values():
+            total += sum(b.total_bytes for b in buckets)
+        for buckets in self.send_buckets.values():
+            total += sum(b.total_bytes for b in buckets if b.transport.value == "local")
+        return total
+
+    def counts(self) -> dict[str, int]:
+        return {
+            "send_buckets": sum(len(b) for b in self.send_buckets.values()),
+            "recv_buckets": sum(len(b) for b in self.recv_buckets.values()),
+            "send_chunks": sum(len(b.chunks) for bs in self.send_buckets.values() for b in bs),
+            "recv_chunks": sum(len(b.chunks) for bs in self.recv_buckets.values() for b in bs),
+        }

@@ -1,0 +1,175 @@
+/*
+ * etha_reshard.h — C ABI of the MI355X (gfx950) redistribute hot path.
+ *
+ * The library sits exactly under the two methods the reference's executor calls on
+ * every bucket: Bucket.prepare() (assemble the send bucket from strided chunks of
+ * the source shard, src/etha/comm/ir.py:229-264 with Chunk.prepare ir.py:101-132)
+ * and Bucket.finalize() (scatter a received bucket into the target shard,
+ * ir.py:300-310 with Chunk.finalize ir.py:134-141).  The host planner describes
+ * every chunk once ("plan once, transfer N times"); the library compiles the
+ * descriptors into a device-resident tile program and each transfer is then one
+ * batched kernel launch per bucket (or per run of buckets).
+ *
+ * Conventions
+ *  - plain C types only; every function returns 0 on success or a negative
+ *    ETHA_ERR_* code and never throws; etha_last_error() gives the message of the
+ *    calling thread's last failure.
+ *  - `stream` arguments are a hipStream_t passed as void* (NULL = default stream).
+ *    Launches are asynchronous; ordering is stream ordering, as in the reference
+ *    where all device work of a transfer goes to the current stream
+ *    (ir.py:262-275, comm_methods.py:119).
+ *  - the library never writes a tensor outside the described chunk regions and
+ *    never writes a source tensor at all (pinned by the reference's
+ *    tests/test_communication_replicate_shard.py:166-170,189-192).
+ */
+#ifndef ETHA_RESHARD_H
+#define ETHA_RESHARD_H
+
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define ETHA_ABI_VERSION 1
+#define ETHA_MAX_NDIM 8
+
+/* status codes */
+#define ETHA_OK 0
+#define ETHA_ERR_INVALID (-1)     /* bad argument / descriptor rejected by validation */
+#define ETHA_ERR_UNSUPPORTED (-2) /* legal in the reference but not implemented here */
+#define ETHA_ERR_HIP (-3)         /* a HIP runtime call failed */
+#define ETHA_ERR_NOMEM (-4)
+
+/* element types.  Same-type transfers are byte moves and work for every type;
+ * conversions are implemented between the four floating types only. */
+enum {
+  ETHA_F16 = 0,
+  ETHA_BF16 = 1,
+  ETHA_F32 = 2,
+  ETHA_F64 = 3,
+  ETHA_B8 = 4,   /* opaque 1-byte element (int8/uint8/bool/fp8) */
+  ETHA_B16 = 5,  /* opaque 2-byte element (int16/...) */
+  ETHA_B32 = 6,  /* opaque 4-byte element (int32/...) */
+  ETHA_B64 = 7   /* opaque 8-byte element (int64/complex32/...) */
+};
+
+/* reduce ops of a Partial source (ir.py:51-57) */
+enum { ETHA_SUM = 0, ETHA_AVG = 1, ETHA_MAX = 2, ETHA_MIN = 3, ETHA_PRODUCT = 4 };
+
+/*
+ * One chunk = one strided region of a local shard plus its place in a bucket.
+ * Information content of the reference's Chunk (ir.py:60-99) and of the bucket
+ * byte offset Bucket.offsets[i] (ir.py:189-194).
+ */
+typedef struct EthaChunkDesc {
+  uint64_t tensor_ptr;            /* device address of the parent tensor's element [0,..,0] (Tensor.data_ptr()) */
+  uint64_t tensor_lo, tensor_hi;  /* byte range [lo,hi) the library may touch on the tensor side; both 0 = unchecked */
+  uint64_t bucket_ptr;            /* device address of this chunk's first byte inside its bucket buffer */
+  uint64_t bucket_lo, bucket_hi;  /* byte range [lo,hi) of that bucket buffer; both 0 = unchecked */
+  int64_t start[ETHA_MAX_NDIM];   /* slice start per dim: src_slice when packing, dst_slice when unpacking */
+  int64_t shape[ETHA_MAX_NDIM];   /* chunk_shape */
+  int64_t stride[ETHA_MAX_NDIM];  /* parent tensor strides, in elements (non-contiguous parents are legal) */
+  uint32_t ndim;                  /* <= ETHA_MAX_NDIM; 0 = scalar (one element) */
+  uint32_t tensor_dtype;          /* ETHA_* element type of the tensor */
+  uint32_t wire_dtype;            /* ETHA_* element type inside the bucket (Chunk.transfer_dtype) */
+  uint32_t n_partials;            /* 0 = plain chunk.  >0 = Partial source: reduce this many peers (pack only) */
+  uint32_t partial_first;         /* index into partial_ptrs of the first peer's data_ptr(); peers in rank order */
+  uint32_t reduce_op;             /* ETHA_SUM.. when n_partials > 0 */
+} EthaChunkDesc;
+
+typedef struct EthaTable EthaTable; /* compiled, device-resident tile program */
+
+typedef struct EthaTableInfo {
+  uint32_t n_chunks;
+  uint32_t n_run_tiles;   /* tiles that are one contiguous run on both sides */
+  uint32_t n_row_tiles;   /* tiles that walk rows (short/ragged rows, strided elements, reduce) */
+  uint32_t tile_threads;  /* work-items per tile (= per workgroup) */
+  uint64_t device_bytes;  /* device memory held by the table */
+  uint64_t payload_bytes; /* sum over chunks of numel * wire element size */
+} EthaTableInfo;
+
+typedef struct EthaIpcHandle {
+  uint8_t handle[64]; /* hipIpcMemHandle_t */
+  uint64_t offset;    /* byte offset of the exported pointer from its allocation base */
+  uint64_t size;      /* size of the whole allocation */
+} EthaIpcHandle;
+
+int etha_abi_version(void);
+const char* etha_last_error(void);
+
+/*
+ * Compile chunk descriptors into a tile program.
+ *  descs/n_chunks     host array, chunk order = bucket order (chunks of one bucket adjacent,
+ *                     so that a bucket is a [first, first+count) range).
+ *  partial_ptrs       host array of peer data_ptr() values referenced by reduce chunks (may be NULL).
+ *  upload             non-zero: copy the program to the current HIP device (needed to launch);
+ *                     zero: keep it on the host only (planning/inspection without a GPU).
+ * Replaces the per-transfer Python work of Bucket.__post_init__/prepare (ir.py:189-194,246-259).
+ */
+int etha_table_create(const EthaChunkDesc* descs, uint32_t n_chunks, const uint64_t* partial_ptrs,
+                      uint32_t n_partial_ptrs, int upload, EthaTable** out);
+
+/*
+ * Same-rank (LOCAL transport) chunks: copy src region i to dst region i directly, no bucket.
+ * bucket_* fields are ignored; shapes must match pairwise; src.tensor_dtype is converted to
+ * dst.tensor_dtype.  Replaces the self-copy bucket path (ir.py:238-244,254-257,136-140).
+ */
+int etha_selfcopy_table_create(const EthaChunkDesc* src, const EthaChunkDesc* dst, uint32_t n_chunks, int upload,
+                               EthaTable** out);
+
+int etha_table_destroy(EthaTable* table);
+int etha_table_info(const EthaTable* table, EthaTableInfo* out);
+
+/*
+ * Inspection of the compiled program (host copies), for CPU-side checking.
+ * which: 0 = run tiles (uint64 a, b; uint32 n, meta), 1 = row tiles (see etha_reshard.hip).
+ * Copies up to cap_bytes into out and stores the full size in *need_bytes.
+ */
+int etha_table_read_tiles(const EthaTable* table, int which, void* out, uint64_t cap_bytes, uint64_t* need_bytes);
+/* per-chunk first-tile indices, n_chunks+1 entries each */
+int etha_table_read_ranges(const EthaTable* table, uint32_t* run_begin, uint32_t* row_begin);
+
+/*
+ * Gather chunks [first, first+count) of the table from their tensors into their bucket
+ * positions, converting tensor_dtype -> wire_dtype.  One kernel launch.
+ * Replaces Bucket.prepare() for a source bucket (ir.py:229-264; Chunk.prepare ir.py:112-126).
+ * The range must not contain reduce chunks.
+ */
+int etha_pack_bucket(const EthaTable* table, uint32_t first, uint32_t count, void* stream);
+
+/*
+ * Scatter chunks [first, first+count) from their bucket positions into their tensors,
+ * converting wire_dtype -> tensor_dtype.  One kernel launch.
+ * Replaces Bucket.finalize() for a target bucket (ir.py:300-310; Chunk.finalize ir.py:134-141).
+ */
+int etha_unpack_bucket(const EthaTable* table, uint32_t first, uint32_t count, void* stream);
+
+/*
+ * Partial-source buckets: for every chunk combine the n_partials peer regions element-wise
+ * (fp32 accumulation in rank order for f16/bf16/f32 inputs, f64 for f64), convert to
+ * wire_dtype once, and write the bucket.  One kernel launch; the peers are only read.
+ * Replaces the clone + all_reduce + cast of Chunk.prepare (ir.py:116-126).
+ * Every chunk of the range must be a reduce chunk.
+ */
+int etha_reduce_pack_bucket(const EthaTable* table, uint32_t first, uint32_t count, void* stream);
+
+/* Run chunks [first, first+count) of a self-copy table.  One kernel launch. */
+int etha_selfcopy_bucket(const EthaTable* table, uint32_t first, uint32_t count, void* stream);
+
+/*
+ * Bucket-pool memory that can cross a process boundary on the same GPU (the worker <-> agent
+ * hand-off the reference does with CUDA-IPC pickling, tensor_bus/client.py:314,
+ * tensor_bus/agent.py:608, tensor_bus/utils.py:14-69).  etha_arena_create is a plain
+ * hipMalloc so that the allocation base can be exported.
+ */
+int etha_arena_create(uint64_t nbytes, void** out_ptr);
+int etha_arena_destroy(void* ptr);
+int etha_ipc_export(const void* dev_ptr, EthaIpcHandle* out);
+int etha_ipc_open(const EthaIpcHandle* handle, void** out_ptr); /* returns base + offset */
+int etha_ipc_close(void* opened_ptr);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* ETHA_RESHARD_H */

@@ -1,0 +1,92 @@
+"""Shared test plumbing: identical inputs for the HIP path (GPU) and the oracle (CPU)."""
+
+from __future__ import annotations
+
+import copy
+
+import numpy as np
+import torch
+
+from etha_amd.world import ReshardJob, TensorSpec
+from oracle import dtensor_layout, reference_path
+
+
+def cpu_fill(spec: TensorSpec) -> torch.Tensor:
+    """Seeded values generated on the CPU so that GPU and CPU jobs see the same bits."""
+    gen = torch.Generator(device="cpu")
+    gen.manual_seed(spec.seed)
+    if spec.dist == "uniform":
+        g = torch.rand(spec.shape, generator=gen, dtype=torch.float32) * 2 - 1
+    elif spec.dist == "bits":  # every bit pattern class, for byte-move tests
+        n = int(np.prod(spec.shape))
+        raw = torch.randint(0, 256, (n * spec.source_dtype.itemsize,), generator=gen, dtype=torch.uint8)
+        return raw.view(spec.source_dtype).reshape(spec.shape)
+    else:
+        g = torch.randn(spec.shape, generator=gen, dtype=torch.float32) * spec.std
+    return g.to(spec.source_dtype)
+
+
+def mirror_partials(gpu_job: ReshardJob, cpu_job: ReshardJob) -> None:
+    """Partial sources are generated per device; make the CPU job's partials equal the GPU job's."""
+    for g_src, c_src in zip(gpu_job.source_locals, cpu_job.source_locals):
+        for r, t in c_src.items():
+            t.copy_(g_src[r].cpu())
+
+
+def run_oracle(cpu_job: ReshardJob) -> None:
+    """Execute a CPU-resident job with the oracle's restatement of the reference path."""
+    box = reference_path.Mailbox()
+    for r, buckets in cpu_job.send_buckets.items():
+        reference_path.run_rank(buckets, box, rank=r)
+    for r, buckets in cpu_job.recv_buckets.items():
+        reference_path.run_rank(buckets, box, rank=r)
+
+
+def expected_target(spec: TensorSpec, glob: torch.Tensor, rank: int) -> torch.Tensor:
+    """Closed form: the DTensor slice of the global tensor, through the wire dtype, in target dtype."""
+    from etha_amd.world import transfer_dtype_rule
+
+    mesh = np.asarray(spec.target_mesh)
+    pos = [int(x) for x in mesh.reshape(-1)].index(rank)
+    shard = dtensor_layout.local_shard(glob, mesh.shape, spec.target_placements, dtensor_layout.mesh_coord(mesh.shape, pos))
+    tgt = spec.target_dtype or spec.source_dtype
+    return shard.to(transfer_dtype_rule(spec.source_dtype, tgt)).to(tgt)
+
+
+def bits(t: torch.Tensor) -> torch.Tensor:
+    """Raw bytes of a tensor, for bit-exact comparison (NaNs and -0 included)."""
+    return t.detach().cpu().contiguous().view(torch.uint8).reshape(-1)
+
+
+def assert_bit_equal(a: torch.Tensor, b: torch.Tensor, what: str = "") -> None:
+    assert a.shape == b.shape and a.dtype == b.dtype, f"{what}: {a.shape}/{a.dtype} vs {b.shape}/{b.dtype}"
+    ba, bb = bits(a), bits(b)
+    if not torch.equal(ba, bb):
+        bad = (ba != bb).nonzero().reshape(-1)
+        raise AssertionError(f"{what}: {bad.numel()} differing bytes, first at byte {int(bad[0])}")
+
+
+def clone_specs(specs):
+    return [copy.copy(s) for s in specs]
+
+
+def gpu_vs_oracle(specs, device, bucket_size, target_ranks=None, merge_launches=False, check_closed_form=True):
+    """Run the same job on the GPU (HIP path) and on the CPU (oracle); compare every target shard."""
+    gpu_job = ReshardJob(clone_specs(specs), device=device, bucket_size=bucket_size, target_ranks=target_ranks,
+                         keep_globals=True, fill=cpu_fill)
+    cpu_job = ReshardJob(clone_specs(specs), device="cpu", bucket_size=bucket_size, target_ranks=target_ranks,
+                         keep_globals=True, fill=cpu_fill)
+    mirror_partials(gpu_job, cpu_job)
+    src_before = [{r: t.clone() for r, t in d.items()} for d in gpu_job.source_locals]
+    gpu_job.run(merge_launches=merge_launches)
+    run_oracle(cpu_job)
+    for i, spec in enumerate(specs):
+        for r, t in gpu_job.target_locals[i].items():
+            assert_bit_equal(t, cpu_job.target_locals[i][r], f"{spec.name} target rank {r} vs oracle")
+            if check_closed_form and gpu_job.globals_[i] is not None:
+                assert_bit_equal(t, expected_target(spec, cpu_job.globals_[i], r), f"{spec.name} rank {r} vs closed form")
+        for r, t in gpu_job.source_locals[i].items():
+            same_obj = any(t is x for x in gpu_job.target_locals[i].values())
+            if not same_obj:
+                assert_bit_equal(t, src_before[i][r], f"{spec.name} source rank {r} mutated")
+    return gpu_job, cpu_job
