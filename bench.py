@@ -1,0 +1,223 @@
+"""Headline benchmark: effective reshard GB/s (pack + unpack) on one MI355X.
+
+One step = one pass of the hot path over the workload: every source rank packs its buckets for the
+measured target rank's share, then that target rank unpacks them.  Inputs are resident in HBM
+before the timed region.  Prints ONE JSON line.
+
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload NAME] [--per-bucket]
+"""
+
+from __future__ import annotations
+
+import argparse
+import json
+import os
+import sys
+import time
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+sys.path.insert(0, ROOT)
+
+HBM_PEAK_GBS = 8000.0  # MI355X HBM3E, published
+
+
+def parse_args():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=20)
+    ap.add_argument("--warmup", type=int, default=3)
+    ap.add_argument("--workload", default="llama3_8b_fsdp8_to_tp2")
+    ap.add_argument("--per-bucket", action="store_true", help="one launch per bucket instead of one per run of buckets")
+    ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--cpu-layers", type=int, default=2, help="layers of the workload the CPU baseline sample covers")
+    return ap.parse_args()
+
+
+def cpu_baseline(workload: str, layers: int):
+    """The oracle's op-for-op restatement of the reference path, timed on this host's cores."""
+    import torch
+
+    from etha_amd import workloads
+    from etha_amd.world import ReshardJob
+    from oracle import reference_path
+
+    if workload == "llama3_8b_fsdp8_to_tp2":
+        specs, targets, bucket = workloads.llama3_8b_fsdp8_to_tp2(n_layers=layers, with_embeddings=False)
+        sample = f"{layers} decoder layers of the workload (no embeddings), same layouts and 64 MiB buckets"
+    else:
+        specs, targets, bucket = workloads.WORKLOADS[workload]()
+        sample = "whole workload"
+
+    def cheap_fill(spec):  # values do not affect timing; avoid minutes of CPU randn
+        n = 1
+        for s in spec.shape:
+            n *= s
+        return (torch.arange(n, dtype=torch.int32) % 251).to(spec.source_dtype).reshape(spec.shape)
+
+    job = ReshardJob(specs, device="cpu", bucket_size=bucket, target_ranks=targets, fill=cheap_fill)
+    payload = job.payload_bytes()
+
+    def one_pass():
+        box = reference_path.Mailbox()
+        for r, buckets in job.send_buckets.items():
+            reference_path.run_rank(buckets, box, rank=r)
+        for r, buckets in job.recv_buckets.items():
+            reference_path.run_rank(buckets, box, rank=r)
+
+    one_pass()
+    times = []
+    t_end = time.perf_counter() + 20.0
+    while len(times) < 10 and (len(times) < 3 or time.perf_counter() < t_end):
+        t0 = time.perf_counter()
+        one_pass()
+        times.append(time.perf_counter() - t0)
+    times.sort()
+    med = times[len(times) // 2]
+    return {
+        "value": payload / med / 1e9,
+        "unit": "GB/s",
+        "cores": torch.get_num_threads(),
+        "kind": "port",
+        "sample": f"{sample}; {payload} payload bytes per pass, median of {len(times)} passes",
+        "host_cpus": os.cpu_count(),
+    }
+
+
+def main():
+    args = parse_args()
+    if args.gpus != 1:
+        print("bench.py measures one GPU's share of the reshard; runs with --gpus > 1 are not part of this build",
+              file=sys.stderr)
+        sys.exit(2)
+    import torch
+
+    from etha_amd import _native, workloads
+    from etha_amd.world import ReshardJob
+
+    _native.lib()
+    if not torch.cuda.is_available():
+        print("bench.py needs a GPU: the hot path has no CPU fallback", file=sys.stderr)
+        sys.exit(1)
+    dev = torch.device("cuda:0")
+    torch.cuda.set_device(dev)
+    specs, targets, bucket = workloads.WORKLOADS[args.workload]()
+    t0 = time.time()
+    job = ReshardJob(specs, device=dev, bucket_size=bucket, target_ranks=targets)
+    merge = not args.per_bucket
+    # plan (compiles the tile programs) + warm-up
+    for _ in range(max(args.warmup, 1)):
+        job.run(merge_launches=merge)
+    setup_s = time.time() - t0
+
+    S = job.payload_bytes()
+    send_plans = [job.wire.plan(b) for b in job.send_buckets.values()]
+    recv_plans = [job.wire.plan(b) for b in job.recv_buckets.values()]
+    steps_of = (lambda p: p.merged_steps) if merge else (lambda p: p.steps)
+    n_pack = sum(1 for p in send_plans for s in steps_of(p) if s[0] in ("pack", "reduce_pack"))
+    n_self = sum(1 for p in send_plans + recv_plans for s in steps_of(p) if s[0] == "selfcopy")
+    n_unpack = sum(1 for p in send_plans + recv_plans for s in steps_of(p) if s[0] == "unpack")
+
+    # algorithmic bytes: pack reads the source dtype and writes the wire dtype; unpack reads the wire
+    # dtype and writes the target dtype; a reduce-pack reads every member's partial
+    def table_bytes(plan, which):
+        t = getattr(plan, which)
+        return t.info().payload_bytes if t is not None else 0
+
+    wire_bytes = sum(table_bytes(p, "send_table") for p in send_plans)
+    pack_read = 0
+    for p in send_plans:
+        for b in p.buckets:
+            if b.transport.value in ("p2p", "broadcast") and b.is_source:
+                for c in b.chunks:
+                    peers = c.partial_peers()
+                    n = 1
+                    for d in c.chunk_shape:
+                        n *= d
+                    pack_read += n * c.tensor.element_size() * (len(peers[0]) if peers else 1)
+    unpack_write = 0
+    for p in recv_plans:
+        for b in p.buckets:
+            for c in b.chunks:
+                n = 1
+                for d in c.chunk_shape:
+                    n *= d
+                unpack_write += n * c.tensor.element_size()
+    unpack_read = sum(table_bytes(p, "recv_table") for p in recv_plans)
+    pack_bytes = pack_read + wire_bytes
+    unpack_bytes = unpack_read + unpack_write
+
+    stream = torch.cuda.current_stream(dev)
+    ev = [[torch.cuda.Event(enable_timing=True) for _ in range(3)] for _ in range(args.steps)]
+    torch.cuda.synchronize()
+    wall0 = time.perf_counter()
+    for k in range(args.steps):
+        ev[k][0].record(stream)
+        job.run_send(merge)
+        ev[k][1].record(stream)
+        job.run_recv(merge)
+        ev[k][2].record(stream)
+    torch.cuda.synchronize()
+    wall = time.perf_counter() - wall0
+    pack_ms = [ev[k][0].elapsed_time(ev[k][1]) for k in range(args.steps)]
+    unpack_ms = [ev[k][1].elapsed_time(ev[k][2]) for k in range(args.steps)]
+    step_ms = wall * 1e3 / args.steps
+    pack_avg, unpack_avg = sum(pack_ms) / len(pack_ms), sum(unpack_ms) / len(unpack_ms)
+    dev_ms = pack_avg + unpack_avg
+
+    value = S / (step_ms * 1e-3) / 1e9
+    pack_gbs = pack_bytes / (pack_avg * 1e-3) / 1e9
+    unpack_gbs = unpack_bytes / (unpack_avg * 1e-3) / 1e9 if unpack_avg > 0 else 0.0
+    dominant = "pack" if pack_avg >= unpack_avg else "unpack"
+    dom_bytes, dom_ms, dom_launches = (
+        (pack_bytes, pack_avg, max(n_pack, 1)) if dominant == "pack" else (unpack_bytes, unpack_avg, max(n_unpack, 1))
+    )
+    kernel_name = {"pack": "etha_tile_kernel<false>", "unpack": "etha_tile_kernel<true>"}[dominant]
+    if dominant == "pack" and any(s[0] == "reduce_pack" for p in send_plans for s in steps_of(p)):
+        kernel_name = "etha_reduce_kernel"
+    achieved = dom_bytes / (dom_ms * 1e-3) / 1e9
+    out = {
+        "metric": "effective reshard GB/s (pack+unpack, 1 GPU) and % of HBM peak",
+        "value": round(value, 2),
+        "unit": "GB/s",
+        "n_gpus": 1,
+        "steps": args.steps,
+        "warmup": args.warmup,
+        "ms_per_step": round(step_ms, 4),
+        "higher_is_better": True,
+        "scaling": "weak",
+        "vs_baseline": None,
+        "dtype": "u8" if pack_read == wire_bytes else "f32",
+        "data": "synthetic",
+        "config": {
+            "workload": args.workload,
+            "payload_bytes": S,
+            "bucket_bytes": bucket,
+            "launch_granularity": "run of buckets" if merge else "bucket",
+            **job.counts(),
+        },
+        "device_ms_per_step": round(dev_ms, 4),
+        "pct_of_hbm_peak": round(100.0 * (pack_bytes + unpack_bytes) / (dev_ms * 1e-3) / 1e9 / HBM_PEAK_GBS, 2),
+        "pack": {"GB/s": round(pack_gbs, 1), "ms": round(pack_avg, 4), "bytes": pack_bytes, "launches": n_pack},
+        "unpack": {"GB/s": round(unpack_gbs, 1), "ms": round(unpack_avg, 4), "bytes": unpack_bytes, "launches": n_unpack},
+        "selfcopy_launches": n_self,
+        "roofline": {
+            "bound": "hbm",
+            "kernel": kernel_name,
+            "achieved": round(achieved, 1),
+            "peak": HBM_PEAK_GBS,
+            "unit": "GB/s",
+            "frac": round(achieved / HBM_PEAK_GBS, 4),
+            "traffic": None,
+            "bytes_per_launch": dom_bytes // dom_launches,
+            "avg_launch_ms": round(dom_ms / dom_launches, 5),
+            "launches_per_step": dom_launches,
+        },
+        "setup_s": round(setup_s, 1),
+    }
+    if not args.no_cpu_baseline:
+        out["cpu_baseline"] = cpu_baseline(args.workload, args.cpu_layers)
+    print(json.dumps(out))
+
+
+if __name__ == "__main__":
+    main()

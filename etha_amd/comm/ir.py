@@ -149,24 +149,21 @@ class Chunk:
     def partial_peers(self) -> tuple[tuple[torch.Tensor, ...], str] | None:
         """Peers (rank order) and op of this chunk's Partial collapse, or None.
 
-        The reference runs one in-place all-reduce per group in sequence (``ir.py:123-124``); with
-        one op that equals a single reduction over the union of the groups' members, which is
-        what is returned here.  Different ops on different mesh dims are not supported.
+        The reference runs one in-place all-reduce per sub-group in sequence (``ir.py:123-124``),
+        which reduces over the whole connected component of the Partial mesh dims.  Here that
+        component must be given as ONE group (``etha_amd.world.create_partial_groups`` builds it):
+        the union of a rank's own per-dim sub-groups would miss members that share no line with it.
         """
         if not self.source_partial_groups:
             return None
-        ops = {op for _, op in self.source_partial_groups}
-        if len(ops) != 1:
-            raise NotImplementedError(f"Partial dims with different reduce ops {sorted(ops)} are not supported")
-        op = ops.pop()
+        if len(self.source_partial_groups) != 1:
+            raise NotImplementedError(
+                "pass one PartialGroup covering the whole Partial connected component, not one per mesh dim"
+            )
+        group, op = self.source_partial_groups[0]
         if op not in REDUCE_OPS:
             raise ValueError(f"unknown reduce op {op!r}")
-        members: dict[int, torch.Tensor] = {}
-        for group, _ in self.source_partial_groups:
-            for r, t in zip(group.ranks, group.tensors):
-                members[r] = t
-        ranks = sorted(members)
-        return tuple(members[r] for r in ranks), op
+        return group.tensors, op
 
 
 @dataclass(kw_only=True, eq=False)

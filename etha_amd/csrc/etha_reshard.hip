@@ -109,7 +109,13 @@ struct TagF64 { typedef uint64_t bits; };
 __device__ __forceinline__ float to_f32(TagF16, uint16_t x) { return (float)__builtin_bit_cast(_Float16, x); }
 __device__ __forceinline__ float to_f32(TagBF16, uint16_t x) { return __builtin_bit_cast(float, (uint32_t)x << 16); }
 __device__ __forceinline__ float to_f32(TagF32, uint32_t x) { return __builtin_bit_cast(float, x); }
-__device__ __forceinline__ float to_f32(TagF64, uint64_t x) { return (float)__builtin_bit_cast(double, x); }
+// f64 -> narrower float is two roundings (f64 -> f32 -> target), as c10::Half(double) and
+// c10::BFloat16(double) do; the empty asm keeps the compiler from fusing them into one rounding.
+__device__ __forceinline__ float to_f32(TagF64, uint64_t x) {
+  float f = (float)__builtin_bit_cast(double, x);
+  asm volatile("" : "+v"(f));
+  return f;
+}
 
 __device__ __forceinline__ uint16_t from_f32(TagF16, float f) { return __builtin_bit_cast(uint16_t, (_Float16)f); }
 // round-to-nearest-even on the bit pattern; every NaN becomes the canonical quiet NaN 0x7FC0
@@ -291,8 +297,11 @@ __device__ __forceinline__ void reduce_f64(const uint64_t* __restrict__ peers, u
     if (op == ETHA_AVG) r = r / (double)np;
     if (sizeof(typename D::bits) == 8)
       out.set(i, (typename D::bits)__builtin_bit_cast(uint64_t, r));
-    else
-      out.set(i, from_f32(D(), (float)r));
+    else {
+      float rf = (float)r;
+      asm volatile("" : "+v"(rf));  // two roundings, as in the plain f64 -> D move
+      out.set(i, from_f32(D(), rf));
+    }
   }
   out.store(dst);
 }
@@ -399,7 +408,6 @@ int tensor_region(const EthaChunkDesc& d, uint32_t idx, uint64_t base_ptr, bool 
   const int es = dtype_size(d.tensor_dtype);
   if (es == 0) return fail(ETHA_ERR_INVALID, "chunk %u: unknown tensor_dtype %u", idx, d.tensor_dtype);
   if (d.ndim > ETHA_MAX_NDIM) return fail(ETHA_ERR_INVALID, "chunk %u: ndim %u > %d", idx, d.ndim, ETHA_MAX_NDIM);
-  if (base_ptr == 0 && !relative) return fail(ETHA_ERR_INVALID, "chunk %u: null tensor pointer", idx);
   Region r;
   r.nd = (int)d.ndim;
   __int128 off = 0, lo = 0, hi = 0;
@@ -414,6 +422,8 @@ int tensor_region(const EthaChunkDesc& d, uint32_t idx, uint64_t base_ptr, bool 
     const __int128 ext = (__int128)(d.shape[i] - 1) * d.stride[i] * es;
     if (d.shape[i] > 0) (ext < 0 ? lo : hi) += ext;
   }
+  // an empty tensor has no storage and a null data pointer; it also produces no tiles
+  if (base_ptr == 0 && !relative && !empty) return fail(ETHA_ERR_INVALID, "chunk %u: null tensor pointer", idx);
   const __int128 first = (__int128)base_ptr + off;
   if (first < 0 || first > (__int128)UINT64_MAX) return fail(ETHA_ERR_INVALID, "chunk %u: address overflow", idx);
   r.base = (uint64_t)first;

@@ -1,0 +1,106 @@
+"""Synthetic workloads: the layouts and shapes the headline numbers are quoted on.
+
+Each builder returns ``(specs, target_ranks, bucket_size)`` for :class:`etha_amd.world.ReshardJob`.
+Source ranks are numbered from 0; target ranks follow the source ranks unless a workload says
+otherwise (overlapping rank sets are what creates same-rank LOCAL chunks).
+"""
+
+from __future__ import annotations
+
+import numpy as np
+import torch
+from torch.distributed.tensor.placement_types import Partial, Replicate, Shard
+
+from .world import TensorSpec
+
+MIB = 1 << 20
+
+
+def _mesh(start: int, shape) -> list:
+    n = int(np.prod(shape))
+    return np.arange(start, start + n).reshape(shape).tolist()
+
+
+def single_fp32_shard0_to_shard1():
+    """fp32 [1024,1024] uniform(-1,1) seed 0; mesh (2,) Shard(0) -> mesh (4,) Shard(1)."""
+    spec = TensorSpec("w", (1024, 1024), _mesh(0, (2,)), (Shard(0),), _mesh(2, (4,)), (Shard(1),),
+                      torch.float32, seed=0, dist="uniform")
+    return [spec], None, None
+
+
+def llama3_8b_fsdp8_to_tp2(n_layers: int = 32, with_embeddings: bool = True, dtype=torch.bfloat16,
+                           hidden: int = 4096, inter: int = 14336, kv: int = 1024, vocab: int = 128256):
+    """Llama-3-8B weight set, FSDP Shard(0) over 8 ranks -> TP=2; one TP rank's share.
+
+    Column-parallel (q/k/v/gate/up/embed/lm_head): Shard(0) -> Shard(0).  Row-parallel (o/down):
+    Shard(0) -> Shard(1).  RMSNorm weights: Shard(0) -> Replicate.  Values normal(0, 0.02), seed =
+    tensor index.  290 tensors at the full size.
+    """
+    src, tgt = _mesh(0, (8,)), _mesh(8, (2,))
+    col, row, rep = (Shard(0),), (Shard(1),), (Replicate(),)
+    specs: list[TensorSpec] = []
+
+    def add(name, shape, tgt_pl):
+        specs.append(TensorSpec(name, shape, src, (Shard(0),), tgt, tgt_pl, dtype, seed=len(specs)))
+
+    if with_embeddings:
+        add("embed_tokens", (vocab, hidden), col)
+    for i in range(n_layers):
+        add(f"layers.{i}.input_layernorm", (hidden,), rep)
+        add(f"layers.{i}.q_proj", (hidden, hidden), col)
+        add(f"layers.{i}.k_proj", (kv, hidden), col)
+        add(f"layers.{i}.v_proj", (kv, hidden), col)
+        add(f"layers.{i}.o_proj", (hidden, hidden), row)
+        add(f"layers.{i}.post_attention_layernorm", (hidden,), rep)
+        add(f"layers.{i}.gate_proj", (inter, hidden), col)
+        add(f"layers.{i}.up_proj", (inter, hidden), col)
+        add(f"layers.{i}.down_proj", (hidden, inter), row)
+    if with_embeddings:
+        add("lm_head", (vocab, hidden), col)
+    return specs, [8], 64 * MIB
+
+
+def many_small_2d_to_replicate(n_tensors: int = 256, rows: int = 2048, k_seed: int = 1234, dtype=torch.bfloat16):
+    """256 bf16 [2048, k], k uniform over {64, 128, ..., 4096} (numpy RandomState(1234));
+    mesh (2,4) (Shard(0), Shard(1)) -> mesh (4,) Replicate; one target rank; 64 MiB buckets."""
+    ks = np.random.RandomState(k_seed).randint(1, 65, size=n_tensors) * 64
+    src, tgt = _mesh(0, (2, 4)), _mesh(8, (4,))
+    specs = [
+        TensorSpec(f"t{i}", (rows, int(k)), src, (Shard(0), Shard(1)), tgt, (Replicate(),), dtype, seed=i)
+        for i, k in enumerate(ks)
+    ]
+    return specs, [8], 64 * MIB
+
+
+def partial4_to_shard2(n_tensors: int = 16, n: int = 8192, dtype=torch.bfloat16):
+    """16 bf16 [8192,8192], mesh (4,) Partial(sum) -> mesh (2,) Shard(0); one target rank.
+    Partial of source rank r of tensor i: normal(0, 0.02) with seed 4*i + r."""
+    src, tgt = _mesh(0, (4,)), _mesh(4, (2,))
+    specs = [
+        TensorSpec(f"p{i}", (n, n), src, (Partial("sum"),), tgt, (Shard(0),), dtype, seed=4 * i)
+        for i in range(n_tensors)
+    ]
+    return specs, [4], 64 * MIB
+
+
+def moe_experts_and_uneven_vocab(n_experts: int = 8, hidden: int = 4096, inter: int = 14336, vocab: int = 151936,
+                                 dtype=torch.bfloat16):
+    """Mixtral-style grouped experts Shard(0)@8 -> Shard(1)@4 and a 151936-row embedding
+    Shard(0)@6 (uneven tail shard) -> Shard(1)@4.  Target ranks 0..3 overlap the source ranks, so
+    chunks whose source and destination rank coincide take the LOCAL (self-copy) path."""
+    specs = [
+        TensorSpec("experts.w1", (n_experts, inter, hidden), _mesh(0, (8,)), (Shard(0),), _mesh(0, (4,)), (Shard(1),), dtype, seed=0),
+        TensorSpec("experts.w3", (n_experts, inter, hidden), _mesh(0, (8,)), (Shard(0),), _mesh(0, (4,)), (Shard(1),), dtype, seed=1),
+        TensorSpec("experts.w2", (n_experts, hidden, inter), _mesh(0, (8,)), (Shard(0),), _mesh(0, (4,)), (Shard(1),), dtype, seed=2),
+        TensorSpec("embed_tokens", (vocab, hidden), _mesh(0, (6,)), (Shard(0),), _mesh(0, (4,)), (Shard(1),), dtype, seed=3),
+    ]
+    return specs, [0], 64 * MIB
+
+
+WORKLOADS = {
+    "single_fp32_shard0_to_shard1": single_fp32_shard0_to_shard1,
+    "llama3_8b_fsdp8_to_tp2": llama3_8b_fsdp8_to_tp2,
+    "many_small_2d_to_replicate": many_small_2d_to_replicate,
+    "partial4_to_shard2": partial4_to_shard2,
+    "moe_experts_and_uneven_vocab": moe_experts_and_uneven_vocab,
+}

@@ -14,10 +14,9 @@ from dataclasses import dataclass, field
 
 import numpy as np
 import torch
-from torch.distributed.tensor.placement_types import Partial
+from torch.distributed.tensor.placement_types import Partial, Replicate
 
 from .comm import LoopbackWire, PartialGroup, bucket_comm, chunk_to_bucket_ops, get_m2m_map, m2m_to_chunks
-from .comm.utils import enumerate_partial_subgroup_ranks
 from .layout import local_shape, local_shard, mesh_coord
 
 
@@ -49,18 +48,28 @@ def transfer_dtype_rule(source: torch.dtype, target: torch.dtype) -> torch.dtype
 
 
 def create_partial_groups(mesh, partial_reductions, this_rank: int, tensors_by_rank: dict[int, torch.Tensor]):
-    """Partial sub-groups ``this_rank`` belongs to, as (PartialGroup, op) pairs.
+    """The Partial reduction ``this_rank`` takes part in, as a one-element list of (PartialGroup, op).
 
-    Same enumeration as ``_create_partial_groups`` (``agent.py:46-70``): for every Partial mesh
-    dim, every line of ranks along that dim that contains this rank.
+    The reference builds one process group per Partial mesh dim and line of ranks
+    (``_create_partial_groups``, ``agent.py:46-70``) and all-reduces over them one after the other
+    (``ir.py:123-124``); the net effect is one reduction over every rank that differs from this one
+    only in Partial mesh coordinates.  That whole set is returned as a single group, so that the
+    reduce kernel can combine all members in one pass, in rank order.
     """
-    groups = []
-    for mesh_dim, op in partial_reductions:
-        for sub in enumerate_partial_subgroup_ranks(mesh, mesh_dim):
-            if this_rank in sub:
-                ranks = sorted(sub)
-                groups.append((PartialGroup(ranks=ranks, tensors=[tensors_by_rank[r] for r in ranks]), op))
-    return groups
+    if not partial_reductions:
+        return []
+    ops = {op for _, op in partial_reductions}
+    if len(ops) != 1:
+        raise NotImplementedError(f"Partial dims with different reduce ops {sorted(ops)} are not supported")
+    mesh = np.asarray(mesh)
+    where = np.argwhere(mesh == this_rank)
+    if len(where) != 1:
+        raise ValueError(f"rank {this_rank} is not a unique member of the source mesh")
+    index: list = [int(c) for c in where[0]]
+    for mesh_dim, _ in partial_reductions:
+        index[mesh_dim] = slice(None)
+    ranks = sorted(int(r) for r in np.asarray(mesh[tuple(index)]).reshape(-1))
+    return [(PartialGroup(ranks=ranks, tensors=[tensors_by_rank[r] for r in ranks]), ops.pop())]
 
 
 def _flat_ranks(mesh) -> list[int]:
@@ -95,6 +104,7 @@ class ReshardJob:
     keep_globals: bool = False
     fill: object = "random"
     wire: LoopbackWire | None = None
+    local_view: object = None  # optional ``(kind, tensor) -> view``: re-home a local shard inside another parent
     source_locals: list[dict[int, torch.Tensor]] = field(default_factory=list, init=False)
     target_locals: list[dict[int, torch.Tensor]] = field(default_factory=list, init=False)
     globals_: list[torch.Tensor | None] = field(default_factory=list, init=False)
@@ -118,21 +128,31 @@ class ReshardJob:
             src_local: dict[int, torch.Tensor] = {}
             glob = None
             if partial:
-                # every member holds a full-shape contribution with its own seed (seed + rank position)
+                # every member holds its own contribution: seed + flat position, where replicated mesh
+                # dims do not count (replicas of a Partial layout hold identical contributions)
                 for pos, r in enumerate(src_ranks):
-                    shape = local_shape(spec.shape, src_mesh.shape, spec.source_placements, mesh_coord(src_mesh.shape, pos))
-                    src_local[r] = make_global(spec, self.device, seed=spec.seed + pos, shape=shape)
+                    coord = list(mesh_coord(src_mesh.shape, pos))
+                    shape = local_shape(spec.shape, src_mesh.shape, spec.source_placements, coord)
+                    for i, p in enumerate(spec.source_placements):
+                        if isinstance(p, Replicate):
+                            coord[i] = 0
+                    canon = int(np.ravel_multi_index(coord, src_mesh.shape))
+                    src_local[r] = make_global(spec, self.device, seed=spec.seed + canon, shape=shape)
             else:
                 glob = self.fill(spec).to(self.device) if callable(self.fill) else make_global(spec, self.device)
                 for pos, r in enumerate(src_ranks):
                     view = local_shard(glob, src_mesh.shape, spec.source_placements, mesh_coord(src_mesh.shape, pos))
                     src_local[r] = view.clone(memory_format=torch.contiguous_format)
+            if self.local_view is not None:
+                src_local = {r: self._rehome("source", t) for r, t in src_local.items()}
             tgt_local: dict[int, torch.Tensor] = {}
             for pos, r in enumerate(tgt_ranks):
                 if wanted is not None and r not in wanted:
                     continue
                 shape = local_shape(spec.shape, tgt_mesh.shape, spec.target_placements, mesh_coord(tgt_mesh.shape, pos))
                 tgt_local[r] = torch.zeros(shape, dtype=tgt_dtype, device=self.device)
+                if self.local_view is not None:
+                    tgt_local[r] = self._rehome("target", tgt_local[r])
             self.source_locals.append(src_local)
             self.target_locals.append(tgt_local)
             self.globals_.append(glob if self.keep_globals else None)
@@ -161,6 +181,13 @@ class ReshardJob:
         size = self.bucket_size or 1
         self.send_buckets = {r: chunk_to_bucket_ops(cs, size) for r, cs in sorted(send_chunks.items())}
         self.recv_buckets = {r: chunk_to_bucket_ops(cs, size) for r, cs in sorted(recv_chunks.items())}
+
+    def _rehome(self, kind: str, t: torch.Tensor) -> torch.Tensor:
+        view = self.local_view(kind, t)
+        if tuple(view.shape) != tuple(t.shape) or view.dtype != t.dtype:
+            raise ValueError("local_view must keep shape and dtype")
+        view.copy_(t)
+        return view
 
     @staticmethod
     def _cell_wanted(m2m, chunk, wanted) -> bool:

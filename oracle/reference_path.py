@@ -51,13 +51,9 @@ def _peers(chunk):
     groups = getattr(chunk, "source_partial_groups", None)
     if not groups:
         return None
-    ops = {op for _, op in groups}
-    assert len(ops) == 1, "oracle: one reduce op per chunk"
-    members = {}
-    for g, _ in groups:
-        for r, t in zip(g.ranks, g.tensors):
-            members[r] = t
-    return [members[r] for r in sorted(members)], ops.pop()
+    assert len(groups) == 1, "oracle: the Partial connected component comes as one group"
+    group, op = groups[0]
+    return list(group.tensors), op
 
 
 def chunk_prepare(chunk, contiguous: bool = True) -> torch.Tensor:

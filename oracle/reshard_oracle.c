@@ -14,8 +14,10 @@
  * round trips and torch's CPU casts; gather/scatter against numpy slicing; the reduce against
  * order-sensitive closed forms; the self-copy cases against the reference's own vectors
  * (tests/test_self_copy_bucket.py:51-63).
- * Parity unpinned: NaN payloads of fp16 casts (the reference's CPU result depends on whether
- * ATen uses F16C hardware or its software routine) and NaN handling of max/min (backend-defined).
+ * Parity unpinned: the bit pattern a NaN gets in a narrowing cast (ATen's vectorised CPU cast, its
+ * scalar c10 rule and the CUDA intrinsic write 0xFFFF, 0x7FC0 and 0x7FFF for bf16; fp16 depends on
+ * F16C hardware vs software) - NaN-ness is pinned, the payload is not - and NaN handling of
+ * max/min (backend-defined).
  */
 #include <stdint.h>
 #include <string.h>
@@ -160,8 +162,6 @@ int oracle_reduce(const OracleChunk* c, void* out /* wire dtype, contiguous */, 
   if (c->tensor_dtype == OR_F64) {  /* f64 partials accumulate in f64 */
     double* acc = (double*)scratch;
     walk(c, c->peers[0], es, (char*)acc, 0);
-    char* tmp = (char*)out; /* reuse: gather each peer element-wise below */
-    (void)tmp;
     for (int p = 1; p < c->n_partials; p++) {
       int64_t idx[OR_MAX_NDIM] = {0};
       for (int64_t k = 0; k < n; k++) {

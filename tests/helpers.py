@@ -90,3 +90,40 @@ def gpu_vs_oracle(specs, device, bucket_size, target_ranks=None, merge_launches=
             if not same_obj:
                 assert_bit_equal(t, src_before[i][r], f"{spec.name} source rank {r} mutated")
     return gpu_job, cpu_job
+
+
+# ---- fixtures ------------------------------------------------------------------------------------
+def load_cases() -> dict:
+    import json
+    import os
+
+    with open(os.path.join(os.path.dirname(os.path.abspath(__file__)), "golden", "reference_cases.json")) as f:
+        return json.load(f)
+
+
+def parse_placement(code: str):
+    from torch.distributed.tensor.placement_types import Partial, Replicate, Shard, _StridedShard
+
+    if code == "R":
+        return Replicate()
+    if code.startswith("SS"):
+        dim, sf = code[2:].split("/")
+        return _StridedShard(int(dim), split_factor=int(sf))
+    if code.startswith("S"):
+        return Shard(int(code[1:]))
+    if code.startswith("P"):
+        return Partial(code[1:])
+    raise ValueError(code)
+
+
+def parse_placements(codes) -> tuple:
+    return tuple(parse_placement(c) for c in codes)
+
+
+def mesh_of(start: int, shape) -> list:
+    n = int(np.prod(shape))
+    return np.arange(start, start + n).reshape(tuple(shape)).tolist()
+
+
+DTYPES = {"fp32": torch.float32, "fp16": torch.float16, "bf16": torch.bfloat16, "float32": torch.float32,
+          "bfloat16": torch.bfloat16}

@@ -1,0 +1,102 @@
+"""The C-ABI library: loads, exports what the header declares, validates descriptors (no GPU)."""
+
+import os
+import re
+
+import numpy as np
+import pytest
+
+from etha_amd import _native as nat
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+
+
+def _header_functions():
+    text = open(os.path.join(ROOT, "include", "etha_reshard.h")).read()
+    text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
+    return sorted(set(re.findall(r"\b(etha_[a-z0-9_]+)\s*\(", text)))
+
+
+def test_every_declared_symbol_is_exported_and_bound():
+    declared = _header_functions()
+    assert len(declared) >= 15
+    lib = nat.lib()
+    for name in declared:
+        assert hasattr(lib, name), f"{name} declared in the header but not exported"
+    assert sorted(nat.exported_symbols()) == declared
+    assert lib.etha_abi_version() == nat.ABI_VERSION
+
+
+def test_struct_layouts_match_header():
+    assert nat.CHUNK_DESC.itemsize == 6 * 8 + 3 * 8 * nat.ETHA_MAX_NDIM + 6 * 4
+    assert nat.CHUNK_DESC.fields["start"][1] == 48
+    assert nat.CHUNK_DESC.fields["ndim"][1] == 48 + 3 * 64
+    info = nat.TableInfo()
+    assert info.n_chunks == 0
+
+
+def _desc(**kw):
+    d = np.zeros(1, dtype=nat.CHUNK_DESC)
+    d["tensor_ptr"], d["bucket_ptr"] = 0x10000, 0x900000
+    d["ndim"] = 2
+    d["shape"][0][:2] = [8, 16]
+    d["stride"][0][:2] = [16, 1]
+    d["tensor_dtype"] = d["wire_dtype"] = nat.F32
+    for k, v in kw.items():
+        if isinstance(v, (list, tuple)):
+            d[k][0][: len(v)] = v
+        else:
+            d[k] = v
+    return d
+
+
+def test_host_only_table_and_tile_counts():
+    t = nat.Table.create(_desc(), upload=False)
+    info = t.info()
+    assert (info.n_chunks, info.payload_bytes, info.tile_threads) == (1, 8 * 16 * 4, 256)
+    run, row = t.tiles()
+    assert len(run) == 1 and len(row) == 0  # fully contiguous: one run of 32 16-byte units
+    assert int(run[0]["n"]) == 32 and int(run[0]["a"]) == 0x10000 and int(run[0]["b"]) == 0x900000
+    with pytest.raises(nat.EthaNativeError, match="without upload"):
+        t.pack(0, 1)
+
+
+def test_validation_rejects_bad_descriptors():
+    with pytest.raises(nat.EthaNativeError, match="leaves the allowed range"):
+        nat.Table.create(_desc(tensor_lo=0x10000, tensor_hi=0x10000 + 8 * 16 * 4 - 1), upload=False)
+    with pytest.raises(nat.EthaNativeError, match="leave the bucket buffer"):
+        nat.Table.create(_desc(bucket_lo=0x900000, bucket_hi=0x900000 + 100), upload=False)
+    with pytest.raises(nat.EthaNativeError, match="ndim"):
+        nat.Table.create(_desc(ndim=9), upload=False)
+    with pytest.raises(nat.EthaNativeError, match="only implemented between floating"):
+        nat.Table.create(_desc(tensor_dtype=nat.B32, wire_dtype=nat.F32), upload=False)
+    with pytest.raises(nat.EthaNativeError, match="unknown"):
+        nat.Table.create(_desc(wire_dtype=99), upload=False)
+    with pytest.raises(nat.EthaNativeError, match="null tensor"):
+        nat.Table.create(_desc(tensor_ptr=0), upload=False)
+    with pytest.raises(nat.EthaNativeError, match="partial pointer range"):
+        nat.Table.create(_desc(n_partials=2, partial_first=0), upload=False)
+    with pytest.raises(nat.EthaNativeError, match="not aligned"):
+        nat.Table.create(_desc(tensor_ptr=0x10002, wire_dtype=nat.BF16), upload=False)
+    ok = nat.Table.create(_desc(tensor_lo=0x10000, tensor_hi=0x10000 + 8 * 16 * 4), upload=False)
+    with pytest.raises(nat.EthaNativeError, match="exceeds table"):
+        ok.pack(0, 2)
+
+
+def test_empty_and_zero_sized():
+    t = nat.Table.create(np.zeros(0, dtype=nat.CHUNK_DESC), upload=False)
+    assert t.info().n_chunks == 0
+    t = nat.Table.create(_desc(shape=[0, 16]), upload=False)
+    assert t.info().n_run_tiles + t.info().n_row_tiles == 0
+
+
+def test_executor_refuses_cpu_tensors():
+    import torch
+    from torch.distributed.tensor.placement_types import Shard
+
+    from etha_amd.world import ReshardJob, TensorSpec
+
+    job = ReshardJob([TensorSpec("w", (8, 8), [0, 1], (Shard(0),), [2, 3], (Shard(1),), torch.float32)],
+                     device="cpu", bucket_size=None)
+    with pytest.raises(RuntimeError, match="no CPU path"):
+        job.run()

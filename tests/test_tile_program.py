@@ -1,0 +1,182 @@
+"""The host-side tile compiler, executed on the CPU and compared with the C oracle (no GPU)."""
+
+import numpy as np
+import pytest
+
+from etha_amd import _native as nat
+from oracle import c_oracle as co
+
+from tile_interpreter import HostArena, execute
+
+ES = {nat.F16: 2, nat.BF16: 2, nat.F32: 4, nat.F64: 8, nat.B8: 1, nat.B16: 2, nat.B32: 4, nat.B64: 8}
+rs = np.random.RandomState(7)
+
+
+def _mk_desc(tensor_addr, lo, hi, bucket_addr, blo, bhi, start, shape, stride, tdt, wdt):
+    d = np.zeros((), dtype=nat.CHUNK_DESC)
+    d["tensor_ptr"], d["tensor_lo"], d["tensor_hi"] = tensor_addr, lo, hi
+    d["bucket_ptr"], d["bucket_lo"], d["bucket_hi"] = bucket_addr, blo, bhi
+    nd = len(shape)
+    d["ndim"] = nd
+    d["start"][:nd], d["shape"][:nd], d["stride"][:nd] = start, shape, stride
+    d["tensor_dtype"], d["wire_dtype"] = tdt, wdt
+    return d
+
+
+def _oracle_chunk(tensor_addr, start, shape, stride, tdt, wdt, off):
+    return co.make_chunk(tensor_addr, start, shape, stride, tdt, wdt, bucket_off=off)
+
+
+# (parent shape, permutation, slice start, chunk shape, tensor dtype, wire dtype, address skew)
+GEOMETRIES = [
+    ((512, 1024), None, (0, 256), (512, 256), nat.F32, nat.F32, 0),      # 1 KiB rows of a 4 KiB pitch
+    ((64, 4096), None, (0, 2048), (64, 2048), nat.BF16, nat.BF16, 0),    # 4 KiB rows: run tiles per row
+    ((16, 14336), None, (0, 7168), (16, 7168), nat.BF16, nat.BF16, 0),   # 14 KiB rows: ragged row tiles
+    ((1024, 64), None, (0, 16), (1024, 16), nat.BF16, nat.BF16, 0),      # 32-byte rows
+    ((33, 50), None, (1, 3), (31, 45), nat.BF16, nat.BF16, 0),           # odd sizes: 2-byte units
+    ((33, 50), None, (1, 3), (31, 45), nat.B8, nat.B8, 3),               # byte elements at an odd address
+    ((20, 30, 40), None, (2, 5, 8), (7, 11, 24), nat.F32, nat.F32, 0),   # 3-D, nothing merges
+    ((20, 30, 40), (2, 0, 1), (8, 2, 5), (24, 7, 11), nat.F32, nat.F32, 0),  # permuted parent: strided elements
+    ((8, 16, 64), None, (0, 0, 0), (8, 8, 64), nat.B64, nat.B64, 0),     # "slice view": half of dim 1
+    ((4096,), None, (1024,), (2048,), nat.F32, nat.BF16, 0),             # fp32 -> bf16, vectorised
+    ((77, 33), None, (3, 1), (70, 31), nat.F32, nat.BF16, 0),            # fp32 -> bf16, element-wise
+    ((64, 256), None, (0, 0), (64, 256), nat.BF16, nat.F32, 0),          # widening wire
+    ((64, 256), None, (0, 128), (64, 128), nat.F64, nat.F16, 0),
+    ((64, 256), None, (0, 128), (64, 128), nat.F16, nat.BF16, 0),
+    ((3,), None, (0,), (3,), nat.F32, nat.F32, 0),
+    ((5, 0, 7), None, (0, 0, 0), (5, 0, 7), nat.F32, nat.F32, 0),        # empty chunk
+]
+
+
+@pytest.mark.parametrize("geom", GEOMETRIES, ids=lambda g: f"{g[0]}p{g[1]}s{g[2]}c{g[3]}t{g[4]}w{g[5]}k{g[6]}")
+def test_pack_and_unpack_tiles_match_oracle(geom):
+    pshape, perm, start, cshape, tdt, wdt, skew = geom
+    es, ws = ES[tdt], ES[wdt]
+    pn = int(np.prod(pshape))
+    cn = int(np.prod(cshape))
+    arena = HostArena(2 * pn * es + 4 * cn * max(es, ws) + 8192)
+    t_addr = arena.alloc(pn * es, skew=skew)
+    t2_addr = arena.alloc(pn * es, skew=skew)
+    bucket_pad = 48  # the chunk does not start at the bucket's first byte
+    b_addr = arena.alloc(cn * ws + 2 * bucket_pad)
+    # element strides of the (possibly permuted) parent view
+    strides = np.array([int(np.prod(pshape[i + 1:])) for i in range(len(pshape))], dtype=np.int64)
+    if perm is not None:
+        strides = strides[list(perm)]
+    if tdt in (nat.F16, nat.BF16, nat.F32, nat.F64) and tdt != wdt:
+        vals = (rs.randn(pn) * 3).astype(np.float64)
+        raw = co.cast(vals.view(np.uint64), co.F64, tdt, {2: np.uint16, 4: np.uint32, 8: np.uint64}[es])
+        arena.bytes_at(t_addr, pn * es)[:] = raw.view(np.uint8)
+    else:
+        arena.bytes_at(t_addr, pn * es)[:] = rs.randint(0, 256, pn * es)
+    before_t2 = arena.bytes_at(t2_addr, pn * es).copy()
+    off = bucket_pad - (bucket_pad % ws)
+    desc = _mk_desc(t_addr, t_addr, t_addr + pn * es, b_addr + off, b_addr, b_addr + cn * ws + 2 * bucket_pad,
+                    start, cshape, strides, tdt, wdt)
+    table = nat.Table.create(desc.reshape(1), upload=False)
+    assert table.info().payload_bytes == cn * ws
+    # ---- pack
+    src_before = arena.bytes_at(t_addr, pn * es).copy()
+    bucket_before = arena.bytes_at(b_addr, cn * ws + 2 * bucket_pad).copy()
+    execute(table, arena, "pack")
+    want_bucket = bucket_before.copy()
+    scratch = np.zeros(max(cn * es, 8), dtype=np.uint8)
+    oc = _oracle_chunk(t_addr, start, cshape, strides, tdt, wdt, off)
+    assert co.lib().oracle_pack_bucket(oc, 1, want_bucket.ctypes.data, scratch.ctypes.data) == 0
+    assert np.array_equal(arena.bytes_at(b_addr, cn * ws + 2 * bucket_pad), want_bucket)
+    assert np.array_equal(arena.bytes_at(t_addr, pn * es), src_before), "pack wrote the source tensor"
+    w = arena.writes
+    assert w.max(initial=0) <= 1 and int(w.sum()) == cn * ws, "every bucket byte exactly once"
+    # ---- unpack into a second tensor of the same geometry
+    arena.writes[:] = 0
+    desc2 = _mk_desc(t2_addr, t2_addr, t2_addr + pn * es, b_addr + off, b_addr, b_addr + cn * ws + 2 * bucket_pad,
+                     start, cshape, strides, tdt, wdt)
+    table2 = nat.Table.create(desc2.reshape(1), upload=False)
+    execute(table2, arena, "unpack")
+    want_t2 = before_t2.copy()
+    oc2 = _oracle_chunk(want_t2.ctypes.data, start, cshape, strides, tdt, wdt, off)
+    assert co.lib().oracle_unpack_bucket(oc2, 1, want_bucket.ctypes.data, scratch.ctypes.data) == 0
+    assert np.array_equal(arena.bytes_at(t2_addr, pn * es), want_t2), "unpack result / untouched bytes differ"
+    assert arena.writes.max(initial=0) <= 1 and int(arena.writes.sum()) == cn * es
+
+
+def test_bucket_ranges_and_many_chunks():
+    """Chunk ranges select exactly their own tiles; un-padded prefix-sum offsets inside one bucket."""
+    shapes = [(40, 24), (7, 5), (128,), (3, 9, 11), (256, 8)]
+    es = 2
+    total = sum(int(np.prod(s)) for s in shapes) * es
+    arena = HostArena(4 * total + 65536)
+    b_addr = arena.alloc(total)
+    descs, ocs, off = [], [], 0
+    tensors = []
+    for s in shapes:
+        n = int(np.prod(s))
+        t = arena.alloc(n * es)
+        arena.bytes_at(t, n * es)[:] = rs.randint(0, 256, n * es)
+        strides = [int(np.prod(s[i + 1:])) for i in range(len(s))]
+        descs.append(_mk_desc(t, t, t + n * es, b_addr + off, b_addr, b_addr + total, [0] * len(s), s, strides,
+                              nat.BF16, nat.BF16))
+        ocs.append((t, s, strides, off))
+        tensors.append((t, n))
+        off += n * es
+    table = nat.Table.create(np.stack(descs), upload=False)
+    run_begin, row_begin = table.ranges()
+    assert len(run_begin) == len(shapes) + 1
+    for first, count in ((0, 5), (1, 2), (4, 1), (2, 0)):
+        arena.bytes_at(b_addr, total)[:] = 0xEE
+        arena.writes[:] = 0
+        execute(table, arena, "pack", first, count)
+        want = np.full(total, 0xEE, dtype=np.uint8)
+        scratch = np.zeros(total, dtype=np.uint8)
+        for t, s, strides, o in ocs[first : first + count]:
+            oc = _oracle_chunk(t, [0] * len(s), s, strides, co.BF16, co.BF16, o)
+            assert co.lib().oracle_pack_bucket(oc, 1, want.ctypes.data, scratch.ctypes.data) == 0
+        assert np.array_equal(arena.bytes_at(b_addr, total), want)
+
+
+@pytest.mark.parametrize("op", ["sum", "avg", "max", "min", "product"])
+@pytest.mark.parametrize("tdt,wdt", [(nat.BF16, nat.BF16), (nat.F32, nat.BF16), (nat.F16, nat.F16), (nat.F64, nat.F32)])
+def test_reduce_tiles_match_oracle(op, tdt, wdt):
+    pshape, start, cshape = (24, 96), (4, 32), (16, 64)
+    es, ws = ES[tdt], ES[wdt]
+    pn, cn = int(np.prod(pshape)), int(np.prod(cshape))
+    n_peers = 5
+    arena = HostArena(n_peers * pn * es + 2 * cn * ws + 16384)
+    peers = []
+    for p in range(n_peers):
+        addr = arena.alloc(pn * es)
+        vals = (rs.randn(pn) * (1.0 if op != "product" else 0.9) + (0.0 if op != "product" else 1.0)).astype(np.float64)
+        raw = co.cast(vals.view(np.uint64), co.F64, tdt, {2: np.uint16, 4: np.uint32, 8: np.uint64}[es])
+        arena.bytes_at(addr, pn * es)[:] = raw.view(np.uint8)
+        peers.append(addr)
+    b_addr = arena.alloc(cn * ws)
+    strides = [pshape[1], 1]
+    d = _mk_desc(0, 0, 0, b_addr, b_addr, b_addr + cn * ws, start, cshape, strides, tdt, wdt)
+    d["n_partials"], d["partial_first"], d["reduce_op"] = n_peers, 0, nat.REDUCE_OPS[op]
+    ptrs = np.asarray(peers, dtype=np.uint64)
+    table = nat.Table.create(d.reshape(1), ptrs, upload=False)
+    run, row = table.tiles()
+    assert len(run) == 0 and len(row) > 0 and np.all(row["n_peers"] == n_peers)
+    peer_bytes = [arena.bytes_at(p, pn * es).copy() for p in peers]
+    execute(table, arena, "pack", peers=ptrs)
+    want = np.zeros(cn * ws, dtype=np.uint8)
+    scratch = np.zeros(cn * 8, dtype=np.uint8)
+    oc = co.make_chunk(0, start, cshape, strides, tdt, wdt, peers=peers, op=op)
+    assert co.lib().oracle_pack_bucket(oc, 1, want.ctypes.data, scratch.ctypes.data) == 0
+    assert np.array_equal(arena.bytes_at(b_addr, cn * ws), want)
+    for p, before in zip(peers, peer_bytes):
+        assert np.array_equal(arena.bytes_at(p, pn * es), before), "a partial was written"
+
+
+def test_selfcopy_tiles():
+    n = 64
+    arena = HostArena(n * 4 * 4 + 8192)
+    t = arena.alloc(n * 4)
+    vals = np.arange(n, dtype=np.float32)
+    arena.bytes_at(t, n * 4)[:] = vals.view(np.uint8)
+    src = _mk_desc(t, t, t + n * 4, 0, 0, 0, (0,), (16,), (1,), nat.F32, nat.F32)
+    dst = _mk_desc(t, t, t + n * 4, 0, 0, 0, (32,), (16,), (1,), nat.F32, nat.F32)
+    table = nat.Table.create_selfcopy(src.reshape(1), dst.reshape(1), upload=False)
+    execute(table, arena, "selfcopy")
+    got = arena.bytes_at(t, n * 4).view(np.float32)
+    assert np.array_equal(got[32:48], vals[:16]) and np.array_equal(got[:32], vals[:32]) and np.array_equal(got[48:], vals[48:])

@@ -1,0 +1,141 @@
+"""A CPU interpreter of the compiled tile program (test infrastructure).
+
+Descriptor addresses are plain integers, so a table can be compiled against *host* buffers and its
+tiles executed here with numpy, doing exactly what the kernels do per work-item.  That checks the
+host-side tile compiler (addresses, alignment classes, row walking, tails) with full bounds and
+coverage checking and no GPU.
+"""
+
+from __future__ import annotations
+
+import ctypes
+
+import numpy as np
+
+from oracle import c_oracle as co
+
+THREADS = 256
+_CODE_RAW = {0: np.uint16, 1: np.uint16, 2: np.uint32, 3: np.uint64}
+
+
+class HostArena:
+    """One host allocation holding every buffer, so that addresses map to offsets."""
+
+    def __init__(self, nbytes: int, fill: int = 0xA5):
+        self.buf = np.full(nbytes + 256, fill, dtype=np.uint8)
+        base = self.buf.ctypes.data
+        self.pad = (-base) % 256
+        self.base = base + self.pad
+        self.nbytes = nbytes
+        self.cursor = 0
+        self.writes = np.zeros(nbytes, dtype=np.uint16)
+
+    def alloc(self, nbytes: int, align: int = 256, skew: int = 0) -> int:
+        self.cursor = -(-self.cursor // align) * align + skew
+        addr = self.base + self.cursor
+        self.cursor += nbytes
+        assert self.cursor <= self.nbytes
+        return addr
+
+    def bytes_at(self, addr: int, n: int) -> np.ndarray:
+        off = addr - self.base
+        assert 0 <= off and off + n <= self.nbytes, "address outside the arena"
+        return self.buf[self.pad + off : self.pad + off + n]
+
+    def offsets(self, addrs: np.ndarray, width: int) -> np.ndarray:
+        off = addrs.astype(np.int64) - self.base
+        assert off.min() >= 0 and off.max() + width <= self.nbytes, "tile touches memory outside the arena"
+        return off
+
+
+def _unit_positions(run_tiles, row_tiles):
+    """Per active work-item: (a address, b address, meta, tile kind, row-tile index)."""
+    out = []
+    if len(run_tiles):
+        n = run_tiles["n"].astype(np.int64)
+        tid = np.concatenate([np.arange(k) for k in n]) if n.sum() else np.zeros(0, np.int64)
+        rep = np.repeat(np.arange(len(run_tiles)), n)
+        meta = run_tiles["meta"][rep]
+        a = run_tiles["a"][rep].astype(np.int64) + (tid << (meta & 15))
+        b = run_tiles["b"][rep].astype(np.int64) + (tid << ((meta >> 4) & 15))
+        out.append((a, b, meta, np.full(len(a), -1)))
+    if len(row_tiles):
+        n = row_tiles["n"].astype(np.int64)
+        tid = np.concatenate([np.arange(k) for k in n]) if n.sum() else np.zeros(0, np.int64)
+        rep = np.repeat(np.arange(len(row_tiles)), n)
+        t = row_tiles[rep]
+        meta = t["meta"]
+        run = t["run"].astype(np.int64)
+        q = t["c0"].astype(np.int64) + tid
+        assert np.all(t["c0"] < t["run"])
+        big = run >= THREADS
+        r = np.where(big, (q >= run).astype(np.int64), q // run)
+        c = q - r * run
+        assert np.all(c < run) and np.all(c >= 0)
+        a = t["a"].astype(np.int64) + r * t["a_pitch"] + (c << (meta & 15))
+        b = t["b"].astype(np.int64) + r * t["b_pitch"] + (c << ((meta >> 4) & 15))
+        out.append((a, b, meta, rep))
+    return out
+
+
+def execute(table, arena: HostArena, direction: str, first: int = 0, count: int | None = None,
+            peers: np.ndarray | None = None) -> None:
+    """Run chunks [first, first+count) of a table on the host. direction: 'pack' | 'unpack' | 'selfcopy'."""
+    run_tiles, row_tiles = table.tiles()
+    run_begin, row_begin = table.ranges()
+    if count is None:
+        count = len(run_begin) - 1 - first
+    run_tiles = run_tiles[run_begin[first] : run_begin[first + count]]
+    row_tiles = row_tiles[row_begin[first] : row_begin[first + count]]
+    assert np.all(run_tiles["n"] <= THREADS) and np.all(row_tiles["n"] <= THREADS)
+    assert np.all(run_tiles["n"] > 0) and np.all(row_tiles["n"] > 0)
+    rev = direction == "unpack"
+    mem = arena.buf[arena.pad : arena.pad + arena.nbytes]
+    for a, b, meta, row_idx in _unit_positions(run_tiles, row_tiles):
+        for m in np.unique(meta):
+            sel = meta == m
+            ua, ub = 1 << (int(m) & 15), 1 << ((int(m) >> 4) & 15)
+            dta, dtb = (int(m) >> 8) & 15, (int(m) >> 12) & 15
+            cvt, vec = bool(int(m) & (1 << 16)), bool(int(m) & (1 << 17))
+            assert np.all(a[sel] % ua == 0) and np.all(b[sel] % ub == 0), "misaligned vector access"
+            reduce = row_idx[sel][0] >= 0 and int(row_tiles["n_peers"][row_idx[sel][0]]) > 0
+            if reduce:
+                _reduce_units(arena, mem, row_tiles, row_idx[sel], a[sel], b[sel], ua, ub, dta, dtb, peers)
+                continue
+            src, dst, us, ud, ds_, dd = (b[sel], a[sel], ub, ua, dtb, dta) if rev else (a[sel], b[sel], ua, ub, dta, dtb)
+            so = arena.offsets(src, us)[:, None] + np.arange(us)
+            do = arena.offsets(dst, ud)[:, None] + np.arange(ud)
+            data = mem[so]
+            if cvt:
+                assert vec == (max(us, ud) == 16) or not vec
+                raw_s, raw_d = _CODE_RAW[ds_], _CODE_RAW[dd]
+                elems = np.ascontiguousarray(data).view(raw_s)
+                data = co.cast(elems, ds_, dd, raw_d).view(np.uint8).reshape(len(so), ud)
+            else:
+                assert us == ud
+            np.add.at(arena.writes, do.reshape(-1), 1)
+            mem[do] = data
+
+
+def _reduce_units(arena, mem, row_tiles, row_idx, a_off, b, ua, ub, dta, dtb, peers):
+    es = {0: 2, 1: 2, 2: 4, 3: 8}[dta]
+    n_el = ua // es
+    for ti in np.unique(row_idx):
+        sel = row_idx == ti
+        t = row_tiles[ti]
+        bases = peers[int(t["peer_first"]) : int(t["peer_first"]) + int(t["n_peers"])].astype(np.int64)
+        op = {0: "sum", 1: "avg", 2: "max", 3: "min", 4: "product"}[int(t["reduce_op"])]
+        offs = a_off[sel]
+        n_units = len(offs)
+        out = np.zeros(n_units * n_el, dtype=_CODE_RAW[dtb])
+        scratch = np.zeros(n_units * n_el, dtype=np.float64)
+        # gather each peer's units into a contiguous staging array, then let the C oracle combine them
+        staged = []
+        for base in bases:
+            so = arena.offsets(base + offs, ua)[:, None] + np.arange(ua)
+            staged.append(np.ascontiguousarray(mem[so]).reshape(-1).copy())
+        ch = co.make_chunk(0, (0,), (n_units * n_el,), (1,), dta, dtb, peers=[s.ctypes.data for s in staged], op=op)
+        assert co.lib().oracle_reduce(ch, out.ctypes.data, scratch.ctypes.data) == 0
+        do = arena.offsets(b[sel], ub)[:, None] + np.arange(ub)
+        np.add.at(arena.writes, do.reshape(-1), 1)
+        mem[do] = out.view(np.uint8).reshape(n_units, ub)
