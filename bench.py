@@ -20,6 +20,14 @@ sys.path.insert(0, ROOT)
 
 HBM_PEAK_GBS = 8000.0  # MI355X HBM3E, published
 
+# HBM bytes per launch of the dominant kernel, from two rocprofv3 --pmc runs (FETCH_SIZE, WRITE_SIZE), each
+# scaled by what the counter reads for a plain 1 GiB copy; the summary of those runs is
+# profiles/etha_tile_kernel_llama3_8b_fsdp8_to_tp2.txt.  Keyed by (workload, kernel, launch granularity).
+MEASURED_TRAFFIC_BYTES = {
+    ("llama3_8b_fsdp8_to_tp2", "etha_tile_kernel<false>", "run of buckets"): 2045192678,
+    ("llama3_8b_fsdp8_to_tp2", "etha_tile_kernel<true>", "run of buckets"): 16376158395,
+}
+
 
 def parse_args():
     ap = argparse.ArgumentParser()
@@ -30,6 +38,9 @@ def parse_args():
     ap.add_argument("--per-bucket", action="store_true", help="one launch per bucket instead of one per run of buckets")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--cpu-layers", type=int, default=2, help="layers of the workload the CPU baseline sample covers")
+    ap.add_argument("--calibration-copy", action="store_true",
+                    help="after the timed region run three plain 1 GiB torch copies (known traffic, for scaling "
+                         "hardware counters collected with rocprofv3 --pmc)")
     return ap.parse_args()
 
 
@@ -207,13 +218,21 @@ def main():
             "peak": HBM_PEAK_GBS,
             "unit": "GB/s",
             "frac": round(achieved / HBM_PEAK_GBS, 4),
-            "traffic": None,
+            "traffic": MEASURED_TRAFFIC_BYTES.get(
+                (args.workload, kernel_name, "run of buckets" if merge else "bucket")),
             "bytes_per_launch": dom_bytes // dom_launches,
             "avg_launch_ms": round(dom_ms / dom_launches, 5),
             "launches_per_step": dom_launches,
         },
         "setup_s": round(setup_s, 1),
     }
+    if args.calibration_copy:
+        a = torch.empty(1 << 30, dtype=torch.uint8, device=dev).fill_(1)
+        b = torch.empty(1 << 30, dtype=torch.uint8, device=dev)
+        for _ in range(3):
+            b.copy_(a)
+        torch.cuda.synchronize()
+        out["calibration_copy"] = {"bytes_read": 1 << 30, "bytes_written": 1 << 30, "launches": 3}
     if not args.no_cpu_baseline:
         out["cpu_baseline"] = cpu_baseline(args.workload, args.cpu_layers)
     print(json.dumps(out))
