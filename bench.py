@@ -154,7 +154,18 @@ def main():
                     n *= d
                 unpack_write += n * c.tensor.element_size()
     unpack_read = sum(table_bytes(p, "recv_table") for p in recv_plans)
-    pack_bytes = pack_read + wire_bytes
+    # LOCAL chunks run inside the send phase as direct copies: read the source region, write the target
+    self_bytes = 0
+    for p in send_plans:
+        for b in p.buckets:
+            if b.transport.value == "local":
+                for c in b.chunks:
+                    n = 1
+                    for d in c.chunk_shape:
+                        n *= d
+                    src_t = c.src_tensor if c.src_tensor is not None else c.tensor
+                    self_bytes += n * (src_t.element_size() + c.tensor.element_size())
+    pack_bytes = pack_read + wire_bytes + self_bytes
     unpack_bytes = unpack_read + unpack_write
 
     stream = torch.cuda.current_stream(dev)
@@ -210,7 +221,7 @@ def main():
         "pct_of_hbm_peak": round(100.0 * (pack_bytes + unpack_bytes) / (dev_ms * 1e-3) / 1e9 / HBM_PEAK_GBS, 2),
         "pack": {"GB/s": round(pack_gbs, 1), "ms": round(pack_avg, 4), "bytes": pack_bytes, "launches": n_pack},
         "unpack": {"GB/s": round(unpack_gbs, 1), "ms": round(unpack_avg, 4), "bytes": unpack_bytes, "launches": n_unpack},
-        "selfcopy_launches": n_self,
+        "selfcopy": {"launches": n_self, "bytes": self_bytes, "note": "timed inside the pack phase"},
         "roofline": {
             "bound": "hbm",
             "kernel": kernel_name,

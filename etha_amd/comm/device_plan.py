@@ -41,7 +41,7 @@ def check_cast(src: torch.dtype, dst: torch.dtype) -> None:
         raise NotImplementedError(f"conversion {src} -> {dst} is only implemented between floating dtypes")
 
 
-def _storage_range(t: torch.Tensor) -> tuple[int, int]:
+def _storage_range(t) -> tuple[int, int]:
     st = t.untyped_storage()
     lo = st.data_ptr()
     return lo, lo + st.nbytes()
@@ -167,14 +167,27 @@ class SelfCopyBuilder:
         return nat.Table.create_selfcopy(np.stack(self.src), np.stack(self.dst), upload=True)
 
 
-def region_hull(tensor: torch.Tensor, slices: tuple) -> tuple[int, int]:
-    """Smallest byte interval covering ``tensor[slices]`` (empty regions give lo == hi)."""
-    view = tensor[slices] if slices else tensor
-    if view.numel() == 0:
-        return view.data_ptr(), view.data_ptr()
-    span = sum((n - 1) * s for n, s in zip(view.shape, view.stride()))
-    lo = view.data_ptr()
-    return lo, lo + (span + 1) * view.element_size()
+def region_hull(tensor, slices: tuple) -> tuple[int, int]:
+    """Smallest byte interval covering ``tensor[slices]`` (empty regions give lo == hi).
+
+    Pure arithmetic on shape/stride/data_ptr, so it also works for tensors that only exist as an
+    IPC-mapped pointer.
+    """
+    shape, stride, es = tuple(tensor.shape), tuple(tensor.stride()), tensor.element_size()
+    lo_el, span_el, empty = 0, 0, False
+    for d, n in enumerate(shape):
+        start, stop = 0, n
+        if d < len(slices):
+            start, stop, _ = slices[d].indices(n)
+        ext = max(stop - start, 0)
+        if ext == 0:
+            empty = True
+        lo_el += start * stride[d]
+        span_el += (ext - 1) * stride[d] if ext > 0 else 0
+    lo = tensor.data_ptr() + lo_el * es
+    if empty:
+        return lo, lo
+    return lo, lo + (span_el + 1) * es
 
 
 def local_bucket_needs_staging(bucket: Bucket) -> bool:

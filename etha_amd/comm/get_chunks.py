@@ -18,6 +18,9 @@ Deliberate differences:
   chunk keeps only the remote destinations and disappears when none is left.  The LOCAL chunk
   reads ``source_tensor`` (``Chunk.src_tensor``) and writes ``target_tensor``.
 * broadcast sub-groups need no pre-creation (``get_chunks.py:48-55``): there is no process group.
+* A role whose tensor is not given produces no chunks: without ``source_tensor`` the rank does not act
+  as a source, without ``target_tensor`` not as a destination (the reference would build chunks around
+  ``None`` and fail in ``Chunk.__post_init__``, ``ir.py:87-89``).
 """
 
 from __future__ import annotations
@@ -94,9 +97,8 @@ def m2m_to_chunks(
         src_rank, src_idx = route.src.rank, route.src.cell
         all_dsts = tuple(sorted({d.rank for d in route.dsts}))
         src_slices: tuple[slice, ...] = ()
-        if src_rank == rank:
-            if src_tuples is not None:
-                src_slices = get_slice_from_multi_index(src_idx, src_ext, src_tuples)
+        if src_rank == rank and source_tensor is not None:
+            src_slices = get_slice_from_multi_index(src_idx, src_ext, src_tuples)
             remote = tuple(r for r in all_dsts if r != rank)
             if remote or route.kind == Transport.NONE:
                 kind = route.kind
@@ -119,12 +121,14 @@ def m2m_to_chunks(
                     )
                 )
         for dst in route.dsts:
-            if dst.rank != rank:
+            if dst.rank != rank or target_tensor is None:
                 continue
-            dst_slices: tuple[slice, ...] = ()
-            if tgt_tuples is not None:
-                dst_slices = get_slice_from_multi_index(dst.cell, tgt_ext, tgt_tuples)
+            dst_slices = get_slice_from_multi_index(dst.cell, tgt_ext, tgt_tuples)
             if src_rank == rank:
+                if source_tensor is None:
+                    raise ValueError(
+                        f"rank {rank} is both source and destination of cell {src_idx}: pass source_tensor too"
+                    )
                 if source_partial_groups:
                     raise NotImplementedError("same-rank delivery of a Partial source is not supported")
                 chunks.append(

@@ -15,6 +15,7 @@
 
 #include <cstdarg>
 #include <cstdio>
+#include <array>
 #include <cstring>
 #include <map>
 #include <mutex>
@@ -361,8 +362,18 @@ __global__ __launch_bounds__(256) void etha_reduce_kernel(const RowTile* __restr
 // Host side: validation and the tile compiler.
 // =================================================================================================
 thread_local std::string g_err;
+// An allocation may be opened once per process; several tensors usually share one allocation, so
+// mappings are cached per handle and reference-counted.
+struct IpcMapping {
+  void* base = nullptr;
+  int refs = 0;
+};
+typedef std::array<uint8_t, 64> IpcKey;
 std::mutex g_ipc_mutex;
-std::map<void*, void*> g_ipc_bases;  // pointer handed out by etha_ipc_open -> mapping base
+std::map<IpcKey, IpcMapping> g_ipc_open;
+std::map<void*, IpcKey> g_ipc_ptrs;  // pointer handed out by etha_ipc_open -> its handle (multimap not needed:
+                                     // equal pointers come from equal handles and share the count)
+std::map<void*, int> g_ipc_ptr_refs;
 
 int fail(int code, const char* fmt, ...) {
   char buf[512];
@@ -914,27 +925,45 @@ int etha_ipc_open(const EthaIpcHandle* handle, void** out_ptr) {
   if (handle->size >= (2ull << 30))
     return fail(ETHA_ERR_UNSUPPORTED, "IPC allocation of %llu bytes: keep shared allocations under 2 GiB",
                 (unsigned long long)handle->size);
-  hipIpcMemHandle_t h;
-  memcpy(&h, handle->handle, 64);
-  void* base = nullptr;
-  HIP_TRY(hipIpcOpenMemHandle(&base, h, hipIpcMemLazyEnablePeerAccess));
-  *out_ptr = (char*)base + handle->offset;
+  IpcKey key;
+  memcpy(key.data(), handle->handle, 64);
   std::lock_guard<std::mutex> lock(g_ipc_mutex);
-  g_ipc_bases[*out_ptr] = base;
+  IpcMapping& m = g_ipc_open[key];
+  if (m.refs == 0) {
+    hipIpcMemHandle_t h;
+    memcpy(&h, handle->handle, 64);
+    void* base = nullptr;
+    hipError_t e = hipIpcOpenMemHandle(&base, h, hipIpcMemLazyEnablePeerAccess);
+    if (e != hipSuccess) {
+      g_ipc_open.erase(key);
+      return fail(ETHA_ERR_HIP, "hipIpcOpenMemHandle: %s", hipGetErrorString(e));
+    }
+    m.base = base;
+  }
+  m.refs++;
+  void* p = (char*)m.base + handle->offset;
+  g_ipc_ptrs[p] = key;
+  g_ipc_ptr_refs[p]++;
+  *out_ptr = p;
   return ETHA_OK;
 }
 
 int etha_ipc_close(void* opened_ptr) {
   if (!opened_ptr) return ETHA_OK;
-  void* base = nullptr;
-  {
-    std::lock_guard<std::mutex> lock(g_ipc_mutex);
-    auto it = g_ipc_bases.find(opened_ptr);
-    if (it == g_ipc_bases.end()) return fail(ETHA_ERR_INVALID, "pointer was not returned by etha_ipc_open");
-    base = it->second;
-    g_ipc_bases.erase(it);
+  std::lock_guard<std::mutex> lock(g_ipc_mutex);
+  auto it = g_ipc_ptrs.find(opened_ptr);
+  if (it == g_ipc_ptrs.end()) return fail(ETHA_ERR_INVALID, "pointer was not returned by etha_ipc_open");
+  const IpcKey key = it->second;
+  if (--g_ipc_ptr_refs[opened_ptr] == 0) {
+    g_ipc_ptr_refs.erase(opened_ptr);
+    g_ipc_ptrs.erase(it);
   }
-  HIP_TRY(hipIpcCloseMemHandle(base));
+  IpcMapping& m = g_ipc_open[key];
+  if (--m.refs == 0) {
+    void* base = m.base;
+    g_ipc_open.erase(key);
+    HIP_TRY(hipIpcCloseMemHandle(base));
+  }
   return ETHA_OK;
 }
 

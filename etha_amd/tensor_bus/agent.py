@@ -1,0 +1,412 @@
+"""The agent side of the tensor bus, as one hub process for all ranks of one GPU.
+
+In the reference every rank runs its own ``TensorBusAgent`` process inside a torchrun world and the
+agents rendezvous through a KV store and NCCL (``src/etha/tensor_bus/agent.py``).  That control plane
+is outside this build.  What the hot path needs from it is kept, in one process that plays every
+agent rank of the GPU:
+
+* one command queue and one state/heartbeat file per agent rank (``bootstrap.py:105-106`` naming);
+* ``InitPair``: a pair matches when ``expected_world_size`` ranks of both sides have registered;
+  meshes are rebuilt as ``arange`` from each side's first rank and the M2M map is planned in both
+  directions, skipping a direction whose target is Partial (``agent.py:203-436``);
+* ``RegisterTensors``: tensors arrive as hipIPC handles; when every rank of the batch has
+  registered, chunks and buckets are planned per rank with the transfer-dtype rule
+  (``agent.py:543-687``) and compiled into device tile programs;
+* ``Transfer``: runs that rank's send or recv buckets through the HIP path (``agent.py:438-507``).
+  The reference brackets a transfer with barriers over both sides; here a send waits until its
+  previous generation has been consumed and a recv waits for its sources' sends, which gives the
+  same lock step;
+* ``QueryStatus`` (``transfer_signal``) and ``CleanupBatch``.
+
+A failing command is reported back to the worker as an exception of the same type; the reference
+logs it, releases the semaphore and lets the agent die (``agent.py:196-201``).
+"""
+
+from __future__ import annotations
+
+import json
+import logging
+import os
+import queue
+import threading
+import time
+from dataclasses import dataclass, field
+
+import numpy as np
+import torch
+from torch.distributed.tensor.placement_types import Partial
+
+from ..comm import LoopbackWire, bucket_comm, chunk_to_bucket_ops, get_m2m_map, m2m_to_chunks
+from ..comm.transfer import Transport
+from ..world import create_partial_groups, transfer_dtype_rule
+from .command_queue import CommandQueue
+from .commands import CleanupBatch, InitPair, QueryStatus, RegisterTensors, Transfer
+from .ipc_tensor import IpcTensor, import_tensor
+
+logger = logging.getLogger(__name__)
+
+
+def default_path_naming(rank: int) -> tuple[str, str]:
+    return f"/tmp/agent_rank{rank}_command.lmdb", f"/tmp/agent_rank{rank}_state.lmdb"
+
+
+@dataclass
+class PairState:
+    pair_name: str
+    sides: dict = field(default_factory=dict)  # name -> {"expected": n, "ranks": {rank: (mesh_shape, placements)}}
+    matched: bool = False
+    ranks: dict = field(default_factory=dict)  # name -> sorted ranks
+    meshes: dict = field(default_factory=dict)  # name -> (mesh ndarray, placements)
+    m2m: dict = field(default_factory=dict)  # (source name, target name) -> M2MMap | None
+
+
+@dataclass
+class BatchState:
+    batch_id: str
+    pair_names: list[str]
+    bucket_size: int | None
+    registrations: dict = field(default_factory=dict)  # rank -> [(pair_name, tensor)]
+    planned: bool = False
+    send_buckets: dict = field(default_factory=dict)
+    recv_buckets: dict = field(default_factory=dict)
+    send_count: dict = field(default_factory=dict)
+    recv_count: dict = field(default_factory=dict)
+    owed: dict = field(default_factory=dict)  # destination rank -> number of receives its sources have asked of it
+    transfer_signal: bool = False
+
+
+@dataclass
+class _Entry:
+    rank: int
+    conn: object
+    command: object
+    started: bool = False
+
+
+class TensorBusAgent:
+    """Hub agent: serves ``world_size`` agent ranks on one device."""
+
+    def __init__(self, world_size: int, path_naming_fn=None, device: str | torch.device = "cuda:0",
+                 heartbeat_interval: float = 0.2):
+        self.world_size = world_size
+        self.device = torch.device(device)
+        self.path_naming_fn = path_naming_fn or default_path_naming
+        self.heartbeat_interval = heartbeat_interval
+        self.wire = LoopbackWire(self.device if self.device.type == "cuda" else None)
+        self.pairs: dict[str, PairState] = {}
+        self.batches: dict[str, BatchState] = {}
+        self._inbox: queue.Queue = queue.Queue()
+        self._pending: list[_Entry] = []
+        self._stop = threading.Event()
+        self._queues: dict[int, CommandQueue] = {}
+        self._state_paths: dict[int, str] = {}
+        self._threads: list[threading.Thread] = []
+        self._last_heartbeat = 0.0
+        self.stats = {"ipc_tensors": 0, "in_process_tensors": 0, "transfers": 0}
+        for rank in range(world_size):
+            cmd_path, state_path = self.path_naming_fn(rank)
+            self._queues[rank] = CommandQueue(cmd_path, serve=True)
+            self._state_paths[rank] = state_path
+            t = threading.Thread(target=self._accept_loop, args=(rank,), daemon=True)
+            t.start()
+            self._threads.append(t)
+        self._write_state(force=True)
+
+    # ---- plumbing ---------------------------------------------------------------------------
+    def _accept_loop(self, rank: int) -> None:
+        q = self._queues[rank]
+        while not self._stop.is_set():
+            try:
+                conn = q.accept()
+            except (OSError, EOFError):
+                return
+            try:
+                command = conn.recv()
+            except (EOFError, OSError):
+                conn.close()
+                continue
+            self._inbox.put(_Entry(rank=rank, conn=conn, command=command))
+
+    def _write_state(self, force: bool = False) -> None:
+        now = time.time()
+        if not force and now - self._last_heartbeat < self.heartbeat_interval:
+            return
+        self._last_heartbeat = now
+        state = {
+            "agent:heartbeat": now,
+            "pairs": {name: ("matched" if p.matched else "pending") for name, p in self.pairs.items()},
+            "batches": {bid: {"transfer_signal": b.transfer_signal} for bid, b in self.batches.items()},
+        }
+        blob = json.dumps(state)
+        for path in self._state_paths.values():
+            tmp = f"{path}.tmp{os.getpid()}"
+            with open(tmp, "w") as f:
+                f.write(blob)
+            os.replace(tmp, path)
+
+    def run(self) -> None:
+        """Serve until :meth:`close` is called (the reference's ``TensorBusAgent.run``)."""
+        while not self._stop.is_set():
+            self.step(0.02)
+
+    def start_in_thread(self) -> threading.Thread:
+        t = threading.Thread(target=self.run, daemon=True, name="etha-agent")
+        t.start()
+        return t
+
+    def step(self, timeout: float = 0.0) -> None:
+        self._write_state()
+        try:
+            entry = self._inbox.get(timeout=timeout)
+            self._pending.append(entry)
+        except queue.Empty:
+            pass
+        while True:
+            try:
+                self._pending.append(self._inbox.get_nowait())
+            except queue.Empty:
+                break
+        progressed, changed = True, False
+        while progressed:
+            progressed = False
+            for entry in list(self._pending):
+                try:
+                    done, value = self._advance(entry)
+                except Exception as e:  # report to the worker, keep serving
+                    logger.exception("agent rank %s: %s failed", entry.rank, type(entry.command).__name__)
+                    self._reply(entry, ("error", (type(e).__name__, str(e))))
+                    self._pending.remove(entry)
+                    progressed = True
+                    continue
+                if done:
+                    # the state file must show the new state before the worker is released
+                    self._write_state(force=True)
+                    self._reply(entry, ("ok", value))
+                    self._pending.remove(entry)
+                    progressed = changed = True
+        self._write_state(force=changed)
+
+    @staticmethod
+    def _reply(entry: _Entry, message) -> None:
+        try:
+            entry.conn.send(message)
+        except (OSError, BrokenPipeError):
+            pass
+        finally:
+            try:
+                entry.conn.close()
+            except OSError:
+                pass
+
+    def close(self) -> None:
+        self._stop.set()
+        for q in self._queues.values():
+            q.close()
+        for b in list(self.batches.values()):
+            self._release_batch(b)
+        self.batches.clear()
+        for path in self._state_paths.values():
+            if os.path.exists(path):
+                os.unlink(path)
+
+    # ---- commands ---------------------------------------------------------------------------
+    def _advance(self, entry: _Entry):
+        cmd = entry.command
+        if isinstance(cmd, InitPair):
+            return self._init_pair(entry, cmd)
+        if isinstance(cmd, RegisterTensors):
+            return self._register_tensors(entry, cmd)
+        if isinstance(cmd, Transfer):
+            return self._transfer(entry, cmd)
+        if isinstance(cmd, QueryStatus):
+            batch = self.batches.get(cmd.batch_id)
+            if batch is None or cmd.state_name != "transfer_signal":
+                return True, False
+            return True, batch.transfer_signal
+        if isinstance(cmd, CleanupBatch):
+            batch = self.batches.get(cmd.batch_id)
+            if batch is not None:
+                batch.registrations.pop(entry.rank, None)
+                if not batch.registrations:
+                    self._release_batch(batch)
+                    del self.batches[cmd.batch_id]
+            return True, None
+        raise ValueError(f"unknown command {type(cmd).__name__}")
+
+    def _init_pair(self, entry: _Entry, cmd: InitPair):
+        pair = self.pairs.setdefault(cmd.pair_name, PairState(pair_name=cmd.pair_name))
+        if not entry.started:
+            entry.started = True
+            side = pair.sides.setdefault(cmd.local_name, {"expected": cmd.expected_world_size, "ranks": {}, "remote": cmd.remote_name})
+            if side["expected"] != cmd.expected_world_size:
+                raise ValueError(f"pair {cmd.pair_name}: ranks of '{cmd.local_name}' disagree on expected_world_size")
+            side["ranks"][entry.rank] = (cmd.mesh_shape_payload, cmd.placements_payload)
+        if pair.matched:
+            return True, "matched"
+        local, remote = pair.sides.get(cmd.local_name), pair.sides.get(cmd.remote_name)
+        if local is None or remote is None:
+            return False, None
+        if len(local["ranks"]) < local["expected"] or len(remote["ranks"]) < remote["expected"]:
+            return False, None
+        self._match_pair(pair)
+        return True, "matched"
+
+    def _match_pair(self, pair: PairState) -> None:
+        for name, side in pair.sides.items():
+            infos = list(side["ranks"].values())
+            if any(i != infos[0] for i in infos):
+                raise ValueError(f"pair {pair.pair_name}: ranks of '{name}' disagree on mesh shape or placements")
+            ranks = sorted(side["ranks"])
+            pair.ranks[name] = ranks
+            mesh_shape, placements = infos[0]
+            if mesh_shape is not None and placements is not None:
+                n = int(np.prod(mesh_shape))
+                if n != len(ranks):
+                    raise ValueError(f"pair {pair.pair_name}: mesh {mesh_shape} does not hold {len(ranks)} ranks")
+                # same rebuild as the reference: consecutive ranks from the side's first rank
+                pair.meshes[name] = (np.arange(ranks[0], ranks[0] + n).reshape(mesh_shape), tuple(placements))
+        names = sorted(pair.sides)
+        if len(names) == 2 and all(n in pair.meshes for n in names):
+            for a, b in ((names[0], names[1]), (names[1], names[0])):
+                (mesh_a, pl_a), (mesh_b, pl_b) = pair.meshes[a], pair.meshes[b]
+                if any(isinstance(p, Partial) for p in pl_b):
+                    pair.m2m[(a, b)] = None  # a Partial target is not supported: that direction is skipped
+                else:
+                    pair.m2m[(a, b)] = get_m2m_map(mesh_a, pl_a, mesh_b, pl_b)
+        pair.matched = True
+
+    def _side_of(self, pair: PairState, rank: int) -> str:
+        for name, ranks in pair.ranks.items():
+            if rank in ranks:
+                return name
+        raise ValueError(f"rank {rank} is not part of pair {pair.pair_name}")
+
+    def _register_tensors(self, entry: _Entry, cmd: RegisterTensors):
+        if not entry.started:
+            entry.started = True
+            pair_names = list(dict.fromkeys(p for p, _ in cmd.tensors))
+            for p in pair_names:
+                if p not in self.pairs or not self.pairs[p].matched:
+                    raise ValueError(f"RegisterTensors for unknown pair: {p}")
+            batch = self.batches.setdefault(cmd.batch_id, BatchState(cmd.batch_id, pair_names, cmd.bucket_size))
+            if batch.planned:
+                raise ValueError(f"batch {cmd.batch_id} is already registered")
+            index = self.device.index if self.device.type == "cuda" else None
+            batch.registrations[entry.rank] = [(p, import_tensor(payload, index)) for p, payload in cmd.tensors]
+            for _, t in batch.registrations[entry.rank]:
+                self.stats["ipc_tensors" if isinstance(t, IpcTensor) else "in_process_tensors"] += 1
+        batch = self.batches[cmd.batch_id]
+        if batch.planned:
+            return True, None
+        expected = set()
+        for p in batch.pair_names:
+            for ranks in self.pairs[p].ranks.values():
+                expected.update(ranks)
+        if not expected.issubset(batch.registrations):
+            return False, None
+        self._plan_batch(batch)
+        return True, None
+
+    def _plan_batch(self, batch: BatchState) -> None:
+        send_chunks: dict[int, list] = {}
+        recv_chunks: dict[int, list] = {}
+        for pair_name in batch.pair_names:
+            pair = self.pairs[pair_name]
+            per_rank = {r: [t for p, t in regs if p == pair_name] for r, regs in batch.registrations.items()}
+            names = sorted(pair.sides)
+            counts = {len(per_rank[r]) for name in names for r in pair.ranks[name]}
+            if len(counts) != 1:
+                raise ValueError(f"batch {batch.batch_id}: ranks registered different numbers of tensors for '{pair_name}'")
+            for i in range(counts.pop()):
+                for a, b in ((names[0], names[1]), (names[1], names[0])):
+                    m2m = pair.m2m.get((a, b))
+                    if m2m is None:
+                        continue
+                    src = {r: per_rank[r][i] for r in pair.ranks[a]}
+                    tgt = {r: per_rank[r][i] for r in pair.ranks[b]}
+                    wire_dtype = transfer_dtype_rule(next(iter(src.values())).dtype, next(iter(tgt.values())).dtype)
+                    mesh_a = pair.meshes[a][0]
+                    for r, t in src.items():
+                        groups = create_partial_groups(mesh_a, m2m.source_partial_reductions, r, src) or None
+                        send_chunks.setdefault(r, []).extend(
+                            m2m_to_chunks(m2m, r, source_tensor=t, transfer_dtype=wire_dtype, source_partial_groups=groups))
+                    for r, t in tgt.items():
+                        recv_chunks.setdefault(r, []).extend(
+                            m2m_to_chunks(m2m, r, target_tensor=t, transfer_dtype=wire_dtype))
+        size = batch.bucket_size or 1
+        batch.send_buckets = {r: chunk_to_bucket_ops(c, size) for r, c in sorted(send_chunks.items())}
+        batch.recv_buckets = {r: chunk_to_bucket_ops(c, size) for r, c in sorted(recv_chunks.items())}
+        # compile now, sources first, so that the first transfer finds every slot
+        for buckets in batch.send_buckets.values():
+            self._plan_if_device(buckets)
+        for buckets in batch.recv_buckets.values():
+            self._plan_if_device(buckets)
+        batch.send_count = {r: 0 for r in batch.send_buckets}
+        batch.recv_count = {r: 0 for r in batch.recv_buckets}
+        batch.planned = True
+
+    def _plan_if_device(self, buckets) -> None:
+        if buckets and buckets[0].chunks[0].tensor.device.type == "cuda":
+            self.wire.plan(buckets)
+
+    @staticmethod
+    def _peers(buckets, attr: str) -> set[int]:
+        out: set[int] = set()
+        for b in buckets:
+            if b.transport in (Transport.P2P, Transport.BROADCAST):
+                out.update(b.dst_ranks if attr == "dst" else (b.src_rank,))
+        return out
+
+    def _transfer(self, entry: _Entry, cmd: Transfer):
+        batch = self.batches.get(cmd.batch_id)
+        if batch is None:
+            raise ValueError(f"Transfer for unknown batch: {cmd.batch_id}")
+        if not batch.planned:
+            return False, None
+        rank = entry.rank
+        table = batch.send_buckets if cmd.transfer_type == "send" else batch.recv_buckets
+        other = batch.recv_buckets if cmd.transfer_type == "send" else batch.send_buckets
+        buckets = table.get(rank)
+        if not buckets:
+            if any(other.values()) or any(table.values()):
+                raise RuntimeError(
+                    f"Batch {cmd.batch_id}: no {cmd.transfer_type} chunks. The pair's {cmd.transfer_type} direction "
+                    "has a Partial target, which is not supported. Partial is only valid as a source placement."
+                )
+            return True, None
+        if cmd.transfer_type == "send":
+            gen = batch.send_count[rank]
+            for d in self._peers(buckets, "dst"):
+                if d in batch.recv_count and batch.recv_count[d] < gen:
+                    return False, None  # the previous generation has not been consumed yet
+            batch.transfer_signal = True
+            t0 = time.perf_counter()
+            bucket_comm(buckets, wire=self.wire, merge_launches=True)
+            batch.send_count[rank] = gen + 1
+            for d in self._peers(buckets, "dst"):
+                batch.owed[d] = max(batch.owed.get(d, 0), gen + 1)
+        else:
+            gen = batch.recv_count[rank]
+            for s in self._peers(buckets, "src"):
+                if batch.send_count.get(s, 0) <= gen:
+                    return False, None  # wait for the source's send of this generation
+            t0 = time.perf_counter()
+            bucket_comm(buckets, wire=self.wire, merge_launches=True)
+            batch.recv_count[rank] = gen + 1
+            if all(batch.recv_count.get(d, 0) >= n for d, n in batch.owed.items()):
+                batch.transfer_signal = False  # every destination of every send so far has received
+        self.stats["transfers"] += 1
+        return True, {"ms": (time.perf_counter() - t0) * 1e3}
+
+    @staticmethod
+    def _release_batch(batch: BatchState) -> None:
+        for regs in batch.registrations.values():
+            for _, t in regs:
+                if isinstance(t, IpcTensor):
+                    try:
+                        t.close()
+                    except Exception:
+                        logger.exception("closing an IPC mapping failed")
+        batch.registrations.clear()
+        batch.send_buckets.clear()
+        batch.recv_buckets.clear()

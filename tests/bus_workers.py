@@ -1,0 +1,153 @@
+"""Worker-process bodies for the tensor-bus tests (importable by multiprocessing 'spawn')."""
+
+from __future__ import annotations
+
+import os
+import sys
+import threading
+import traceback
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+for p in (ROOT, os.path.join(ROOT, "tests")):
+    if p not in sys.path:
+        sys.path.insert(0, p)
+
+
+def path_naming(tmpdir):
+    def fn(rank: int):
+        return os.path.join(tmpdir, f"agent_rank{rank}_command.lmdb"), os.path.join(tmpdir, f"agent_rank{rank}_state.lmdb")
+
+    return fn
+
+
+def run_ranks(fn, ranks):
+    """Run ``fn(rank)`` for every rank in its own thread (each rank blocks on the others)."""
+    errors, results = [], {}
+
+    def body(r):
+        try:
+            results[r] = fn(r)
+        except BaseException:
+            errors.append((r, traceback.format_exc()))
+
+    threads = [threading.Thread(target=body, args=(r,)) for r in ranks]
+    for t in threads:
+        t.start()
+    for t in threads:
+        t.join(120)
+    if errors:
+        raise RuntimeError("rank %d failed:\n%s" % errors[0])
+    return results
+
+
+# specs of the two-process test: (name, shape, source placements code, target placements code, src dtype, tgt dtype)
+BUS_TENSORS = [
+    ("q", (256, 128), ["S0"], ["S0"], "bfloat16", "bfloat16"),
+    ("o", (128, 256), ["S0"], ["S1"], "bfloat16", "bfloat16"),
+    ("norm", (64,), ["S0"], ["R"], "float32", "bfloat16"),
+]
+SRC_RANKS, TGT_RANKS = [0, 1, 2, 3], [4, 5]
+
+
+def _global(i, round_):
+    import torch
+
+    g = torch.Generator().manual_seed(100 * round_ + i)
+    return torch.randn(BUS_TENSORS[i][1], generator=g)
+
+
+def trainer_process(tmpdir, device, rounds, out_q):
+    """All source ranks of the pair, in one worker process: fill shards, send, twice."""
+    try:
+        import torch
+
+        from etha_amd.layout import local_shard
+        from etha_amd.tensor_bus import TensorBusClient
+        from etha_amd.tensor_bus.bootstrap import setup_ptrace
+        from helpers import parse_placements
+
+        setup_ptrace()
+        naming = path_naming(tmpdir)
+        names = {"float32": torch.float32, "bfloat16": torch.bfloat16}
+        shards = {r: [] for r in SRC_RANKS}
+        for i, (_, shape, src, _, sdt, _) in enumerate(BUS_TENSORS):
+            g = _global(i, 0).to(names[sdt])
+            for pos, r in enumerate(SRC_RANKS):
+                shards[r].append(local_shard(g, (len(SRC_RANKS),), parse_placements(src), (pos,)).clone().to(device))
+        barrier = threading.Barrier(len(SRC_RANKS))
+
+        def rank_body(r):
+            cmd, state = naming(r)
+            client = TensorBusClient(r, cmd, state, connection_timeout=20)
+            for i, (name, _, src, _, _, _) in enumerate(BUS_TENSORS):
+                client.init_pair(f"pair_{name}", "trainer", "inference", len(SRC_RANKS), device_mesh=torch.arange(len(SRC_RANKS)),
+                                 placements=parse_placements(src), timeout=30)
+            handler = client.register_tensors("weights", [(t, f"pair_{BUS_TENSORS[i][0]}") for i, t in enumerate(shards[r])],
+                                              bucket_size=16 * 1024, timeout=30)
+            for round_ in range(rounds):
+                if round_ > 0:  # new values in the same registered tensors: plan once, transfer N times
+                    for i, (_, _, src, _, sdt, _) in enumerate(BUS_TENSORS):
+                        g = _global(i, round_).to(names[sdt])
+                        pos = SRC_RANKS.index(r)
+                        shards[r][i].copy_(local_shard(g, (len(SRC_RANKS),), parse_placements(src), (pos,)))
+                    torch.cuda.synchronize()
+                barrier.wait(60)
+                handler.transfer("send", blocking=True, timeout=60)
+            handler.close()
+            client.close()
+            return True
+
+        run_ranks(rank_body, SRC_RANKS)
+        out_q.put(("trainer", "ok", None))
+    except BaseException:
+        out_q.put(("trainer", "error", traceback.format_exc()))
+
+
+def inference_process(tmpdir, device, rounds, out_q):
+    """All target ranks in another worker process: receive and compare with the closed form."""
+    try:
+        import torch
+
+        from etha_amd.layout import local_shape, local_shard
+        from etha_amd.tensor_bus import TensorBusClient
+        from etha_amd.tensor_bus.bootstrap import setup_ptrace
+        from helpers import parse_placements
+
+        setup_ptrace()
+        naming = path_naming(tmpdir)
+        names = {"float32": torch.float32, "bfloat16": torch.bfloat16}
+        locals_ = {r: [] for r in TGT_RANKS}
+        for i, (_, shape, _, tgt, _, tdt) in enumerate(BUS_TENSORS):
+            for pos, r in enumerate(TGT_RANKS):
+                shp = local_shape(shape, (len(TGT_RANKS),), parse_placements(tgt), (pos,))
+                locals_[r].append(torch.full(shp, -1.0, dtype=names[tdt], device=device))
+        mismatches = []
+
+        def rank_body(r):
+            cmd, state = naming(r)
+            client = TensorBusClient(r, cmd, state, connection_timeout=20)
+            for i, (name, _, _, tgt, _, _) in enumerate(BUS_TENSORS):
+                client.init_pair(f"pair_{name}", "inference", "trainer", len(TGT_RANKS), device_mesh=torch.arange(len(TGT_RANKS)),
+                                 placements=parse_placements(tgt), timeout=30)
+            handler = client.register_tensors("weights", [(t, f"pair_{BUS_TENSORS[i][0]}") for i, t in enumerate(locals_[r])],
+                                              bucket_size=16 * 1024, timeout=30)
+            for round_ in range(rounds):
+                handler.transfer("recv", blocking=True, timeout=60)
+                torch.cuda.synchronize()
+                for i, (name, _, _, tgt, sdt, tdt) in enumerate(BUS_TENSORS):
+                    g = _global(i, round_).to(names[sdt])
+                    want = local_shard(g, (len(TGT_RANKS),), parse_placements(tgt), (TGT_RANKS.index(r),))
+                    wire = names[sdt] if names[sdt].itemsize <= names[tdt].itemsize else names[tdt]
+                    want = want.to(wire).to(names[tdt])
+                    got = locals_[r][i].cpu()
+                    if not torch.equal(got.view(torch.uint8), want.contiguous().view(torch.uint8)):
+                        mismatches.append((round_, r, name))
+            signal = handler.query_transfer_signal()
+            handler.close()
+            client.close()
+            return signal
+
+        signals = run_ranks(rank_body, TGT_RANKS)
+        out_q.put(("inference", "ok" if not mismatches else "mismatch", {"mismatches": mismatches, "signals": signals}))
+    except BaseException:
+        out_q.put(("inference", "error", traceback.format_exc()))

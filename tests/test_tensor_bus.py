@@ -1,0 +1,197 @@
+"""The worker-facing surface: TensorBusClient / BatchHandler against the hub agent."""
+
+import json
+import multiprocessing as mp
+import os
+import time
+
+import pytest
+import torch
+from torch.distributed.tensor.placement_types import Partial, Replicate, Shard
+
+from etha_amd.tensor_bus import TensorBusAgent, TensorBusClient, bootstrap_client
+
+from bus_workers import inference_process, path_naming, run_ranks, trainer_process
+
+
+@pytest.fixture
+def agent_factory(tmp_path):
+    agents = []
+
+    def make(world_size, device="cpu"):
+        a = TensorBusAgent(world_size, path_naming(str(tmp_path)), device=device, heartbeat_interval=0.05)
+        a.start_in_thread()
+        agents.append(a)
+        return a, path_naming(str(tmp_path))
+
+    yield make
+    for a in agents:
+        a.close()
+
+
+def _client(naming, rank, **kw):
+    cmd, state = naming(rank)
+    return TensorBusClient(rank, cmd, state, **kw)
+
+
+def test_connection_errors(tmp_path):
+    with pytest.raises(ConnectionError, match="not found"):
+        TensorBusClient(0, str(tmp_path / "c"), str(tmp_path / "missing_state"), connection_timeout=0.3)
+    stale = tmp_path / "stale_state"
+    stale.write_text(json.dumps({"agent:heartbeat": time.time() - 60}))
+    with pytest.raises(ConnectionError, match="Heartbeat is too old"):
+        TensorBusClient(0, str(tmp_path / "c"), str(stale), connection_timeout=0.3)
+    with pytest.raises(ValueError):
+        os.environ.pop("TENSOR_BUS_STATE_PATH", None)
+        TensorBusClient(0)
+
+
+def test_init_pair_register_and_errors_on_cpu(agent_factory):
+    agent, naming = agent_factory(3)
+    clients = {r: _client(naming, r, connection_timeout=5) for r in range(3)}
+    # the remote side never joins: blocking init_pair times out like the reference's semaphore wait
+    with pytest.raises(TimeoutError):
+        clients[0].init_pair("lonely", "a", "b", 1, device_mesh=torch.arange(1), placements=(Replicate(),), timeout=0.3)
+
+    src = {0: torch.arange(8.0).reshape(2, 4), 1: torch.arange(8.0, 16.0).reshape(2, 4)}
+    tgt = {2: torch.zeros(4, 4)}
+
+    def body(r):
+        c = clients[r]
+        if r < 2:
+            c.init_pair("w", "trainer", "inference", 2, device_mesh=torch.arange(2), placements=(Shard(0),), timeout=10)
+            return c.register_tensors("b0", [(src[r], "w")], bucket_size=None, timeout=10)
+        c.init_pair("w", "inference", "trainer", 1, device_mesh=torch.arange(1), placements=(Replicate(),), timeout=10)
+        return c.register_tensors("b0", [(tgt[2], "w")], timeout=10)
+
+    handlers = run_ranks(body, range(3))
+    assert handlers[0].pair_names == ["w"] and handlers[0].batch_id == "b0"
+    state = json.load(open(naming(0)[1]))
+    assert state["pairs"]["w"] == "matched"
+    batch = agent.batches["b0"]
+    assert batch.planned and len(batch.send_buckets[0]) == 1 and len(batch.recv_buckets[2]) == 2
+    assert batch.send_buckets[1][0].chunks[0].dst_ranks == (2,)
+    assert handlers[2].query_transfer_signal() is False
+    with pytest.raises(ValueError, match="cannot be empty"):
+        clients[0].register_tensors("b1", [])
+    with pytest.raises(ValueError, match="unknown pair"):
+        clients[0].register_tensors("b2", [(src[0], "nope")], timeout=5)
+    with pytest.raises(ValueError, match="unknown batch"):
+        clients[0].transfer("never_registered", "send", blocking=True, timeout=5)
+    # the hot path has no CPU implementation: a transfer of host tensors fails loudly
+    with pytest.raises(RuntimeError, match="no CPU path"):
+        handlers[0].transfer("send", blocking=True, timeout=5)
+    sem = handlers[2].transfer("recv", blocking=False)  # its sources never sent: stays pending
+    with pytest.raises(Exception):
+        sem.acquire(timeout=0.3)
+    for h in handlers.values():
+        h.close()
+    assert "b0" not in agent.batches
+    for c in clients.values():
+        c.close()
+
+
+def test_partial_target_direction_is_rejected(agent_factory):
+    agent, naming = agent_factory(2)
+    clients = {r: _client(naming, r, connection_timeout=5) for r in range(2)}
+    t = {0: torch.zeros(4, 4), 1: torch.zeros(4, 4)}
+
+    def body(r):
+        c = clients[r]
+        if r == 0:
+            c.init_pair("p", "a", "b", 1, device_mesh=torch.arange(1), placements=(Partial(),), timeout=10)
+        else:
+            c.init_pair("p", "b", "a", 1, device_mesh=torch.arange(1), placements=(Replicate(),), timeout=10)
+        return c.register_tensors("b", [(t[r], "p")], timeout=10)
+
+    handlers = run_ranks(body, range(2))
+    assert agent.pairs["p"].m2m[("b", "a")] is None and agent.pairs["p"].m2m[("a", "b")] is not None
+    with pytest.raises(RuntimeError, match="Partial target"):
+        handlers[1].transfer("send", blocking=True, timeout=5)  # b -> a would need a Partial target
+    for c in clients.values():
+        c.close()
+
+
+def test_bootstrap_client_resolves_rank_and_paths(agent_factory, monkeypatch):
+    agent, naming = agent_factory(3)
+    monkeypatch.setenv("RANK", "1")
+    monkeypatch.delenv("AGENT_RANK", raising=False)
+    monkeypatch.setenv("AGENT_RANK_OFFSET", "1")
+    client, info = bootstrap_client(naming, connection_timeout=5)
+    assert (info.agent_rank, info.global_rank, info.rank_offset, info.method) == (2, 1, 1, "offset")
+    assert info.command_queue_path == naming(2)[0] and client.agent_rank == 2
+    client.close()
+    monkeypatch.setenv("AGENT_RANK", "0")
+    client, info = bootstrap_client(naming, connection_timeout=5)
+    assert (info.agent_rank, info.rank_offset, info.method) == (0, None, "direct")
+    client.close()
+
+
+@pytest.mark.gpu
+def test_in_process_agent_end_to_end(gpu_device, agent_factory):
+    """Trainer ranks 0..3 (fp32, Shard(0)) -> inference ranks 4..5 (bf16, Shard(1)) through the bus."""
+    agent, naming = agent_factory(6, device=gpu_device)
+    g = torch.Generator().manual_seed(3)
+    glob = torch.randn(64, 96, generator=g)
+    src = {r: glob[16 * r : 16 * (r + 1)].clone().to(gpu_device) for r in range(4)}
+    tgt = {4 + j: torch.zeros(64, 48, dtype=torch.bfloat16, device=gpu_device) for j in range(2)}
+    clients = {r: _client(naming, r, connection_timeout=5) for r in range(6)}
+
+    def body(r):
+        c = clients[r]
+        if r < 4:
+            c.init_pair("w", "trainer", "inference", 4, device_mesh=torch.arange(4), placements=(Shard(0),))
+            h = c.register_tensors("step", [(src[r], "w")], bucket_size=1 << 20)
+            h.transfer("send", blocking=True)
+        else:
+            c.init_pair("w", "inference", "trainer", 2, device_mesh=torch.arange(2), placements=(Shard(1),))
+            h = c.register_tensors("step", [(tgt[r], "w")], bucket_size=1 << 20)
+            h.transfer("recv", blocking=True)
+        return h
+
+    handlers = run_ranks(body, range(6))
+    torch.cuda.synchronize()
+    for j in range(2):
+        want = glob[:, 48 * j : 48 * (j + 1)].to(torch.bfloat16)
+        assert torch.equal(tgt[4 + j].cpu(), want)
+    assert handlers[4].query_transfer_signal() is False  # every receiver has caught up
+    for h in handlers.values():
+        h.close()
+    for c in clients.values():
+        c.close()
+
+
+@pytest.mark.gpu
+def test_two_process_hipipc_handoff(gpu_device, tmp_path):
+    """Worker processes own the tensors; the agent (this process) maps them with hipIpcOpenMemHandle,
+    packs and unpacks, twice, with new values the second time."""
+    agent = TensorBusAgent(6, path_naming(str(tmp_path)), device=gpu_device, heartbeat_interval=0.05)
+    agent.start_in_thread()
+    ctx = mp.get_context("spawn")
+    out_q = ctx.Queue()
+    procs = [ctx.Process(target=trainer_process, args=(str(tmp_path), str(gpu_device), 2, out_q)),
+             ctx.Process(target=inference_process, args=(str(tmp_path), str(gpu_device), 2, out_q))]
+    try:
+        for p in procs:
+            p.start()
+        results = {}
+        deadline = time.time() + 150
+        while len(results) < 2 and time.time() < deadline:
+            try:
+                who, status, detail = out_q.get(timeout=1.0)
+                results[who] = (status, detail)
+            except Exception:
+                if any(p.exitcode not in (None, 0) for p in procs):
+                    break
+        for p in procs:
+            p.join(20)
+        assert results.get("trainer", ("missing", None))[0] == "ok", results.get("trainer")
+        assert results.get("inference", ("missing", None))[0] == "ok", results.get("inference")
+        # the agent really worked on hipIPC-mapped pointers: 3 tensors x (4 + 2) ranks, 2 rounds x 6 transfers
+        assert agent.stats == {"ipc_tensors": 18, "in_process_tensors": 0, "transfers": 12}
+        assert agent.batches == {} or all(not b.registrations for b in agent.batches.values())
+    finally:
+        for p in procs:
+            if p.is_alive():
+                p.kill()
+        agent.close()
