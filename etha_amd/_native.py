@@ -98,6 +98,8 @@ _SIGNATURES = {
     "etha_table_info": (c_int, [c_void_p, POINTER(TableInfo)]),
     "etha_table_read_tiles": (c_int, [c_void_p, c_int, c_void_p, c_uint64, POINTER(c_uint64)]),
     "etha_table_read_ranges": (c_int, [c_void_p, c_void_p, c_void_p]),
+    "etha_table_optimize_range": (c_int, [c_void_p, c_uint32, c_uint32]),
+    "etha_table_read_ordered": (c_int, [c_void_p, c_uint32, c_uint32, c_int, c_void_p, c_uint64, POINTER(c_uint64)]),
     "etha_pack_bucket": (c_int, [c_void_p, c_uint32, c_uint32, c_void_p]),
     "etha_unpack_bucket": (c_int, [c_void_p, c_uint32, c_uint32, c_void_p]),
     "etha_reduce_pack_bucket": (c_int, [c_void_p, c_uint32, c_uint32, c_void_p]),
@@ -200,6 +202,23 @@ class Table:
             lib().etha_table_read_ranges(self._h, run_begin.ctypes.data, row_begin.ctypes.data),
         )
         return run_begin, row_begin
+
+    def optimize_range(self, first: int, count: int) -> None:
+        """Order the tiles of a range that is always launched as one unit by written address."""
+        _check("etha_table_optimize_range", lib().etha_table_optimize_range(self._h, first, count))
+
+    def ordered_tiles(self, first: int, count: int) -> tuple[np.ndarray, np.ndarray]:
+        res = []
+        for which, dt in ((0, RUN_TILE), (1, ROW_TILE)):
+            need = c_uint64()
+            _check("etha_table_read_ordered",
+                   lib().etha_table_read_ordered(self._h, first, count, which, None, 0, byref(need)))
+            arr = np.zeros(need.value // dt.itemsize, dtype=dt)
+            if need.value:
+                _check("etha_table_read_ordered",
+                       lib().etha_table_read_ordered(self._h, first, count, which, arr.ctypes.data, need.value, byref(need)))
+            res.append(arr)
+        return res[0], res[1]
 
     def pack(self, first: int, count: int, stream: int = 0) -> None:
         _check("etha_pack_bucket", lib().etha_pack_bucket(self._h, first, count, c_void_p(stream)))

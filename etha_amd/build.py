@@ -15,7 +15,8 @@ PKG_DIR = os.path.dirname(os.path.abspath(__file__))
 REPO_DIR = os.path.dirname(PKG_DIR)
 SOURCE = os.path.join(PKG_DIR, "csrc", "etha_reshard.hip")
 INCLUDE_DIR = os.path.join(REPO_DIR, "include")
-LIB_PATH = os.path.join(PKG_DIR, "libetha_reshard.so")
+# ETHA_AMD_LIB selects another build of the same library (kernel tuning experiments)
+LIB_PATH = os.environ.get("ETHA_AMD_LIB") or os.path.join(PKG_DIR, "libetha_reshard.so")
 
 HIPCC_FLAGS = [
     "-O3",
@@ -35,16 +36,17 @@ def hipcc_path() -> str:
     return path
 
 
-def build_library(verbose: bool = False) -> str:
+def build_library(verbose: bool = False, defines: tuple[str, ...] = (), out_path: str | None = None) -> str:
     """Compile the shared library (always recompiles) and return its path."""
-    cmd = [hipcc_path(), *HIPCC_FLAGS, f"-I{INCLUDE_DIR}", "-o", LIB_PATH + ".tmp", SOURCE]
+    out_path = out_path or LIB_PATH
+    cmd = [hipcc_path(), *HIPCC_FLAGS, *[f"-D{d}" for d in defines], f"-I{INCLUDE_DIR}", "-o", out_path + ".tmp", SOURCE]
     proc = subprocess.run(cmd, capture_output=True, text=True)
     if proc.returncode != 0:
         raise RuntimeError(f"hipcc failed ({proc.returncode}):\n{' '.join(cmd)}\n{proc.stdout}\n{proc.stderr}")
     if verbose and proc.stderr:
         sys.stderr.write(proc.stderr)
-    os.replace(LIB_PATH + ".tmp", LIB_PATH)
-    return LIB_PATH
+    os.replace(out_path + ".tmp", out_path)
+    return out_path
 
 
 if __name__ == "__main__":

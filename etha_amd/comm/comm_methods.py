@@ -101,6 +101,13 @@ class TransferPlan:
         self.recv_table = recv.build()
         self.local_table = local.build()
         self.merged_steps = self._merge(self.steps)
+        # merged unpack / self-copy launches cover several buckets: let the library order their tiles by
+        # written address, so that rows of one tensor arriving through different buckets are written together
+        for kind, first, count, slots in self.merged_steps:
+            if len(slots) > 1 and kind == _UNPACK:
+                self.recv_table.optimize_range(first, count)
+            elif len(slots) > 1 and kind == _SELF:
+                self.local_table.optimize_range(first, count)
 
     @staticmethod
     def _merge(steps):

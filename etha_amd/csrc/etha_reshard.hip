@@ -15,6 +15,7 @@
 
 #include <cstdarg>
 #include <cstdio>
+#include <algorithm>
 #include <array>
 #include <cstring>
 #include <map>
@@ -27,7 +28,19 @@
 
 namespace {
 
-constexpr uint32_t kTileThreads = 256;  // work-items per tile = units per tile
+#ifndef ETHA_TILE_UNITS
+#define ETHA_TILE_UNITS 1024
+#endif
+#ifndef ETHA_BLOCK_THREADS
+#define ETHA_BLOCK_THREADS 64
+#endif
+// One table entry (tile) describes kTileThreads units; it is executed by kBlocksPerTile workgroups of
+// kBlockThreads work-items (one wavefront each).  Wave-sized workgroups schedule best; the coarser
+// table granularity keeps the tile program small.
+constexpr uint32_t kTileThreads = ETHA_TILE_UNITS;     // units per tile
+constexpr uint32_t kBlockThreads = ETHA_BLOCK_THREADS; // work-items per workgroup
+constexpr uint32_t kBlocksPerTile = kTileThreads / kBlockThreads;
+static_assert(kTileThreads % kBlockThreads == 0 && kBlocksPerTile >= 1, "tile must be a multiple of the workgroup");
 
 // ---- tile program entries (device-visible, also read back by host-side checkers) -------------
 // A "unit" is what one work-item moves: 2^ua bytes on the a side and 2^ub bytes on the b side
@@ -69,13 +82,16 @@ constexpr uint32_t kMetaVec = 1u << 17; // converting move handles the full vect
 typedef uint32_t u32x2 __attribute__((ext_vector_type(2)));
 typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
 
+// Addresses come out of the tile program as integers; the global address space is stated
+// explicitly so that the accesses are global_load/global_store and not generic (flat) ones.
+#define ETHA_GLOBAL __attribute__((address_space(1)))
 template <typename V>
 __device__ __forceinline__ V ld_stream(uint64_t addr) {
-  return __builtin_nontemporal_load(reinterpret_cast<const V*>(addr));
+  return __builtin_nontemporal_load(reinterpret_cast<const ETHA_GLOBAL V*>(addr));
 }
 template <typename V>
 __device__ __forceinline__ void st_stream(uint64_t addr, V v) {
-  __builtin_nontemporal_store(v, reinterpret_cast<V*>(addr));
+  __builtin_nontemporal_store(v, reinterpret_cast<ETHA_GLOBAL V*>(addr));
 }
 template <typename V>
 __device__ __forceinline__ void copy_as(uint64_t src, uint64_t dst) {
@@ -197,9 +213,10 @@ __device__ __forceinline__ void row_position(const RowTile& t, uint32_t tid, uin
 
 // pack (REV = false): a -> b.   unpack (REV = true): b -> a.
 template <bool REV>
-__global__ __launch_bounds__(256) void etha_tile_kernel(const RunTile* __restrict__ run_tiles, uint32_t n_run,
-                                                         const RowTile* __restrict__ row_tiles) {
-  const uint32_t bid = blockIdx.x, tid = threadIdx.x;
+__global__ __launch_bounds__(ETHA_BLOCK_THREADS) void etha_tile_kernel(const RunTile* __restrict__ run_tiles, uint32_t n_run,
+                                                                        const RowTile* __restrict__ row_tiles) {
+  const uint32_t bid = blockIdx.x / kBlocksPerTile;
+  const uint32_t tid = (blockIdx.x % kBlocksPerTile) * kBlockThreads + threadIdx.x;
   uint64_t a, b;
   uint32_t n, meta;
   if (bid < n_run) {
@@ -337,10 +354,10 @@ __device__ __forceinline__ void reduce_from(uint32_t dd, bool vec, const uint64_
   }
 }
 
-__global__ __launch_bounds__(256) void etha_reduce_kernel(const RowTile* __restrict__ row_tiles,
+__global__ __launch_bounds__(ETHA_BLOCK_THREADS) void etha_reduce_kernel(const RowTile* __restrict__ row_tiles,
                                                            const uint64_t* __restrict__ peer_bases) {
-  const uint32_t tid = threadIdx.x;
-  const RowTile t = row_tiles[blockIdx.x];
+  const uint32_t tid = (blockIdx.x % kBlocksPerTile) * kBlockThreads + threadIdx.x;
+  const RowTile t = row_tiles[blockIdx.x / kBlocksPerTile];
   if (tid >= t.n) return;
   uint32_t r, c;
   row_position(t, tid, r, c);
@@ -462,7 +479,7 @@ struct Builder {
   uint64_t payload_bytes = 0;
 };
 
-constexpr uint64_t kMaxTiles = 0x7fff0000ull;  // grid.x limit with margin
+constexpr uint64_t kMaxTiles = 0x7fff0000ull / kBlocksPerTile;  // grid.x limit with margin
 
 struct ReduceSpec {
   uint32_t n_peers = 0, peer_first = 0, op = 0;
@@ -548,7 +565,7 @@ int compile_pair(Builder& bld, uint32_t idx, const Region& A0, const Region& B0,
 
   // 5. tiles.  Long or 256-multiple rows (and single runs) become run tiles; other shapes become
   //    row tiles over the innermost remaining dim; dims further out are unrolled here.
-  const bool use_rows = red.n_peers != 0 || (k > 0 && run_units % kTileThreads != 0 && run_units < 4096);
+  const bool use_rows = red.n_peers != 0 || (k > 0 && run_units % kTileThreads != 0 && run_units < 4 * kTileThreads);
   if (run_units > 0xffffffffull && use_rows && k > 0)
     return fail(ETHA_ERR_UNSUPPORTED, "chunk %u: row longer than 2^32 units", idx);
   const int outer = use_rows && k > 0 ? k - 1 : k;  // dims unrolled on the host
@@ -628,11 +645,20 @@ struct EthaTable {
   uint64_t payload_bytes = 0;
   uint64_t device_bytes = 0;
   bool uploaded = false;
+  // write-ordered copies of the tiles of ranges that are always launched as one unit
+  struct Ordered {
+    std::vector<RunTile> h_run;
+    std::vector<RowTile> h_row;
+    RunTile* d_run = nullptr;
+    RowTile* d_row = nullptr;
+  };
+  std::map<std::pair<uint32_t, uint32_t>, Ordered> ordered;
 };
 
 namespace {
 
 int upload_table(EthaTable* t) {
+
   if (!t->h_run.empty()) {
     const size_t bytes = t->h_run.size() * sizeof(RunTile);
     HIP_TRY(hipMalloc(&t->d_run, bytes));
@@ -660,6 +686,10 @@ void free_table(EthaTable* t) {
   if (t->d_run) (void)hipFree(t->d_run);
   if (t->d_row) (void)hipFree(t->d_row);
   if (t->d_peers) (void)hipFree(t->d_peers);
+  for (auto& kv : t->ordered) {
+    if (kv.second.d_run) (void)hipFree(kv.second.d_run);
+    if (kv.second.d_row) (void)hipFree(kv.second.d_row);
+  }
   delete t;
 }
 
@@ -697,8 +727,17 @@ int launch_tiles(const EthaTable* t, uint32_t first, uint32_t count, void* strea
   const uint32_t w0 = t->row_begin[first], w1 = t->row_begin[first + count];
   const uint32_t n_run = r1 - r0, n_row = w1 - w0;
   if (n_run + n_row == 0) return ETHA_OK;
-  hipLaunchKernelGGL(etha_tile_kernel<REV>, dim3(n_run + n_row), dim3(kTileThreads), 0, (hipStream_t)stream,
-                     t->d_run + r0, n_run, t->d_row + w0);
+  if (REV == (t->kind == 0)) {  // the direction that writes the a side (unpack) / b side (self-copy) of an ordered range
+    auto it = t->ordered.find(std::make_pair(first, count));
+    if (it != t->ordered.end()) {
+      hipLaunchKernelGGL(etha_tile_kernel<REV>, dim3((n_run + n_row) * kBlocksPerTile), dim3(kBlockThreads), 0,
+                         (hipStream_t)stream, it->second.d_run, n_run, it->second.d_row);
+      HIP_TRY(hipGetLastError());
+      return ETHA_OK;
+    }
+  }
+  hipLaunchKernelGGL(etha_tile_kernel<REV>, dim3((n_run + n_row) * kBlocksPerTile), dim3(kBlockThreads), 0,
+                     (hipStream_t)stream, t->d_run + r0, n_run, t->d_row + w0);
   HIP_TRY(hipGetLastError());
   return ETHA_OK;
 }
@@ -857,6 +896,55 @@ int etha_table_read_ranges(const EthaTable* t, uint32_t* run_begin, uint32_t* ro
   return ETHA_OK;
 }
 
+int etha_table_optimize_range(EthaTable* t, uint32_t first, uint32_t count) {
+  if (!t) return fail(ETHA_ERR_INVALID, "null table");
+  if ((uint64_t)first + count > t->n_chunks)
+    return fail(ETHA_ERR_INVALID, "chunk range [%u,%u) exceeds table of %u chunks", first, first + count, t->n_chunks);
+  if (t->reduce_prefix[first + count] != t->reduce_prefix[first]) return ETHA_OK;  // reduce-pack writes buckets: already ordered
+  const auto key = std::make_pair(first, count);
+  if (t->ordered.count(key)) return ETHA_OK;
+  EthaTable::Ordered o;
+  o.h_run.assign(t->h_run.begin() + t->run_begin[first], t->h_run.begin() + t->run_begin[first + count]);
+  o.h_row.assign(t->h_row.begin() + t->row_begin[first], t->h_row.begin() + t->row_begin[first + count]);
+  const bool by_a = t->kind == 0;  // unpack writes the tensor (a) side; a self-copy writes its b side
+  const auto unit = [](uint32_t meta, bool a_side) { return 1ull << ((meta >> (a_side ? kMetaUaShift : kMetaUbShift)) & 15u); };
+  std::stable_sort(o.h_run.begin(), o.h_run.end(),
+                   [by_a](const RunTile& x, const RunTile& y) { return by_a ? x.a < y.a : x.b < y.b; });
+  std::stable_sort(o.h_row.begin(), o.h_row.end(), [by_a, unit](const RowTile& x, const RowTile& y) {
+    const uint64_t px = (by_a ? x.a : x.b) + x.c0 * unit(x.meta, by_a), py = (by_a ? y.a : y.b) + y.c0 * unit(y.meta, by_a);
+    return px < py;
+  });
+  if (t->uploaded) {
+    if (!o.h_run.empty()) {
+      const size_t bytes = o.h_run.size() * sizeof(RunTile);
+      HIP_TRY(hipMalloc(&o.d_run, bytes));
+      HIP_TRY(hipMemcpy(o.d_run, o.h_run.data(), bytes, hipMemcpyHostToDevice));
+      t->device_bytes += bytes;
+    }
+    if (!o.h_row.empty()) {
+      const size_t bytes = o.h_row.size() * sizeof(RowTile);
+      HIP_TRY(hipMalloc(&o.d_row, bytes));
+      HIP_TRY(hipMemcpy(o.d_row, o.h_row.data(), bytes, hipMemcpyHostToDevice));
+      t->device_bytes += bytes;
+    }
+  }
+  t->ordered.emplace(key, std::move(o));
+  return ETHA_OK;
+}
+
+int etha_table_read_ordered(const EthaTable* t, uint32_t first, uint32_t count, int which, void* out, uint64_t cap_bytes,
+                            uint64_t* need_bytes) {
+  if (!t || !need_bytes) return fail(ETHA_ERR_INVALID, "null argument");
+  auto it = t->ordered.find(std::make_pair(first, count));
+  if (it == t->ordered.end()) return fail(ETHA_ERR_INVALID, "range [%u,+%u) has not been optimized", first, count);
+  const void* src = which == 0 ? (const void*)it->second.h_run.data() : (const void*)it->second.h_row.data();
+  const uint64_t bytes = which == 0 ? it->second.h_run.size() * sizeof(RunTile) : it->second.h_row.size() * sizeof(RowTile);
+  if (which != 0 && which != 1) return fail(ETHA_ERR_INVALID, "which must be 0 or 1");
+  *need_bytes = bytes;
+  if (out && bytes) memcpy(out, src, bytes < cap_bytes ? bytes : cap_bytes);
+  return ETHA_OK;
+}
+
 int etha_pack_bucket(const EthaTable* t, uint32_t first, uint32_t count, void* stream) {
   const int rc = check_range(t, first, count, 0);
   if (rc != ETHA_OK) return rc;
@@ -880,7 +968,7 @@ int etha_reduce_pack_bucket(const EthaTable* t, uint32_t first, uint32_t count, 
     return fail(ETHA_ERR_INVALID, "range holds chunks that are not Partial chunks");
   const uint32_t w0 = t->row_begin[first], w1 = t->row_begin[first + count];
   if (w1 == w0) return ETHA_OK;
-  hipLaunchKernelGGL(etha_reduce_kernel, dim3(w1 - w0), dim3(kTileThreads), 0, (hipStream_t)stream, t->d_row + w0,
+  hipLaunchKernelGGL(etha_reduce_kernel, dim3((w1 - w0) * kBlocksPerTile), dim3(kBlockThreads), 0, (hipStream_t)stream, t->d_row + w0,
                      t->d_peers);
   HIP_TRY(hipGetLastError());
   return ETHA_OK;

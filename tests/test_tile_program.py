@@ -180,3 +180,32 @@ def test_selfcopy_tiles():
     execute(table, arena, "selfcopy")
     got = arena.bytes_at(t, n * 4).view(np.float32)
     assert np.array_equal(got[32:48], vals[:16]) and np.array_equal(got[:32], vals[:32]) and np.array_equal(got[48:], vals[48:])
+
+
+def test_optimized_range_is_a_write_ordered_permutation():
+    """Four column blocks of one [1024, 256] tensor arrive through four buckets; the optimized range must
+    hold exactly the same tiles, ordered by the tensor address they write."""
+    rows, cols, es = 1024, 256, 2
+    arena = HostArena(4 * rows * cols * es + 65536)
+    t = arena.alloc(rows * cols * es)
+    descs, buckets = [], []
+    for j in range(4):
+        b = arena.alloc(rows * (cols // 4) * es)
+        arena.bytes_at(b, rows * (cols // 4) * es)[:] = rs.randint(0, 256, rows * (cols // 4) * es)
+        buckets.append(b)
+        descs.append(_mk_desc(t, t, t + rows * cols * es, b, b, b + rows * (cols // 4) * es, (0, j * (cols // 4)),
+                              (rows, cols // 4), (cols, 1), nat.BF16, nat.BF16))
+    table = nat.Table.create(np.stack(descs), upload=False)
+    table.optimize_range(0, 4)
+    run, row = table.tiles()
+    o_run, o_row = table.ordered_tiles(0, 4)
+    assert len(o_run) == len(run) and len(o_row) == len(row) and len(row) > 0
+    key = lambda tiles: sorted(map(bytes, tiles))
+    assert key(o_row) == key(row) and key(o_run) == key(run)
+    unit = 1 << (int(row[0]["meta"]) & 15)
+    first_written = o_row["a"].astype(np.int64) + o_row["c0"].astype(np.int64) * unit
+    assert np.all(np.diff(first_written) >= 0)
+    logical = row["a"].astype(np.int64) + row["c0"].astype(np.int64) * unit
+    assert not np.all(np.diff(logical) >= 0)  # bucket order is not write order here
+    with pytest.raises(nat.EthaNativeError, match="not been optimized"):
+        table.ordered_tiles(0, 2)

@@ -81,6 +81,8 @@ def _unit_positions(run_tiles, row_tiles):
 def execute(table, arena: HostArena, direction: str, first: int = 0, count: int | None = None,
             peers: np.ndarray | None = None) -> None:
     """Run chunks [first, first+count) of a table on the host. direction: 'pack' | 'unpack' | 'selfcopy'."""
+    global THREADS
+    THREADS = int(table.info().tile_threads)
     run_tiles, row_tiles = table.tiles()
     run_begin, row_begin = table.ranges()
     if count is None:
