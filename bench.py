@@ -36,6 +36,7 @@ def parse_args():
     ap.add_argument("--warmup", type=int, default=3)
     ap.add_argument("--workload", default="llama3_8b_fsdp8_to_tp2")
     ap.add_argument("--per-bucket", action="store_true", help="one launch per bucket instead of one per run of buckets")
+    ap.add_argument("--fanout", type=int, default=1, help="side streams for per-bucket launches (with --per-bucket)")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--cpu-layers", type=int, default=2, help="layers of the workload the CPU baseline sample covers")
     ap.add_argument("--calibration-copy", action="store_true",
@@ -117,7 +118,7 @@ def main():
     merge = not args.per_bucket
     # plan (compiles the tile programs) + warm-up
     for _ in range(max(args.warmup, 1)):
-        job.run(merge_launches=merge)
+        job.run(merge_launches=merge, fanout=args.fanout)
     setup_s = time.time() - t0
 
     S = job.payload_bytes()
@@ -174,9 +175,9 @@ def main():
     wall0 = time.perf_counter()
     for k in range(args.steps):
         ev[k][0].record(stream)
-        job.run_send(merge)
+        job.run_send(merge, args.fanout)
         ev[k][1].record(stream)
-        job.run_recv(merge)
+        job.run_recv(merge, args.fanout)
         ev[k][2].record(stream)
     torch.cuda.synchronize()
     wall = time.perf_counter() - wall0
@@ -215,6 +216,7 @@ def main():
             "payload_bytes": S,
             "bucket_bytes": bucket,
             "launch_granularity": "run of buckets" if merge else "bucket",
+            "fanout_streams": args.fanout,
             **job.counts(),
         },
         "device_ms_per_step": round(dev_ms, 4),

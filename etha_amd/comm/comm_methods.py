@@ -120,32 +120,71 @@ class TransferPlan:
                 merged.append([kind, first, count, [slot]])
         return [(k, f, c, tuple(s)) for k, f, c, s in merged]
 
-    def run(self, stream: int | None = None, merge_launches: bool = False) -> None:
+    def run(self, stream: int | None = None, merge_launches: bool = False, fanout: int = 1) -> None:
+        """Enqueue this bucket list's launches.
+
+        ``fanout > 1`` spreads the launches of independent buckets over that many side streams,
+        forked from and joined back into the current stream with events, so that the tail of one
+        bucket's kernel overlaps the head of the next (a single stream serialises kernels).  Buckets
+        that share a pool slot (a staged self-copy's pack and unpack) stay on one stream, in order.
+        """
         if self.device is None:
+            return
+        steps = self.merged_steps if merge_launches else [(k, f, c, (s,)) for k, f, c, s in self.steps]
+        if fanout > 1 and stream is None and len(steps) > 1:
+            self._run_fanout(steps, fanout)
             return
         if stream is None:
             stream = torch.cuda.current_stream(self.device).cuda_stream
-        steps = self.merged_steps if merge_launches else [(k, f, c, (s,)) for k, f, c, s in self.steps]
         with torch.cuda.device(self.device):
-            for kind, first, count, slots in steps:
-                if kind == _PACK:
-                    self.send_table.pack(first, count, stream)
-                elif kind == _REDUCE:
-                    self.send_table.reduce_pack(first, count, stream)
-                elif kind == _UNPACK:
-                    for s in slots:
-                        if s is not None and s.filled == 0:
-                            raise RuntimeError(
-                                "recv bucket runs before its send bucket was ever packed "
-                                "(a real wire would block here)"
-                            )
-                    self.recv_table.unpack(first, count, stream)
-                else:
-                    self.local_table.selfcopy(first, count, stream)
-                if kind in (_PACK, _REDUCE):
-                    for s in slots:
-                        if s is not None:
-                            s.filled += 1
+            self._enqueue(steps, lambda i, slots: stream)
+
+    def _run_fanout(self, steps, fanout: int) -> None:
+        main = torch.cuda.current_stream(self.device)
+        side = self.wire.side_streams(self.device, fanout)
+        fork = torch.cuda.Event()
+        fork.record(main)
+        for s in side:
+            s.wait_event(fork)
+        lane_of_slot: dict[int, int] = {}
+
+        def pick(i, slots):
+            key = id(slots[0]) if slots and slots[0] is not None else None
+            if key is not None and key in lane_of_slot:
+                lane = lane_of_slot[key]
+            else:
+                lane = i % len(side)
+                if key is not None:
+                    lane_of_slot[key] = lane
+            return side[lane].cuda_stream
+
+        with torch.cuda.device(self.device):
+            self._enqueue(steps, pick)
+        for s in side:
+            done = torch.cuda.Event()
+            done.record(s)
+            main.wait_event(done)
+
+    def _enqueue(self, steps, stream_of) -> None:
+        for i, (kind, first, count, slots) in enumerate(steps):
+            stream = stream_of(i, slots)
+            if kind == _PACK:
+                self.send_table.pack(first, count, stream)
+            elif kind == _REDUCE:
+                self.send_table.reduce_pack(first, count, stream)
+            elif kind == _UNPACK:
+                for s in slots:
+                    if s is not None and s.filled == 0:
+                        raise RuntimeError(
+                            "recv bucket runs before its send bucket was ever packed (a real wire would block here)"
+                        )
+                self.recv_table.unpack(first, count, stream)
+            else:
+                self.local_table.selfcopy(first, count, stream)
+            if kind in (_PACK, _REDUCE):
+                for s in slots:
+                    if s is not None:
+                        s.filled += 1
 
     def payload_bytes(self) -> dict[str, int]:
         out = {}
@@ -161,13 +200,15 @@ def bucket_comm(
     wire=None,
     merge_launches: bool = False,
     synchronize: bool = True,
+    fanout: int = 1,
 ) -> None:
     """Run the bucket pipeline for one rank's buckets.
 
     ``max_in_flight`` is accepted for compatibility; every bucket owns a persistent pool slot, so
     there is nothing to throttle.  The keyword-only arguments are additions: ``wire`` selects the
     loopback wire (default: the process-wide one), ``merge_launches`` fuses consecutive buckets of
-    one kind into a single launch, ``synchronize=False`` leaves the stream un-synchronised.
+    one kind into a single launch, ``synchronize=False`` leaves the stream un-synchronised, ``fanout``
+    spreads per-bucket launches over that many side streams (see :meth:`TransferPlan.run`).
     """
     del max_in_flight
     if wire is None:
@@ -177,6 +218,6 @@ def bucket_comm(
     if not buckets:
         return
     plan = wire.plan(buckets)
-    plan.run(merge_launches=merge_launches)
+    plan.run(merge_launches=merge_launches, fanout=fanout)
     if synchronize and plan.device is not None:
         torch.cuda.current_stream(plan.device).synchronize()

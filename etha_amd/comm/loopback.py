@@ -74,6 +74,7 @@ class LoopbackWire:
         self.pool: BucketPool | None = None
         self._sent: dict[tuple, list[tuple[Slot, tuple[int, ...]]]] = defaultdict(list)
         self._plans: dict[tuple, object] = {}
+        self._side_streams: list[torch.cuda.Stream] = []
 
     def _pool_for(self, device: torch.device) -> BucketPool:
         if self.pool is None:
@@ -113,6 +114,12 @@ class LoopbackWire:
 
     def private_slot(self, nbytes: int, device: torch.device) -> Slot:
         return self._pool_for(device).alloc(nbytes)
+
+    def side_streams(self, device: torch.device, n: int) -> list:
+        """``n`` extra streams of default priority, created on first use and kept."""
+        while len(self._side_streams) < n:
+            self._side_streams.append(torch.cuda.Stream(device=device))
+        return self._side_streams[:n]
 
     # -- plan cache -----------------------------------------------------------------------------
     def plan(self, buckets: list[Bucket]):

@@ -77,6 +77,7 @@ constexpr uint32_t kMetaDtaShift = 8;   // 4 bits: ETHA_* dtype, a side
 constexpr uint32_t kMetaDtbShift = 12;  // 4 bits: ETHA_* dtype, b side
 constexpr uint32_t kMetaCvt = 1u << 16; // converting move (else byte move)
 constexpr uint32_t kMetaVec = 1u << 17; // converting move handles the full vector (else 1 element)
+constexpr uint32_t kMetaSkew = 1u << 18; // byte move of 16-byte units whose a-side address is not 16-byte aligned
 
 // ---- typed vector access ----------------------------------------------------------------------
 typedef uint32_t u32x2 __attribute__((ext_vector_type(2)));
@@ -97,6 +98,9 @@ template <typename V>
 __device__ __forceinline__ void copy_as(uint64_t src, uint64_t dst) {
   st_stream<V>(dst, ld_stream<V>(src));
 }
+// 16-byte access at any byte address (the device runs in unaligned-access mode; consecutive
+// work-items still cover one contiguous byte range, so the memory system sees full lines)
+typedef u32x4 u32x4_any __attribute__((aligned(1)));
 
 // N elements of storage type T as one naturally aligned vector.
 template <typename T, int N>
@@ -180,6 +184,13 @@ template <bool REV>
 __device__ __forceinline__ void move_unit(uint32_t meta, uint64_t a, uint64_t b) {
   const uint64_t src = REV ? b : a, dst = REV ? a : b;
   if (!(meta & kMetaCvt)) {
+    if (meta & kMetaSkew) {  // a side unaligned, b side aligned
+      if (REV)
+        __builtin_nontemporal_store(ld_stream<u32x4>(b), reinterpret_cast<ETHA_GLOBAL u32x4_any*>(a));
+      else
+        st_stream<u32x4>(b, __builtin_nontemporal_load(reinterpret_cast<const ETHA_GLOBAL u32x4_any*>(a)));
+      return;
+    }
     switch (meta & 15u) {
       case 4: copy_as<u32x4>(src, dst); break;
       case 3: copy_as<u32x2>(src, dst); break;
@@ -562,6 +573,61 @@ int compile_pair(Builder& bld, uint32_t idx, const Region& A0, const Region& B0,
   meta |= ((uint32_t)ua_log2 << kMetaUaShift) | ((uint32_t)ub_log2 << kMetaUbShift) | (dta << kMetaDtaShift) |
           (dtb << kMetaDtbShift);
   const uint64_t ua = 1ull << ua_log2, ub = 1ull << ub_log2;
+
+  // Skewed byte moves: the two sides disagree on their position inside a 16-byte vector (typically
+  // a chunk that follows an odd-sized one in an un-padded bucket).  Long runs are peeled per run so
+  // that the b side is 16-byte aligned: a head and a tail of < 16 bytes go through narrow tiles, the
+  // body moves in 16-byte units whose a-side access is unaligned.
+  constexpr uint64_t kSkewMinRunBytes = 512;
+  if (!cvt && !red.n_peers && ua_log2 < 4 && run_elems * (uint64_t)esa >= kSkewMinRunBytes) {
+    const uint64_t run_bytes = run_elems * (uint64_t)esa;
+    const uint32_t dt_bits = (dta << kMetaDtaShift) | (dtb << kMetaDtbShift);
+    const uint32_t body_meta = dt_bits | (4u << kMetaUaShift) | (4u << kMetaUbShift) | kMetaSkew;
+    auto narrow = [&](uint64_t a, uint64_t b, uint64_t bytes) {  // bytes < 16
+      if (!bytes) return;
+      uint64_t m = a | b | bytes;
+      int v = 3;
+      while (v > 0 && (m & ((1ull << v) - 1))) v--;
+      RunTile t;
+      t.a = a;
+      t.b = b;
+      t.n = (uint32_t)(bytes >> v);
+      t.meta = dt_bits | ((uint32_t)v << kMetaUaShift) | ((uint32_t)v << kMetaUbShift);
+      bld.run.push_back(t);
+    };
+    int64_t pos[ETHA_MAX_NDIM] = {0};
+    uint64_t off_a = 0, off_b = 0;
+    while (true) {
+      const uint64_t a0 = A0.base + off_a, b0 = B0.base + off_b;
+      const uint64_t head = (16 - (b0 & 15)) & 15;
+      const uint64_t body_units = (run_bytes - head) / 16;
+      const uint64_t tail = run_bytes - head - body_units * 16;
+      narrow(a0, b0, head);
+      for (uint64_t q = 0; q < body_units; q += kTileThreads) {
+        RunTile t;
+        t.a = a0 + head + q * 16;
+        t.b = b0 + head + q * 16;
+        t.n = (uint32_t)(body_units - q < kTileThreads ? body_units - q : kTileThreads);
+        t.meta = body_meta;
+        bld.run.push_back(t);
+      }
+      narrow(a0 + head + body_units * 16, b0 + head + body_units * 16, tail);
+      if (bld.run.size() + bld.row.size() > kMaxTiles)
+        return fail(ETHA_ERR_UNSUPPORTED, "tile program too large (> %llu tiles)", (unsigned long long)kMaxTiles);
+      int d = k - 1;
+      for (; d >= 0; d--) {
+        pos[d]++;
+        off_a += (uint64_t)sa[d];
+        off_b += (uint64_t)sb[d];
+        if (pos[d] < n[d]) break;
+        off_a -= (uint64_t)(sa[d] * n[d]);
+        off_b -= (uint64_t)(sb[d] * n[d]);
+        pos[d] = 0;
+      }
+      if (d < 0) break;
+    }
+    return ETHA_OK;
+  }
 
   // 5. tiles.  Long or 256-multiple rows (and single runs) become run tiles; other shapes become
   //    row tiles over the innermost remaining dim; dims further out are unrolled here.

@@ -198,18 +198,18 @@ class ReshardJob:
         return False
 
     # ------------------------------------------------------------------------------------------
-    def run_send(self, merge_launches: bool = False) -> None:
+    def run_send(self, merge_launches: bool = False, fanout: int = 1) -> None:
         for buckets in self.send_buckets.values():
-            bucket_comm(buckets, wire=self.wire, merge_launches=merge_launches, synchronize=False)
+            bucket_comm(buckets, wire=self.wire, merge_launches=merge_launches, synchronize=False, fanout=fanout)
 
-    def run_recv(self, merge_launches: bool = False) -> None:
+    def run_recv(self, merge_launches: bool = False, fanout: int = 1) -> None:
         for buckets in self.recv_buckets.values():
-            bucket_comm(buckets, wire=self.wire, merge_launches=merge_launches, synchronize=False)
+            bucket_comm(buckets, wire=self.wire, merge_launches=merge_launches, synchronize=False, fanout=fanout)
 
-    def run(self, merge_launches: bool = False, synchronize: bool = True) -> None:
+    def run(self, merge_launches: bool = False, synchronize: bool = True, fanout: int = 1) -> None:
         """One transfer: every source rank packs (and self-copies), then every target rank unpacks."""
-        self.run_send(merge_launches)
-        self.run_recv(merge_launches)
+        self.run_send(merge_launches, fanout)
+        self.run_recv(merge_launches, fanout)
         if synchronize:
             torch.cuda.current_stream(self.device).synchronize()
 

@@ -21,7 +21,7 @@ pytestmark = pytest.mark.gpu
 CASES = load_cases()
 
 
-# ---- BASELINE config 1 and the reference's own case tables --------------------------------------
+# ---- the single-fp32-tensor config and the reference's own case tables ----------------------------
 
 def test_config1_fp32_shard0_to_shard1(gpu_device):
     """fp32 [1024,1024] uniform(-1,1) seed 0; (2,) Shard(0) -> (4,) Shard(1); full reassembly."""
@@ -347,3 +347,40 @@ def test_llama3_8b_full_size_properties(gpu_device):
         d[8].zero_()
     job.run(merge_launches=False)  # second transfer, one launch per bucket this time
     check()
+
+
+def test_per_bucket_launches_on_side_streams(gpu_device):
+    """Fan-out over side streams (fork/join with events) gives the same bytes as one stream."""
+    specs, targets, _ = workloads.llama3_8b_fsdp8_to_tp2(n_layers=3, hidden=256, inter=896, kv=64, vocab=2056)
+    gpu_job = ReshardJob(specs, device=gpu_device, bucket_size=32 * 1024, target_ranks=targets, keep_globals=True, fill=cpu_fill)
+    cpu_job = ReshardJob(specs, device="cpu", bucket_size=32 * 1024, target_ranks=targets, keep_globals=True, fill=cpu_fill)
+    run_oracle(cpu_job)
+    for fanout in (3, 1, 4):
+        for d in gpu_job.target_locals:
+            for t in d.values():
+                t.zero_()
+        gpu_job.run(merge_launches=False, fanout=fanout)
+        for i, spec in enumerate(specs):
+            for r, t in gpu_job.target_locals[i].items():
+                assert_bit_equal(t, cpu_job.target_locals[i][r], f"{spec.name} rank {r} fanout {fanout}")
+
+
+def test_skewed_buckets_large(gpu_device):
+    """An odd-sized first chunk skews every later chunk of its bucket; long runs then move as 16-byte
+    units with an unaligned tensor-side access.  Both directions, contiguous and strided rows."""
+    one = (mesh_of(0, [1]), (Replicate(),), mesh_of(1, [1]), (Replicate(),))
+    specs = [
+        TensorSpec("odd", (7,), *one, torch.bfloat16, seed=1, dist="bits"),            # 14 bytes
+        TensorSpec("big", (1 << 20,), *one, torch.bfloat16, seed=2, dist="bits"),       # skew 14
+        TensorSpec("rows", (300, 1000), mesh_of(0, [1]), (Replicate(),), mesh_of(1, [2]), (Shard(1),), torch.bfloat16,
+                   seed=3, dist="bits"),                                               # 1000-byte strided rows
+    ]
+    job, _ = gpu_vs_oracle(specs, gpu_device, 1 << 30)
+    specs32 = [
+        TensorSpec("odd", (3,), *one, torch.float32, seed=5, dist="bits"),             # 12 bytes: dword-aligned skew
+        TensorSpec("f32", (257, 513), *one, torch.float32, seed=4, dist="bits"),
+    ]
+    gpu_vs_oracle(specs32, gpu_device, 1 << 30)
+    plan = job.wire.plan(job.send_buckets[0])
+    run, _ = plan.send_table.tiles()
+    assert ((run["meta"] & (1 << 18)) != 0).sum() > 0  # the skew path was really taken

@@ -44,6 +44,10 @@ GEOMETRIES = [
     ((64, 256), None, (0, 128), (64, 128), nat.F64, nat.F16, 0),
     ((64, 256), None, (0, 128), (64, 128), nat.F16, nat.BF16, 0),
     ((3,), None, (0,), (3,), nat.F32, nat.F32, 0),
+    ((40000,), None, (3,), (39990,), nat.BF16, nat.BF16, 0),             # long run, the two sides skewed
+    ((64, 1024), None, (0, 5), (64, 777), nat.BF16, nat.BF16, 2),        # skewed rows of 1554 bytes
+    ((9000,), None, (1,), (8990,), nat.B8, nat.B8, 1),                   # byte elements, odd everything
+    ((30, 600), None, (0, 1), (30, 599), nat.F32, nat.F32, 4),           # dword-aligned skew
     ((5, 0, 7), None, (0, 0, 0), (5, 0, 7), nat.F32, nat.F32, 0),        # empty chunk
 ]
 
@@ -98,6 +102,22 @@ def test_pack_and_unpack_tiles_match_oracle(geom):
     assert co.lib().oracle_unpack_bucket(oc2, 1, want_bucket.ctypes.data, scratch.ctypes.data) == 0
     assert np.array_equal(arena.bytes_at(t2_addr, pn * es), want_t2), "unpack result / untouched bytes differ"
     assert arena.writes.max(initial=0) <= 1 and int(arena.writes.sum()) == cn * es
+
+
+def test_skewed_chunks_use_wide_units():
+    """A long chunk whose two sides are skewed must not fall back to element-sized units."""
+    n, es = 1 << 20, 2
+    arena = HostArena(3 * n * es + 65536)
+    t = arena.alloc(n * es)
+    b = arena.alloc(n * es + 64)
+    d = _mk_desc(t, t, t + n * es, b + 6, b, b + n * es + 64, (0,), (n,), (1,), nat.BF16, nat.BF16)
+    table = nat.Table.create(d.reshape(1), upload=False)
+    run, row = table.tiles()
+    body = run[(run["meta"] & (1 << 18)) != 0]
+    assert len(row) == 0 and len(body) >= 1
+    assert int(body["n"].sum()) * 16 >= n * es - 32  # all but head and tail move as 16-byte units
+    assert len(run) - len(body) <= 2
+    assert np.all(body["b"] % 16 == 0) and np.all(body["a"] % 16 == 10)
 
 
 def test_bucket_ranges_and_many_chunks():
