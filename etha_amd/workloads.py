@@ -29,7 +29,8 @@ def single_fp32_shard0_to_shard1():
 
 
 def llama3_8b_fsdp8_to_tp2(n_layers: int = 32, with_embeddings: bool = True, dtype=torch.bfloat16,
-                           hidden: int = 4096, inter: int = 14336, kv: int = 1024, vocab: int = 128256):
+                           hidden: int = 4096, inter: int = 14336, kv: int = 1024, vocab: int = 128256,
+                           target_dtype=None):
     """Llama-3-8B weight set, FSDP Shard(0) over 8 ranks -> TP=2; one TP rank's share.
 
     Column-parallel (q/k/v/gate/up/embed/lm_head): Shard(0) -> Shard(0).  Row-parallel (o/down):
@@ -41,7 +42,7 @@ def llama3_8b_fsdp8_to_tp2(n_layers: int = 32, with_embeddings: bool = True, dty
     specs: list[TensorSpec] = []
 
     def add(name, shape, tgt_pl):
-        specs.append(TensorSpec(name, shape, src, (Shard(0),), tgt, tgt_pl, dtype, seed=len(specs)))
+        specs.append(TensorSpec(name, shape, src, (Shard(0),), tgt, tgt_pl, dtype, target_dtype, seed=len(specs)))
 
     if with_embeddings:
         add("embed_tokens", (vocab, hidden), col)
@@ -97,9 +98,16 @@ def moe_experts_and_uneven_vocab(n_experts: int = 8, hidden: int = 4096, inter: 
     return specs, [0], 64 * MIB
 
 
+def llama3_8b_fsdp8_to_tp2_fp32_to_bf16():
+    """Same layouts with fp32 source shards and bf16 target shards (trainer master weights -> serving
+    weights): the wire dtype is bf16, so the pack kernel converts."""
+    return llama3_8b_fsdp8_to_tp2(dtype=torch.float32, target_dtype=torch.bfloat16)
+
+
 WORKLOADS = {
     "single_fp32_shard0_to_shard1": single_fp32_shard0_to_shard1,
     "llama3_8b_fsdp8_to_tp2": llama3_8b_fsdp8_to_tp2,
+    "llama3_8b_fsdp8_to_tp2_fp32_to_bf16": llama3_8b_fsdp8_to_tp2_fp32_to_bf16,
     "many_small_2d_to_replicate": many_small_2d_to_replicate,
     "partial4_to_shard2": partial4_to_shard2,
     "moe_experts_and_uneven_vocab": moe_experts_and_uneven_vocab,
