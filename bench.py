@@ -39,6 +39,7 @@ def parse_args():
     ap.add_argument("--workload", default="llama3_8b_fsdp8_to_tp2")
     ap.add_argument("--per-bucket", action="store_true", help="one launch per bucket instead of one per run of buckets")
     ap.add_argument("--fanout", type=int, default=1, help="side streams for per-bucket launches (with --per-bucket)")
+    ap.add_argument("--graph", action="store_true", help="replay the step from a captured HIP graph (whole step timed)")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--cpu-layers", type=int, default=2, help="layers of the workload the CPU baseline sample covers")
     ap.add_argument("--calibration-copy", action="store_true",
@@ -173,18 +174,31 @@ def main():
 
     stream = torch.cuda.current_stream(dev)
     ev = [[torch.cuda.Event(enable_timing=True) for _ in range(3)] for _ in range(args.steps)]
+    graph = None
+    if args.graph:
+        graph = job.capture(merge_launches=merge)
+        graph.replay()
     torch.cuda.synchronize()
     wall0 = time.perf_counter()
     for k in range(args.steps):
         ev[k][0].record(stream)
-        job.run_send(merge, args.fanout)
-        ev[k][1].record(stream)
-        job.run_recv(merge, args.fanout)
+        if graph is not None:
+            graph.replay()
+            ev[k][1].record(stream)
+        else:
+            job.run_send(merge, args.fanout)
+            ev[k][1].record(stream)
+            job.run_recv(merge, args.fanout)
         ev[k][2].record(stream)
     torch.cuda.synchronize()
     wall = time.perf_counter() - wall0
     pack_ms = [ev[k][0].elapsed_time(ev[k][1]) for k in range(args.steps)]
     unpack_ms = [ev[k][1].elapsed_time(ev[k][2]) for k in range(args.steps)]
+    if graph is not None:  # a replayed graph is one unit: split the step time by algorithmic bytes
+        whole = [p + u for p, u in zip(pack_ms, unpack_ms)]
+        share = pack_bytes / max(pack_bytes + unpack_bytes, 1)
+        pack_ms = [w * share for w in whole]
+        unpack_ms = [w * (1 - share) for w in whole]
     step_ms = wall * 1e3 / args.steps
     pack_avg, unpack_avg = sum(pack_ms) / len(pack_ms), sum(unpack_ms) / len(unpack_ms)
     dev_ms = pack_avg + unpack_avg
@@ -219,6 +233,7 @@ def main():
             "bucket_bytes": bucket,
             "launch_granularity": "run of buckets" if merge else "bucket",
             "fanout_streams": args.fanout,
+            "hip_graph": bool(args.graph),
             **job.counts(),
         },
         "device_ms_per_step": round(dev_ms, 4),

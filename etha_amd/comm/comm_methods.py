@@ -139,6 +139,15 @@ class TransferPlan:
         with torch.cuda.device(self.device):
             self._enqueue(steps, lambda i, slots: stream)
 
+    def run_kinds(self, kinds: tuple[str, ...]) -> None:
+        """Enqueue only the steps of the given kinds on the current stream (single-bucket protocol)."""
+        if self.device is None:
+            return
+        stream = torch.cuda.current_stream(self.device).cuda_stream
+        steps = [(k, f, c, (s,)) for k, f, c, s in self.steps if k in kinds]
+        with torch.cuda.device(self.device):
+            self._enqueue(steps, lambda i, slots: stream)
+
     def _run_fanout(self, steps, fanout: int) -> None:
         main = torch.cuda.current_stream(self.device)
         side = self.wire.side_streams(self.device, fanout)

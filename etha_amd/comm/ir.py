@@ -225,3 +225,30 @@ class Bucket:
             f"Bucket({self.transport.name[:3]}/{role}, n={len(self.chunks)}, bytes={self.total_bytes}, "
             f"src={self.src_rank}->{self.dst_ranks})"
         )
+
+    # -- the reference's per-bucket protocol (ir.py:229-310), on top of the compiled plan -----------
+    # ``bucket_comm`` is the normal entry; these exist for code that drives single buckets itself.
+    def _plan(self, wire=None):
+        if wire is None:
+            from .loopback import default_wire
+
+            wire = default_wire()
+        return wire.plan([self])
+
+    def prepare(self, wire=None) -> None:
+        """Source bucket: enqueue its pack (or reduce-pack / self-copy) launch.  Target bucket: nothing
+        to do, its bytes arrive in the producer's pool slot (``Bucket.prepare``, ``ir.py:229-264``)."""
+        self._plan(wire).run_kinds(("pack", "reduce_pack", "selfcopy"))
+
+    def launch(self) -> bool:
+        """The wire step.  Always ready: the loopback hands the pool slot over in place
+        (``Bucket.launch``, ``ir.py:266-284``)."""
+        return True
+
+    def is_complete(self) -> bool:
+        return True
+
+    def finalize(self, wire=None) -> None:
+        """Target bucket (and staged self-copy): enqueue its unpack launch (``Bucket.finalize``,
+        ``ir.py:300-310``)."""
+        self._plan(wire).run_kinds(("unpack",))

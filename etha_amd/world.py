@@ -213,6 +213,15 @@ class ReshardJob:
         if synchronize:
             torch.cuda.current_stream(self.device).synchronize()
 
+    def capture(self, merge_launches: bool = True):
+        """Record one transfer into a HIP graph and return it; ``graph.replay()`` then re-issues every
+        launch of the transfer with one call.  The plans must exist (run once eagerly first): planning
+        allocates and uploads, which cannot be captured.  Useful when a transfer is launch-bound."""
+        graph = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(graph):
+            self.run(merge_launches=merge_launches, synchronize=False)
+        return graph
+
     def payload_bytes(self) -> int:
         """Bytes the measured target ranks end up holding, in wire dtype (the reference's
         effective-throughput numerator, ``bench/transfer_benchmark.py:339-360``)."""
