@@ -41,14 +41,15 @@ def parse_args():
     ap.add_argument("--fanout", type=int, default=1, help="side streams for per-bucket launches (with --per-bucket)")
     ap.add_argument("--graph", action="store_true", help="replay the step from a captured HIP graph (whole step timed)")
     ap.add_argument("--no-cpu-baseline", action="store_true")
-    ap.add_argument("--cpu-layers", type=int, default=2, help="layers of the workload the CPU baseline sample covers")
+    ap.add_argument("--cpu-layers", type=int, default=8, help="layers of the workload the CPU baseline sample covers")
+    ap.add_argument("--cpu-seconds", type=float, default=15.0, help="CPU work the baseline leg is bounded to")
     ap.add_argument("--calibration-copy", action="store_true",
                     help="after the timed region run three plain 1 GiB torch copies (known traffic, for scaling "
                          "hardware counters collected with rocprofv3 --pmc)")
     return ap.parse_args()
 
 
-def cpu_baseline(workload: str, layers: int):
+def cpu_baseline(workload: str, layers: int, seconds: float):
     """The oracle's op-for-op restatement of the reference path, timed on this host's cores."""
     import torch
 
@@ -81,8 +82,8 @@ def cpu_baseline(workload: str, layers: int):
 
     one_pass()
     times = []
-    t_end = time.perf_counter() + 20.0
-    while len(times) < 10 and (len(times) < 3 or time.perf_counter() < t_end):
+    t_end = time.perf_counter() + seconds
+    while len(times) < 3 or (time.perf_counter() < t_end and len(times) < 200):
         t0 = time.perf_counter()
         one_pass()
         times.append(time.perf_counter() - t0)
@@ -93,7 +94,8 @@ def cpu_baseline(workload: str, layers: int):
         "unit": "GB/s",
         "cores": torch.get_num_threads(),
         "kind": "port",
-        "sample": f"{sample}; {payload} payload bytes per pass, median of {len(times)} passes",
+        "sample": f"{sample}; {payload} payload bytes per pass, median of {len(times)} passes "
+                  f"({sum(times):.1f} s of CPU work)",
         "host_cpus": os.cpu_count(),
     }
 
@@ -264,7 +266,7 @@ def main():
         torch.cuda.synchronize()
         out["calibration_copy"] = {"bytes_read": 1 << 30, "bytes_written": 1 << 30, "launches": 3}
     if not args.no_cpu_baseline:
-        out["cpu_baseline"] = cpu_baseline(args.workload, args.cpu_layers)
+        out["cpu_baseline"] = cpu_baseline(args.workload, args.cpu_layers, args.cpu_seconds)
     print(json.dumps(out))
 
 

@@ -97,12 +97,19 @@ class TransferPlan:
                     recv.add_chunk(c, c.tensor, c.dst_slice, slot, off, reduce=False)
                 self.steps.append((_UNPACK, first, len(bucket.chunks), slot))
         self._keepalive = send.keepalive + recv.keepalive + local.keepalive
-        self.send_table = send.build()
-        self.recv_table = recv.build()
-        self.local_table = local.build()
         self.merged_steps = self._merge(self.steps)
-        # merged unpack / self-copy launches cover several buckets: let the library order their tiles by
-        # written address, so that rows of one tensor arriving through different buckets are written together
+        self.send_table = self.recv_table = self.local_table = None
+        if self.device is None:
+            return
+        with torch.cuda.device(self.device):  # the tile programs are uploaded to the tensors' device
+            self.send_table = send.build()
+            self.recv_table = recv.build()
+            self.local_table = local.build()
+            self._optimize_merged_ranges()
+
+    def _optimize_merged_ranges(self) -> None:
+        """Merged unpack / self-copy launches cover several buckets: let the library order their tiles by
+        written address, so that rows of one tensor arriving through different buckets are written together."""
         for kind, first, count, slots in self.merged_steps:
             if len(slots) > 1 and kind == _UNPACK:
                 self.recv_table.optimize_range(first, count)
