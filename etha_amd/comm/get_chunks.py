@@ -18,6 +18,9 @@ Deliberate differences:
   chunk keeps only the remote destinations and disappears when none is left.  The LOCAL chunk
   reads ``source_tensor`` (``Chunk.src_tensor``) and writes ``target_tensor``.
 * broadcast sub-groups need no pre-creation (``get_chunks.py:48-55``): there is no process group.
+* Receive chunks of a Partial source carry the producer's Partial signature
+  (``Chunk.source_partial_signature``), so that sender and receiver split a wire key's chunks into the same
+  buckets when a batch mixes Partial and plain tensors.
 * A role whose tensor is not given produces no chunks: without ``source_tensor`` the rank does not act
   as a source, without ``target_tensor`` not as a destination (the reference would build chunks around
   ``None`` and fail in ``Chunk.__post_init__``, ``ir.py:87-89``).
@@ -62,6 +65,25 @@ def _side_slicers(tensor, num_slicers, this_mesh, this_pl, other_mesh, other_pl,
                 "does not define an uneven split for it (the reference would silently drop the tail)"
             )
     return ext, get_slicer_tuples(shape, ext)
+
+
+def _partial_signature(m2m: M2MMap, src_rank: int) -> tuple:
+    """``((member ranks), op)`` of the Partial reduction ``src_rank`` takes part in, as one group over the
+    whole connected component - the form ``etha_amd.world.create_partial_groups`` builds on the sending side."""
+    if not m2m.source_partial_reductions or m2m.source_mesh is None:
+        return ()
+    import numpy as np
+
+    mesh = np.asarray(m2m.source_mesh)
+    where = np.argwhere(mesh == src_rank)
+    if len(where) != 1:
+        return ()
+    index: list = [int(c) for c in where[0]]
+    for mesh_dim, _ in m2m.source_partial_reductions:
+        index[mesh_dim] = slice(None)
+    ranks = tuple(sorted(int(r) for r in np.asarray(mesh[tuple(index)]).reshape(-1)))
+    ops = {op for _, op in m2m.source_partial_reductions}
+    return ((ranks, ops.pop()),) if len(ops) == 1 else ()
 
 
 def _shape_of(slices: tuple[slice, ...]) -> tuple[int, ...]:
@@ -164,6 +186,7 @@ def m2m_to_chunks(
                         tensor=target_tensor,
                         transfer_dtype=transfer_dtype,
                         rank=rank,
+                        source_partial_signature=_partial_signature(m2m, src_rank),
                     )
                 )
     return chunks

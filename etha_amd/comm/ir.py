@@ -109,6 +109,10 @@ class Chunk:
     # additions
     rank: int | None = None  # rank this chunk was materialised for
     src_tensor: torch.Tensor | None = None  # LOCAL chunks: tensor that src_slice indexes (default: tensor)
+    # consume-only chunks: the Partial signature of the producing side, so that both ends of a wire split
+    # their buckets the same way (the reference's receive chunks carry no Partial information, which makes
+    # sender and receiver bundle differently when a batch mixes Partial and plain tensors)
+    source_partial_signature: tuple = ()
 
     def __post_init__(self) -> None:
         if self.transfer_dtype is None and self.tensor is not None:
@@ -123,7 +127,7 @@ class Chunk:
     @property
     def partial_signature(self) -> tuple:
         if not self.source_partial_groups:
-            return ()
+            return tuple(self.source_partial_signature)
         return tuple((g.ranks, op) for g, op in self.source_partial_groups)
 
     @property
@@ -136,9 +140,10 @@ class Chunk:
         equal groups either way).
         """
         cell_key: tuple = ()
-        if self.source_partial_groups and not self.dst_ranks:
+        signature = self.partial_signature
+        if signature and not self.dst_ranks:
             cell_key = tuple(self.src_idx)
-        return (self.src_rank, self.dst_ranks, self.partial_signature, cell_key, self.transport)
+        return (self.src_rank, self.dst_ranks, signature, cell_key, self.transport)
 
     @property
     def nbytes(self) -> int:

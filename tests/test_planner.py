@@ -139,3 +139,23 @@ def test_llama3_8b_share_matches_the_published_shape_of_the_workload():
     buckets = chunk_to_bucket_ops(recv, bucket)
     assert sum(b.total_bytes for b in buckets) == 8_030_519_296
     assert all(b.total_bytes < 2 * bucket or len(b.chunks) == 1 for b in buckets)
+
+
+def test_partial_and_plain_tensors_bucket_alike_on_both_ends():
+    """A batch with a Partial-source tensor and a plain tensor between the same ranks: the sender keeps
+    them in different buckets (different reduce signature), so the receiver must too."""
+    from etha_amd.world import create_partial_groups
+
+    plain = get_m2m_map([0, 1], (Shard(0),), [2], (Replicate(),))
+    part = get_m2m_map([0, 1], (Partial(),), [2], (Replicate(),))
+    src_plain = {r: torch.empty(4, 8, device="meta") for r in (0, 1)}
+    src_part = {r: torch.empty(8, 8, device="meta") for r in (0, 1)}
+    tgt = torch.empty(8, 8, device="meta")
+    groups = create_partial_groups([0, 1], part.source_partial_reductions, 0, src_part)
+    send = m2m_to_chunks(plain, 0, source_tensor=src_plain[0]) + m2m_to_chunks(part, 0, source_tensor=src_part[0],
+                                                                             source_partial_groups=groups)
+    recv = m2m_to_chunks(plain, 2, target_tensor=tgt) + m2m_to_chunks(part, 2, target_tensor=tgt)
+    send_b = [b for b in chunk_to_bucket_ops(send, 1 << 30) if b.dst_ranks]
+    recv_b = [b for b in chunk_to_bucket_ops(recv, 1 << 30) if b.src_rank == 0]
+    assert [[c.nbytes for c in b.chunks] for b in send_b] == [[c.nbytes for c in b.chunks] for b in recv_b]
+    assert len(send_b) == 2 and recv_b[1].chunks[0].source_partial_signature == (((0, 1), "sum"),)
