@@ -51,7 +51,7 @@ class TransferPlan:
             if first_tensor is None:
                 raise ValueError(f"{bucket}: chunks without a tensor cannot be executed")
             device = first_tensor.device
-            if device.type != "cuda":
+            if device.type != "cuda" and not getattr(wire, "host_inspection", False):
                 raise RuntimeError(
                     f"{bucket}: tensors live on {device}; this executor only runs on a GPU (there is no CPU path)"
                 )
@@ -101,6 +101,12 @@ class TransferPlan:
         self.send_table = self.recv_table = self.local_table = None
         if self.device is None:
             return
+        if self.device.type != "cuda":  # host inspection: compile the programs, never upload or launch them
+            self.send_table = send.build(upload=False)
+            self.recv_table = recv.build(upload=False)
+            self.local_table = local.build(upload=False)
+            self._optimize_merged_ranges()
+            return
         with torch.cuda.device(self.device):  # the tile programs are uploaded to the tensors' device
             self.send_table = send.build()
             self.recv_table = recv.build()
@@ -137,6 +143,8 @@ class TransferPlan:
         """
         if self.device is None:
             return
+        if self.device.type != "cuda":
+            raise RuntimeError("this plan was compiled for host inspection; the executor only runs on a GPU (there is no CPU path)")
         steps = self.merged_steps if merge_launches else [(k, f, c, (s,)) for k, f, c, s in self.steps]
         if fanout > 1 and stream is None and len(steps) > 1:
             self._run_fanout(steps, fanout)
@@ -150,6 +158,8 @@ class TransferPlan:
         """Enqueue only the steps of the given kinds on the current stream (single-bucket protocol)."""
         if self.device is None:
             return
+        if self.device.type != "cuda":
+            raise RuntimeError("this plan was compiled for host inspection; the executor only runs on a GPU (there is no CPU path)")
         stream = torch.cuda.current_stream(self.device).cuda_stream
         steps = [(k, f, c, (s,)) for k, f, c, s in self.steps if k in kinds]
         with torch.cuda.device(self.device):

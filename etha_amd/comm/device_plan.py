@@ -122,7 +122,7 @@ class DescBuilder:
                 if t.dtype != tensor.dtype or tuple(t.shape) != tuple(tensor.shape) or t.stride() != tensor.stride():
                     raise NotImplementedError("Partial peers must share dtype, shape and strides")
                 if t.device != tensor.device:
-                    raise NotImplementedError("Partial peers must live on the same GPU")
+                    raise NotImplementedError("Partial peers must live on the same device")
             row["n_partials"] = len(tensors)
             row["partial_first"] = len(self.partial_ptrs)
             row["reduce_op"] = nat.REDUCE_OPS[op]
@@ -131,12 +131,12 @@ class DescBuilder:
         self.keepalive.append(tensor)
         self.rows.append(row)
 
-    def build(self) -> nat.Table | None:
+    def build(self, upload: bool = True) -> nat.Table | None:
         if not self.rows:
             return None
         descs = np.stack(self.rows)
         ptrs = np.asarray(self.partial_ptrs, dtype=np.uint64) if self.partial_ptrs else None
-        return nat.Table.create(descs, ptrs, upload=True)
+        return nat.Table.create(descs, ptrs, upload=upload)
 
 
 class SelfCopyBuilder:
@@ -161,10 +161,10 @@ class SelfCopyBuilder:
         self.dst.append(b)
         self.keepalive += [src_t, chunk.tensor]
 
-    def build(self) -> nat.Table | None:
+    def build(self, upload: bool = True) -> nat.Table | None:
         if not self.src:
             return None
-        return nat.Table.create_selfcopy(np.stack(self.src), np.stack(self.dst), upload=True)
+        return nat.Table.create_selfcopy(np.stack(self.src), np.stack(self.dst), upload=upload)
 
 
 def region_hull(tensor, slices: tuple) -> tuple[int, int]:

@@ -68,9 +68,13 @@ def wire_key(bucket: Bucket) -> tuple:
 class LoopbackWire:
     """Process-wide stand-in for the process groups of the reference's executor."""
 
-    def __init__(self, device: torch.device | str | None = None, segment_bytes: int = 1 << 30):
+    def __init__(self, device: torch.device | str | None = None, segment_bytes: int = 1 << 30,
+                 host_inspection: bool = False):
         self.device = torch.device(device) if device is not None else None
         self.segment_bytes = segment_bytes
+        # True: bucket lists on host tensors may be *planned* (tile programs compiled against host
+        # addresses, for checking them on the CPU); they still cannot be run
+        self.host_inspection = host_inspection
         self.pool: BucketPool | None = None
         self._sent: dict[tuple, list[tuple[Slot, tuple[int, ...]]]] = defaultdict(list)
         self._plans: dict[tuple, object] = {}

@@ -1,0 +1,150 @@
+"""Randomised end-to-end check of the host side, on the CPU.
+
+Random meshes, placements, shapes, dtypes, bucket sizes and parent strides go through the product's
+planner and descriptor builder; the native library compiles the tile programs against the live host
+tensors (no upload), and the CPU tile interpreter executes them step by step in the executor's order.
+The result must equal the oracle's restatement of the reference path and the closed-form DTensor slice.
+Everything except the device kernel itself is exercised, with bounds checks, and without a GPU.
+"""
+
+import math
+
+import numpy as np
+import pytest
+import torch
+from torch.distributed.tensor.placement_types import Partial, Replicate, Shard
+
+from etha_amd.comm import LoopbackWire
+from etha_amd.world import ReshardJob, TensorSpec
+
+from helpers import assert_bit_equal, cpu_fill, expected_target, mesh_of, run_oracle
+from tile_interpreter import AbsoluteMemory, execute
+
+FLOATS = [torch.float32, torch.bfloat16, torch.float16, torch.float64]
+
+
+def _random_layout(rng, ndim, allow_partial):
+    mesh_shape = [int(rng.choice([1, 2, 3, 4])) for _ in range(int(rng.integers(1, 4)))]
+    while math.prod(mesh_shape) > 8:
+        mesh_shape[int(rng.integers(len(mesh_shape)))] = 1
+    placements, partial = [], False
+    for _ in mesh_shape:
+        kind = rng.choice(["shard", "rep", "partial"] if allow_partial else ["shard", "rep"], p=None)
+        if kind == "shard":
+            placements.append(Shard(int(rng.integers(ndim))))
+        elif kind == "partial":
+            placements.append(Partial("sum"))
+            partial = True
+        else:
+            placements.append(Replicate())
+    return mesh_shape, tuple(placements), partial
+
+
+def _random_spec(rng, idx, wire_size):
+    ndim = int(rng.integers(1, 4))
+    # Partial sources need a floating dtype of at most 32 bits: only in batches whose wire items are 2 or 4 bytes
+    src_mesh, src_pl, partial = _random_layout(rng, ndim, allow_partial=wire_size in (2, 4) and rng.random() < 0.25)
+    tgt_mesh, tgt_pl, _ = _random_layout(rng, ndim, allow_partial=False)
+    shards = []
+    for d in range(ndim):
+        s = math.prod(m for m, p in zip(src_mesh, src_pl) if isinstance(p, Shard) and p.dim == d)
+        t = math.prod(m for m, p in zip(tgt_mesh, tgt_pl) if isinstance(p, Shard) and p.dim == d)
+        shards.append(math.lcm(s, t))
+    shape = tuple(int(l * rng.integers(1, 7)) for l in shards)
+    shape = shape[:-1] + (shape[-1] * int(rng.choice([1, 1, 8, 19])),)
+    # one wire item size per batch: the reference cannot mix item sizes in a bucket unless every offset
+    # happens to be a multiple of the larger one (its view(dtype) of the bucket slice raises, ir.py:252)
+    pairs = {
+        1: [(torch.int8, torch.int8), (torch.uint8, torch.uint8)],
+        2: [(torch.bfloat16, torch.bfloat16), (torch.float16, torch.float16), (torch.bfloat16, torch.float32),
+            (torch.float32, torch.bfloat16), (torch.float16, torch.float64), (torch.float64, torch.bfloat16),
+            (torch.float16, torch.bfloat16), (torch.float32, torch.float16)],
+        4: [(torch.float32, torch.float32), (torch.int32, torch.int32), (torch.float32, torch.float64),
+            (torch.float64, torch.float32)],
+        8: [(torch.float64, torch.float64), (torch.int64, torch.int64)],
+    }[wire_size]
+    if partial:
+        pairs = [p for p in pairs if p[0] in FLOATS[:3]]
+    sdt, tdt = pairs[int(rng.integers(len(pairs)))]
+    n_src = math.prod(src_mesh)
+    # overlapping rank sets create LOCAL chunks; their wire dtype is the target dtype (as in the reference), so
+    # they stay within the batch's wire item size only when the two dtypes agree
+    overlap = (not partial) and sdt == tdt and rng.random() < 0.4
+    tgt_start = 0 if overlap else n_src
+    return TensorSpec(f"t{idx}", shape, mesh_of(0, src_mesh), src_pl, mesh_of(tgt_start, tgt_mesh), tgt_pl, sdt, tdt,
+                      seed=1000 + idx, std=1.0, dist="normal" if sdt in FLOATS else "bits")
+
+
+def _interpret(job, merged: bool):
+    """What ReshardJob.run would enqueue, executed on the host by the tile interpreter."""
+    plans = [job.wire.plan(b) for b in job.send_buckets.values()] + [job.wire.plan(b) for b in job.recv_buckets.values()]
+    # the span of everything that may legitimately be touched: every shard's storage and the bucket pool
+    ranges = []
+    for d in job.source_locals + job.target_locals:
+        for t in d.values():
+            st = t.untyped_storage()
+            if st.nbytes():
+                ranges.append((st.data_ptr(), st.data_ptr() + st.nbytes()))
+    if job.wire.pool is not None:
+        for seg in job.wire.pool.segments:
+            ranges.append((seg.data_ptr(), seg.data_ptr() + seg.numel()))
+    if not ranges:
+        return
+    lo, hi = min(r[0] for r in ranges), max(r[1] for r in ranges)
+    mem = AbsoluteMemory(lo, hi)
+    for p in plans:
+        steps = p.merged_steps if merged else [(k, f, c, (s,)) for k, f, c, s in p.steps]
+        for kind, first, count, slots in steps:
+            if kind in ("pack", "reduce_pack"):
+                execute(p.send_table, mem, "pack", first, count, peers=_peers_of(p))
+            elif kind == "unpack":
+                execute(p.recv_table, mem, "unpack", first, count, ordered=merged and len(slots) > 1)
+            else:
+                execute(p.local_table, mem, "selfcopy", first, count, ordered=merged and len(slots) > 1)
+
+
+def _peers_of(plan):
+    ptrs = []
+    for b in plan.buckets:
+        if b.chunks and b.is_source and b.chunks[0].source_partial_groups and b.transport.value in ("p2p", "broadcast"):
+            for c in b.chunks:
+                ptrs.extend(t.data_ptr() for t in c.partial_peers()[0])
+    return np.asarray(ptrs, dtype=np.uint64) if ptrs else None
+
+
+@pytest.mark.parametrize("seed", range(150))
+def test_random_batches(seed):
+    rng = np.random.default_rng(seed)
+    wire_size = int(rng.choice([1, 2, 2, 4, 4, 8]))
+    specs = [_random_spec(rng, i, wire_size) for i in range(int(rng.integers(1, 5)))]
+    # all tensors of a batch share rank numbering: re-home each spec's meshes on disjoint or overlapping ranks as drawn
+    bucket_size = [None, 64, 4096, 1 << 20][int(rng.integers(4))]
+    view = None
+    if rng.random() < 0.35:
+        def view(kind, t):  # non-contiguous parents: every local shard is a slice of a wider tensor
+            if t.dim() == 0 or t.numel() == 0:
+                return t
+            shape = list(t.shape)
+            shape[-1] = shape[-1] * 2 + 3
+            wide = torch.zeros(shape, dtype=t.dtype)
+            return wide[..., 1 : 1 + t.shape[-1]]
+    merged = bool(rng.integers(2))
+    job = ReshardJob(specs, device="cpu", bucket_size=bucket_size, keep_globals=True, fill=cpu_fill, local_view=view,
+                     wire=LoopbackWire("cpu", segment_bytes=1 << 22, host_inspection=True))
+    ref = ReshardJob(specs, device="cpu", bucket_size=bucket_size, keep_globals=True, fill=cpu_fill, local_view=view)
+    for a, b in zip(job.source_locals, ref.source_locals):  # Partial sources are drawn per job: make them equal
+        for r in a:
+            b[r].copy_(a[r])
+    src_before = [{r: t.clone() for r, t in d.items()} for d in job.source_locals]
+    _interpret(job, merged)
+    run_oracle(ref)
+    for i, spec in enumerate(specs):
+        for r, t in job.target_locals[i].items():
+            assert_bit_equal(t, ref.target_locals[i][r], f"seed {seed} {spec.name} rank {r} vs oracle")
+            if job.globals_[i] is not None:
+                assert_bit_equal(t, expected_target(spec, job.globals_[i], r), f"seed {seed} {spec.name} rank {r} vs closed form")
+        for r, t in job.source_locals[i].items():
+            if not any(t is x for x in job.target_locals[i].values()):
+                assert_bit_equal(t, src_before[i][r], f"seed {seed} {spec.name} source rank {r} mutated")
+    with pytest.raises(RuntimeError, match="no CPU path"):
+        job.run()

@@ -48,6 +48,23 @@ class HostArena:
         return off
 
 
+class AbsoluteMemory:
+    """The process's own address space as the arena: tiles compiled against live host tensors.
+
+    Only the bytes the tiles name are touched (numpy fancy indexing), so the view may span unmapped
+    gaps between allocations.  No coverage counters (the span can be many gigabytes)."""
+
+    def __init__(self, lo: int, hi: int):
+        self.base, self.nbytes, self.pad = lo, hi - lo, 0
+        self.buf = np.ctypeslib.as_array((ctypes.c_uint8 * (hi - lo)).from_address(lo))
+        self.writes = None
+
+    def offsets(self, addrs: np.ndarray, width: int) -> np.ndarray:
+        off = addrs.astype(np.int64) - self.base
+        assert off.min() >= 0 and off.max() + width <= self.nbytes, "tile touches memory outside the declared span"
+        return off
+
+
 def _unit_positions(run_tiles, row_tiles):
     """Per active work-item: (a address, b address, meta, tile kind, row-tile index)."""
     out = []
@@ -78,17 +95,21 @@ def _unit_positions(run_tiles, row_tiles):
     return out
 
 
-def execute(table, arena: HostArena, direction: str, first: int = 0, count: int | None = None,
-            peers: np.ndarray | None = None) -> None:
-    """Run chunks [first, first+count) of a table on the host. direction: 'pack' | 'unpack' | 'selfcopy'."""
+def execute(table, arena, direction: str, first: int = 0, count: int | None = None,
+            peers: np.ndarray | None = None, ordered: bool = False) -> None:
+    """Run chunks [first, first+count) of a table on the host. direction: 'pack' | 'unpack' | 'selfcopy'.
+    ``ordered``: use the write-ordered copy of the range (it must have been optimized)."""
     global THREADS
     THREADS = int(table.info().tile_threads)
-    run_tiles, row_tiles = table.tiles()
     run_begin, row_begin = table.ranges()
     if count is None:
         count = len(run_begin) - 1 - first
-    run_tiles = run_tiles[run_begin[first] : run_begin[first + count]]
-    row_tiles = row_tiles[row_begin[first] : row_begin[first + count]]
+    if ordered:
+        run_tiles, row_tiles = table.ordered_tiles(first, count)
+    else:
+        run_tiles, row_tiles = table.tiles()
+        run_tiles = run_tiles[run_begin[first] : run_begin[first + count]]
+        row_tiles = row_tiles[row_begin[first] : row_begin[first + count]]
     assert np.all(run_tiles["n"] <= THREADS) and np.all(row_tiles["n"] <= THREADS)
     assert np.all(run_tiles["n"] > 0) and np.all(row_tiles["n"] > 0)
     rev = direction == "unpack"
@@ -118,7 +139,8 @@ def execute(table, arena: HostArena, direction: str, first: int = 0, count: int 
                 data = co.cast(elems, ds_, dd, raw_d).view(np.uint8).reshape(len(so), ud)
             else:
                 assert us == ud
-            np.add.at(arena.writes, do.reshape(-1), 1)
+            if arena.writes is not None:
+                np.add.at(arena.writes, do.reshape(-1), 1)
             mem[do] = data
 
 
@@ -142,5 +164,6 @@ def _reduce_units(arena, mem, row_tiles, row_idx, a_off, b, ua, ub, dta, dtb, pe
         ch = co.make_chunk(0, (0,), (n_units * n_el,), (1,), dta, dtb, peers=[s.ctypes.data for s in staged], op=op)
         assert co.lib().oracle_reduce(ch, out.ctypes.data, scratch.ctypes.data) == 0
         do = arena.offsets(b[sel], ub)[:, None] + np.arange(ub)
-        np.add.at(arena.writes, do.reshape(-1), 1)
+        if arena.writes is not None:
+            np.add.at(arena.writes, do.reshape(-1), 1)
         mem[do] = out.view(np.uint8).reshape(n_units, ub)
