@@ -463,3 +463,32 @@ def test_equal_width_dtypes_convert_instead_of_reinterpreting(gpu_device):
     assert job.recv_buckets[2][0].chunks[0].transfer_dtype == torch.float16
     want = cpu_job.globals_[0][:, :32].to(torch.bfloat16)
     assert torch.equal(job.target_locals[0][2].cpu(), want)
+
+
+@pytest.mark.parametrize("seed", range(60))
+def test_random_batches_gpu(gpu_device, seed):
+    """Random meshes / placements / shapes / dtypes / strides / bucket sizes on the GPU, against the oracle."""
+    from test_random_layouts_cpu import _random_spec
+
+    rng = np.random.default_rng(10_000 + seed)
+    wire_size = int(rng.choice([1, 2, 2, 4, 4, 8]))
+    specs = [_random_spec(rng, i, wire_size) for i in range(int(rng.integers(1, 5)))]
+    bucket_size = [None, 64, 4096, 1 << 20][int(rng.integers(4))]
+    view = None
+    if rng.random() < 0.35:
+        def view(kind, t):
+            if t.dim() == 0 or t.numel() == 0:
+                return t
+            shape = list(t.shape)
+            shape[-1] = shape[-1] * 2 + 3
+            wide = torch.zeros(shape, dtype=t.dtype, device=t.device)
+            return wide[..., 1 : 1 + t.shape[-1]]
+    merge = bool(rng.integers(2))
+    gpu_job = ReshardJob(specs, device=gpu_device, bucket_size=bucket_size, keep_globals=True, fill=cpu_fill, local_view=view)
+    cpu_job = ReshardJob(specs, device="cpu", bucket_size=bucket_size, keep_globals=True, fill=cpu_fill, local_view=view)
+    mirror_partials(gpu_job, cpu_job)
+    gpu_job.run(merge_launches=merge)
+    run_oracle(cpu_job)
+    for i, spec in enumerate(specs):
+        for r, t in gpu_job.target_locals[i].items():
+            assert_bit_equal(t, cpu_job.target_locals[i][r], f"seed {seed} {spec.name} rank {r}")
