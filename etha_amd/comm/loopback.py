@@ -116,6 +116,68 @@ class LoopbackWire:
             raise RuntimeError(f"{bucket}: chunk layout differs from the matching send bucket")
         return slot
 
+    # -- across processes ----------------------------------------------------------------------
+    def export_manifest(self) -> dict:
+        """Describe every planned send slot so that another process on the same GPU can consume it.
+
+        Pool segments are exported with ``hipIpcGetMemHandle`` (allocation base + offset); a slot is
+        ``(segment, offset)``.  The producer sends this once, after planning; afterwards only
+        "generation n is packed" notifications are needed per transfer.
+        """
+        from .. import _native as nat
+
+        if self.pool is None:
+            return {"device": None, "segments": [], "slots": {}}
+        segments = []
+        with torch.cuda.device(self.pool.device):
+            for seg in self.pool.segments:
+                segments.append({"ipc": nat.ipc_export(seg.data_ptr()), "nbytes": seg.numel()})
+        slots: dict = {}
+        for key, entries in self._sent.items():
+            out = []
+            for slot, sizes in entries:
+                idx = next(i for i, seg in enumerate(self.pool.segments)
+                           if seg.data_ptr() <= slot.ptr and slot.ptr + slot.nbytes <= seg.data_ptr() + seg.numel())
+                out.append({"segment": idx, "offset": slot.ptr - self.pool.segments[idx].data_ptr(),
+                            "nbytes": slot.nbytes, "sizes": sizes})
+            slots[key] = out
+        return {"device": self.pool.device.index, "segments": segments, "slots": slots}
+
+    @classmethod
+    def from_manifest(cls, manifest: dict, device: torch.device | str | None = None) -> "LoopbackWire":
+        """Consumer side: map the producer's pool segments and expose its slots for receive planning."""
+        from .. import _native as nat
+
+        dev = torch.device(device) if device is not None else torch.device("cuda", manifest["device"] or 0)
+        wire = cls(dev)
+        wire._imported = []
+        bases = []
+        with torch.cuda.device(dev):
+            for seg in manifest["segments"]:
+                ptr = nat.ipc_open(seg["ipc"])
+                wire._imported.append(ptr)
+                bases.append((ptr, seg["nbytes"]))
+        for key, entries in manifest["slots"].items():
+            for e in entries:
+                base, nbytes = bases[e["segment"]]
+                slot = Slot(ptr=base + e["offset"], nbytes=e["nbytes"], lo=base, hi=base + nbytes)
+                wire._sent[key].append((slot, tuple(e["sizes"])))
+        return wire
+
+    def mark_packed(self) -> None:
+        """Consumer side: the producer reported that every exported slot has been packed (and its stream
+        synchronised) once more."""
+        for entries in self._sent.values():
+            for slot, _ in entries:
+                slot.filled += 1
+
+    def close_imported(self) -> None:
+        from .. import _native as nat
+
+        for ptr in getattr(self, "_imported", []):
+            nat.ipc_close(ptr)
+        self._imported = []
+
     def private_slot(self, nbytes: int, device: torch.device) -> Slot:
         return self._pool_for(device).alloc(nbytes)
 

@@ -151,3 +151,81 @@ def inference_process(tmpdir, device, rounds, out_q):
         out_q.put(("inference", "ok" if not mismatches else "mismatch", {"mismatches": mismatches, "signals": signals}))
     except BaseException:
         out_q.put(("inference", "error", traceback.format_exc()))
+
+
+# ---- bucket pool handed from a producer process to a consumer process ------------------------------------
+def _pool_specs():
+    import torch
+    from torch.distributed.tensor.placement_types import Replicate, Shard
+
+    from etha_amd.world import TensorSpec
+
+    src, tgt = list(range(4)), [4, 5]
+    return [
+        TensorSpec("q", (512, 256), src, (Shard(0),), tgt, (Shard(0),), torch.bfloat16, seed=11, std=1.0),
+        TensorSpec("o", (256, 512), src, (Shard(0),), tgt, (Shard(1),), torch.bfloat16, seed=12, std=1.0),
+        TensorSpec("norm", (256,), src, (Shard(0),), tgt, (Replicate(),), torch.float32, torch.bfloat16, seed=13, std=1.0),
+    ]
+
+
+def producer_process(device, conn, rounds):
+    """Owns the source shards and the bucket pool: plans, exports the pool, packs each round."""
+    try:
+        import torch
+
+        from etha_amd.tensor_bus.bootstrap import setup_ptrace
+        from etha_amd.world import ReshardJob
+        from helpers import cpu_fill
+
+        setup_ptrace()
+        job = ReshardJob(_pool_specs(), device=device, bucket_size=32 * 1024, fill=cpu_fill)
+        for buckets in job.send_buckets.values():
+            job.wire.plan(buckets)  # assigns the slots
+        conn.send(("manifest", job.wire.export_manifest()))
+        for round_ in range(rounds):
+            if round_ > 0:
+                for d in job.source_locals:
+                    for t in d.values():
+                        t.mul_(-2.0)
+            job.run_send(merge_launches=True)
+            torch.cuda.synchronize()  # cross-process ordering is a host-side fence
+            conn.send(("packed", round_))
+            assert conn.recv() == ("consumed", round_)
+        conn.send(("done", None))
+    except BaseException:
+        conn.send(("error", traceback.format_exc()))
+
+
+def consumer_process(device, conn, rounds, out_q):
+    """Maps the producer's pool, plans its receive side against the mapped addresses, unpacks, checks."""
+    try:
+        import torch
+
+        from etha_amd.comm import LoopbackWire
+        from etha_amd.tensor_bus.bootstrap import setup_ptrace
+        from etha_amd.world import ReshardJob
+        from helpers import cpu_fill, expected_target
+
+        setup_ptrace()
+        kind, manifest = conn.recv()
+        assert kind == "manifest", manifest
+        wire = LoopbackWire.from_manifest(manifest, device)
+        specs = _pool_specs()
+        job = ReshardJob(specs, device=device, bucket_size=32 * 1024, fill=cpu_fill, keep_globals=True, wire=wire)
+        bad = []
+        for round_ in range(rounds):
+            assert conn.recv() == ("packed", round_)
+            wire.mark_packed()
+            job.run_recv(merge_launches=True)
+            torch.cuda.synchronize()
+            for i, spec in enumerate(specs):
+                glob = job.globals_[i].cpu().float() * ((-2.0) ** round_)
+                for r, t in job.target_locals[i].items():
+                    want = expected_target(spec, glob.to(spec.source_dtype), r)
+                    if not torch.equal(t.cpu().view(torch.uint8), want.contiguous().view(torch.uint8)):
+                        bad.append((round_, spec.name, r))
+            conn.send(("consumed", round_))
+        wire.close_imported()
+        out_q.put(("consumer", "ok" if not bad else "mismatch", bad))
+    except BaseException:
+        out_q.put(("consumer", "error", traceback.format_exc()))

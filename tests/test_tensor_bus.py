@@ -195,3 +195,28 @@ def test_two_process_hipipc_handoff(gpu_device, tmp_path):
             if p.is_alive():
                 p.kill()
         agent.close()
+
+
+@pytest.mark.gpu
+def test_bucket_pool_crosses_a_process_boundary(gpu_device):
+    """The wire step as a same-GPU loopback between two processes: the producer packs into its pool, the
+    consumer maps the pool with hipIpcOpenMemHandle and unpacks from it; two rounds with new values."""
+    from bus_workers import consumer_process, producer_process
+
+    ctx = mp.get_context("spawn")
+    a, b = ctx.Pipe()
+    out_q = ctx.Queue()
+    procs = [ctx.Process(target=producer_process, args=(str(gpu_device), a, 2)),
+             ctx.Process(target=consumer_process, args=(str(gpu_device), b, 2, out_q))]
+    try:
+        for p in procs:
+            p.start()
+        who, status, detail = out_q.get(timeout=150)
+        for p in procs:
+            p.join(30)
+        assert (who, status) == ("consumer", "ok"), detail
+        assert all(p.exitcode == 0 for p in procs)
+    finally:
+        for p in procs:
+            if p.is_alive():
+                p.kill()
