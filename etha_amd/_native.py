@@ -14,7 +14,7 @@ import numpy as np
 from .build import LIB_PATH
 
 ETHA_MAX_NDIM = 8
-ABI_VERSION = 1
+ABI_VERSION = 2
 
 # element type codes (include/etha_reshard.h)
 F16, BF16, F32, F64, B8, B16, B32, B64 = range(8)
@@ -62,7 +62,9 @@ ROW_TILE = np.dtype(
         ("pad", "<u4"),
     ]
 )
-assert RUN_TILE.itemsize == 24 and ROW_TILE.itemsize == 64
+TRANS_TILE = np.dtype([("a", "<u8"), ("b", "<u8"), ("a_pitch", "<i8"), ("b_pitch", "<i8"), ("nj", "<u4"), ("nk", "<u4"),
+                       ("es_log2", "<u4"), ("pad", "<u4")])
+assert RUN_TILE.itemsize == 24 and ROW_TILE.itemsize == 64 and TRANS_TILE.itemsize == 48
 
 
 class TableInfo(ctypes.Structure):
@@ -73,6 +75,8 @@ class TableInfo(ctypes.Structure):
         ("tile_threads", c_uint32),
         ("device_bytes", c_uint64),
         ("payload_bytes", c_uint64),
+        ("n_trans_tiles", c_uint32),
+        ("reserved", c_uint32),
     ]
 
 
@@ -98,6 +102,7 @@ _SIGNATURES = {
     "etha_table_info": (c_int, [c_void_p, POINTER(TableInfo)]),
     "etha_table_read_tiles": (c_int, [c_void_p, c_int, c_void_p, c_uint64, POINTER(c_uint64)]),
     "etha_table_read_ranges": (c_int, [c_void_p, c_void_p, c_void_p]),
+    "etha_table_read_trans_ranges": (c_int, [c_void_p, c_void_p]),
     "etha_table_optimize_range": (c_int, [c_void_p, c_uint32, c_uint32]),
     "etha_table_read_ordered": (c_int, [c_void_p, c_uint32, c_uint32, c_int, c_void_p, c_uint64, POINTER(c_uint64)]),
     "etha_pack_bucket": (c_int, [c_void_p, c_uint32, c_uint32, c_void_p]),
@@ -192,6 +197,21 @@ class Table:
                 )
             res.append(arr)
         return res[0], res[1]
+
+    def trans_tiles(self) -> np.ndarray:
+        """Host copy of the transposing tiles."""
+        need = c_uint64()
+        _check("etha_table_read_tiles", lib().etha_table_read_tiles(self._h, 2, None, 0, byref(need)))
+        arr = np.zeros(need.value // TRANS_TILE.itemsize, dtype=TRANS_TILE)
+        if need.value:
+            _check("etha_table_read_tiles",
+                   lib().etha_table_read_tiles(self._h, 2, arr.ctypes.data, need.value, byref(need)))
+        return arr
+
+    def trans_ranges(self) -> np.ndarray:
+        out = np.zeros(self.info().n_chunks + 1, dtype=np.uint32)
+        _check("etha_table_read_trans_ranges", lib().etha_table_read_trans_ranges(self._h, out.ctypes.data))
+        return out
 
     def ranges(self) -> tuple[np.ndarray, np.ndarray]:
         n = self.info().n_chunks

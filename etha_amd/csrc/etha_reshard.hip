@@ -6,7 +6,8 @@
 // several vectors per work-item lose 10-30 %.  So all chunk geometry (slices, strides, bucket
 // offsets, dtype pairs, alignment classes) is resolved once on the host into a flat
 // device-resident *tile program*: one entry per workgroup holding absolute addresses.  A
-// workgroup does one scalar table load, each work-item one vector load and one vector store.
+// workgroup does one scalar table load, each work-item one vector load and one vector store.  Only
+// chunks whose contiguous dim differs between the two sides (transposes) are staged through LDS.
 //
 // What it replaces in the reference: the per-chunk ATen launches of Chunk.prepare /
 // Bucket.prepare / Chunk.finalize / Bucket.finalize (src/etha/comm/ir.py:101-141, 229-264,
@@ -69,6 +70,18 @@ struct RowTile {     // walks rows of `run` units; covers units [c0, c0+n) count
   uint32_t pad;
 };
 static_assert(sizeof(RowTile) == 64, "RowTile layout");
+
+struct TransTile {   // a 2-D block whose contiguous dim differs between the two sides (a transposing chunk)
+  uint64_t a;        // address of element (j0, k0) on the a side, contiguous along j
+  uint64_t b;        // address of element (j0, k0) on the b side, contiguous along k
+  int64_t a_pitch;   // bytes between consecutive k on the a side
+  int64_t b_pitch;   // bytes between consecutive j on the b side
+  uint32_t nj, nk;   // extent of the block (<= kTransDim each)
+  uint32_t es_log2;  // log2 of the element size in bytes
+  uint32_t pad;
+};
+static_assert(sizeof(TransTile) == 48, "TransTile layout");
+constexpr uint32_t kTransDim = 64;  // elements per side of a transposing block; one wavefront per block
 
 // meta bits
 constexpr uint32_t kMetaUaShift = 0;    // 4 bits: log2 bytes per unit, a side
@@ -247,6 +260,55 @@ __global__ __launch_bounds__(ETHA_BLOCK_THREADS) void etha_tile_kernel(const Run
   }
   if (tid >= n) return;
   move_unit<REV>(meta, a, b);
+}
+
+// ---- transposing chunks: staged through LDS -----------------------------------------------------
+// The a side is contiguous along j, the b side along k.  A block of up to 64 x 64 elements is read with
+// the wavefront's 64 work-items along the source's contiguous dim (one full run per instruction), parked
+// in LDS with a padded pitch, and written with the work-items along the destination's contiguous dim.
+// Both global sides therefore move whole cache-line runs; without the staging one side would touch a
+// different line per work-item.
+template <typename E, bool REV>
+__device__ __forceinline__ void transpose_block(const TransTile& t, E* __restrict__ lds) {
+  constexpr uint32_t kPitch = kTransDim + 1;  // padded: conflict-free column reads
+  const uint32_t tid = threadIdx.x;
+  if (!REV) {  // a -> b
+    if (tid < t.nj) {
+#pragma unroll 8
+      for (uint32_t k = 0; k < t.nk; k++)
+        lds[k * kPitch + tid] = ld_stream<E>(t.a + (uint64_t)tid * sizeof(E) + (uint64_t)((int64_t)k * t.a_pitch));
+    }
+    __syncthreads();
+    if (tid < t.nk) {
+#pragma unroll 8
+      for (uint32_t j = 0; j < t.nj; j++)
+        st_stream<E>(t.b + (uint64_t)((int64_t)j * t.b_pitch) + (uint64_t)tid * sizeof(E), lds[tid * kPitch + j]);
+    }
+  } else {  // b -> a
+    if (tid < t.nk) {
+#pragma unroll 8
+      for (uint32_t j = 0; j < t.nj; j++)
+        lds[tid * kPitch + j] = ld_stream<E>(t.b + (uint64_t)((int64_t)j * t.b_pitch) + (uint64_t)tid * sizeof(E));
+    }
+    __syncthreads();
+    if (tid < t.nj) {
+#pragma unroll 8
+      for (uint32_t k = 0; k < t.nk; k++)
+        st_stream<E>(t.a + (uint64_t)tid * sizeof(E) + (uint64_t)((int64_t)k * t.a_pitch), lds[k * kPitch + tid]);
+    }
+  }
+}
+
+template <bool REV>
+__global__ __launch_bounds__(64) void etha_transpose_kernel(const TransTile* __restrict__ tiles) {
+  extern __shared__ __attribute__((aligned(16))) uint8_t lds_bytes[];  // kTransDim * (kTransDim + 1) elements
+  const TransTile t = tiles[blockIdx.x];
+  switch (t.es_log2) {
+    case 0: transpose_block<uint8_t, REV>(t, reinterpret_cast<uint8_t*>(lds_bytes)); break;
+    case 1: transpose_block<uint16_t, REV>(t, reinterpret_cast<uint16_t*>(lds_bytes)); break;
+    case 2: transpose_block<uint32_t, REV>(t, reinterpret_cast<uint32_t*>(lds_bytes)); break;
+    default: transpose_block<uint64_t, REV>(t, reinterpret_cast<uint64_t*>(lds_bytes)); break;
+  }
 }
 
 // ---- Partial reduce-pack ------------------------------------------------------------------------
@@ -485,7 +547,8 @@ uint64_t region_numel(const Region& r) {
 struct Builder {
   std::vector<RunTile> run;
   std::vector<RowTile> row;
-  std::vector<uint32_t> run_begin, row_begin;
+  std::vector<TransTile> trans;
+  std::vector<uint32_t> run_begin, row_begin, trans_begin;
   std::vector<uint8_t> is_reduce;
   uint64_t payload_bytes = 0;
 };
@@ -535,6 +598,50 @@ int compile_pair(Builder& bld, uint32_t idx, const Region& A0, const Region& B0,
     run_elems = (uint64_t)n[k - 1];
     k--;
   }
+  // 3b. transposing chunk: no common contiguous dim, but the a side is contiguous along some other dim j
+  //     while the b side is contiguous along the innermost one.  Such chunks go through the LDS-staged
+  //     transposing kernel in blocks of 64 x 64 elements; all other dims are unrolled here.
+  if (run_elems == 1 && !cvt && !red.n_peers && k >= 2 && sb[k - 1] == esb && sa[k - 1] != esa) {
+    int j = -1;
+    for (int i = 0; i < k - 1; i++)
+      if (sa[i] == esa && n[i] >= 8) j = i;
+    if (j >= 0 && n[k - 1] >= 8 && (A0.base % (uint64_t)esa) == 0 && (B0.base % (uint64_t)esb) == 0) {
+      const int kk = k - 1;
+      int64_t pos[ETHA_MAX_NDIM] = {0};
+      uint64_t off_a = 0, off_b = 0;
+      while (true) {
+        for (int64_t j0 = 0; j0 < n[j]; j0 += kTransDim)
+          for (int64_t k0 = 0; k0 < n[kk]; k0 += kTransDim) {
+            TransTile t;
+            memset(&t, 0, sizeof(t));
+            t.a = A0.base + off_a + (uint64_t)(j0 * sa[j]) + (uint64_t)(k0 * sa[kk]);
+            t.b = B0.base + off_b + (uint64_t)(j0 * sb[j]) + (uint64_t)(k0 * sb[kk]);
+            t.a_pitch = sa[kk];
+            t.b_pitch = sb[j];
+            t.nj = (uint32_t)(n[j] - j0 < kTransDim ? n[j] - j0 : kTransDim);
+            t.nk = (uint32_t)(n[kk] - k0 < kTransDim ? n[kk] - k0 : kTransDim);
+            t.es_log2 = (uint32_t)log2u((uint64_t)esa);
+            bld.trans.push_back(t);
+          }
+        if (bld.trans.size() > kMaxTiles)
+          return fail(ETHA_ERR_UNSUPPORTED, "tile program too large (> %llu tiles)", (unsigned long long)kMaxTiles);
+        int d = k - 1;
+        for (; d >= 0; d--) {
+          if (d == j || d == kk) continue;
+          pos[d]++;
+          off_a += (uint64_t)sa[d];
+          off_b += (uint64_t)sb[d];
+          if (pos[d] < n[d]) break;
+          off_a -= (uint64_t)(sa[d] * n[d]);
+          off_b -= (uint64_t)(sb[d] * n[d]);
+          pos[d] = 0;
+        }
+        if (d < 0) break;
+      }
+      return ETHA_OK;
+    }
+  }
+
   // 4. unit size: the widest vector every row start and the run length allow
   int ua_log2, ub_log2;
   uint64_t run_units;
@@ -701,11 +808,14 @@ struct EthaTable {
   int kind = 0;  // 0 = pack/unpack table, 1 = self-copy table
   std::vector<RunTile> h_run;
   std::vector<RowTile> h_row;
-  std::vector<uint32_t> run_begin, row_begin;
+  std::vector<TransTile> h_trans;
+  std::vector<uint32_t> run_begin, row_begin, trans_begin;
   std::vector<uint32_t> reduce_prefix;  // number of reduce chunks before chunk i
   std::vector<uint64_t> h_peers;
   RunTile* d_run = nullptr;
   RowTile* d_row = nullptr;
+  TransTile* d_trans = nullptr;
+  uint32_t trans_es_max = 1;  // largest element size among the transposing tiles (sizes the LDS)
   uint64_t* d_peers = nullptr;
   uint32_t n_chunks = 0;
   uint64_t payload_bytes = 0;
@@ -737,6 +847,12 @@ int upload_table(EthaTable* t) {
     HIP_TRY(hipMemcpy(t->d_row, t->h_row.data(), bytes, hipMemcpyHostToDevice));
     t->device_bytes += bytes;
   }
+  if (!t->h_trans.empty()) {
+    const size_t bytes = t->h_trans.size() * sizeof(TransTile);
+    HIP_TRY(hipMalloc(&t->d_trans, bytes));
+    HIP_TRY(hipMemcpy(t->d_trans, t->h_trans.data(), bytes, hipMemcpyHostToDevice));
+    t->device_bytes += bytes;
+  }
   if (!t->h_peers.empty()) {
     const size_t bytes = t->h_peers.size() * sizeof(uint64_t);
     HIP_TRY(hipMalloc(&t->d_peers, bytes));
@@ -752,6 +868,7 @@ void free_table(EthaTable* t) {
   if (t->d_run) (void)hipFree(t->d_run);
   if (t->d_row) (void)hipFree(t->d_row);
   if (t->d_peers) (void)hipFree(t->d_peers);
+  if (t->d_trans) (void)hipFree(t->d_trans);
   for (auto& kv : t->ordered) {
     if (kv.second.d_run) (void)hipFree(kv.second.d_run);
     if (kv.second.d_row) (void)hipFree(kv.second.d_row);
@@ -762,8 +879,12 @@ void free_table(EthaTable* t) {
 int finish_table(Builder& bld, EthaTable* t, int upload, EthaTable** out) {
   t->h_run.swap(bld.run);
   t->h_row.swap(bld.row);
+  t->h_trans.swap(bld.trans);
   t->run_begin.swap(bld.run_begin);
   t->row_begin.swap(bld.row_begin);
+  t->trans_begin.swap(bld.trans_begin);
+  for (const TransTile& tt : t->h_trans)
+    if ((1u << tt.es_log2) > t->trans_es_max) t->trans_es_max = 1u << tt.es_log2;
   t->reduce_prefix.assign(t->n_chunks + 1, 0);
   for (uint32_t i = 0; i < t->n_chunks; i++) t->reduce_prefix[i + 1] = t->reduce_prefix[i] + bld.is_reduce[i];
   t->payload_bytes = bld.payload_bytes;
@@ -792,6 +913,12 @@ int launch_tiles(const EthaTable* t, uint32_t first, uint32_t count, void* strea
   const uint32_t r0 = t->run_begin[first], r1 = t->run_begin[first + count];
   const uint32_t w0 = t->row_begin[first], w1 = t->row_begin[first + count];
   const uint32_t n_run = r1 - r0, n_row = w1 - w0;
+  const uint32_t x0 = t->trans_begin[first], n_trans = t->trans_begin[first + count] - x0;
+  if (n_trans) {  // transposing chunks run in their own kernel (it needs LDS)
+    const size_t lds = (size_t)kTransDim * (kTransDim + 1) * t->trans_es_max;
+    hipLaunchKernelGGL(etha_transpose_kernel<REV>, dim3(n_trans), dim3(64), lds, (hipStream_t)stream, t->d_trans + x0);
+    HIP_TRY(hipGetLastError());
+  }
   if (n_run + n_row == 0) return ETHA_OK;
   if (REV == (t->kind == 0)) {  // the direction that writes the a side (unpack) / b side (self-copy) of an ordered range
     auto it = t->ordered.find(std::make_pair(first, count));
@@ -828,6 +955,7 @@ int etha_table_create(const EthaChunkDesc* descs, uint32_t n_chunks, const uint6
     const EthaChunkDesc& d = descs[i];
     bld.run_begin.push_back((uint32_t)bld.run.size());
     bld.row_begin.push_back((uint32_t)bld.row.size());
+    bld.trans_begin.push_back((uint32_t)bld.trans.size());
     const int esw = dtype_size(d.wire_dtype);
     if (esw == 0) return fail(ETHA_ERR_INVALID, "chunk %u: unknown wire_dtype %u", i, d.wire_dtype);
     ReduceSpec red;
@@ -883,6 +1011,7 @@ int etha_table_create(const EthaChunkDesc* descs, uint32_t n_chunks, const uint6
   }
   bld.run_begin.push_back((uint32_t)bld.run.size());
   bld.row_begin.push_back((uint32_t)bld.row.size());
+  bld.trans_begin.push_back((uint32_t)bld.trans.size());
   EthaTable* t = new (std::nothrow) EthaTable();
   if (!t) return fail(ETHA_ERR_NOMEM, "out of host memory");
   t->kind = 0;
@@ -901,6 +1030,7 @@ int etha_selfcopy_table_create(const EthaChunkDesc* src, const EthaChunkDesc* ds
   for (uint32_t i = 0; i < n_chunks; i++) {
     bld.run_begin.push_back((uint32_t)bld.run.size());
     bld.row_begin.push_back((uint32_t)bld.row.size());
+    bld.trans_begin.push_back((uint32_t)bld.trans.size());
     if (src[i].n_partials || dst[i].n_partials)
       return fail(ETHA_ERR_UNSUPPORTED, "chunk %u: self-copy of a Partial source is not implemented", i);
     Region A, B;
@@ -914,6 +1044,7 @@ int etha_selfcopy_table_create(const EthaChunkDesc* src, const EthaChunkDesc* ds
   }
   bld.run_begin.push_back((uint32_t)bld.run.size());
   bld.row_begin.push_back((uint32_t)bld.row.size());
+  bld.trans_begin.push_back((uint32_t)bld.trans.size());
   EthaTable* t = new (std::nothrow) EthaTable();
   if (!t) return fail(ETHA_ERR_NOMEM, "out of host memory");
   t->kind = 1;
@@ -931,6 +1062,7 @@ int etha_table_info(const EthaTable* t, EthaTableInfo* out) {
   out->n_chunks = t->n_chunks;
   out->n_run_tiles = (uint32_t)t->h_run.size();
   out->n_row_tiles = (uint32_t)t->h_row.size();
+  out->n_trans_tiles = (uint32_t)t->h_trans.size();
   out->tile_threads = kTileThreads;
   out->device_bytes = t->device_bytes;
   out->payload_bytes = t->payload_bytes;
@@ -947,8 +1079,11 @@ int etha_table_read_tiles(const EthaTable* t, int which, void* out, uint64_t cap
   } else if (which == 1) {
     src = t->h_row.data();
     bytes = t->h_row.size() * sizeof(RowTile);
+  } else if (which == 2) {
+    src = t->h_trans.data();
+    bytes = t->h_trans.size() * sizeof(TransTile);
   } else {
-    return fail(ETHA_ERR_INVALID, "which must be 0 or 1");
+    return fail(ETHA_ERR_INVALID, "which must be 0, 1 or 2");
   }
   *need_bytes = bytes;
   if (out && bytes) memcpy(out, src, bytes < cap_bytes ? bytes : cap_bytes);
@@ -959,6 +1094,12 @@ int etha_table_read_ranges(const EthaTable* t, uint32_t* run_begin, uint32_t* ro
   if (!t || !run_begin || !row_begin) return fail(ETHA_ERR_INVALID, "null argument");
   memcpy(run_begin, t->run_begin.data(), t->run_begin.size() * sizeof(uint32_t));
   memcpy(row_begin, t->row_begin.data(), t->row_begin.size() * sizeof(uint32_t));
+  return ETHA_OK;
+}
+
+int etha_table_read_trans_ranges(const EthaTable* t, uint32_t* trans_begin) {
+  if (!t || !trans_begin) return fail(ETHA_ERR_INVALID, "null argument");
+  memcpy(trans_begin, t->trans_begin.data(), t->trans_begin.size() * sizeof(uint32_t));
   return ETHA_OK;
 }
 

@@ -31,7 +31,7 @@
 extern "C" {
 #endif
 
-#define ETHA_ABI_VERSION 1
+#define ETHA_ABI_VERSION 2
 #define ETHA_MAX_NDIM 8
 
 /* status codes */
@@ -87,6 +87,8 @@ typedef struct EthaTableInfo {
   uint32_t tile_threads;  /* units (work-items) per tile; one tile = tile_threads / 64 workgroups of one wavefront */
   uint64_t device_bytes;  /* device memory held by the table */
   uint64_t payload_bytes; /* sum over chunks of numel * wire element size */
+  uint32_t n_trans_tiles; /* 64 x 64-element blocks of transposing chunks (staged through LDS) */
+  uint32_t reserved;
 } EthaTableInfo;
 
 typedef struct EthaIpcHandle {
@@ -123,13 +125,14 @@ int etha_table_info(const EthaTable* table, EthaTableInfo* out);
 
 /*
  * Inspection of the compiled program (host copies), for CPU-side checking.
- * which: 0 = run tiles (uint64 a, b; uint32 n, meta), 1 = row tiles (see etha_reshard.hip).
+ * which: 0 = run tiles (uint64 a, b; uint32 n, meta), 1 = row tiles, 2 = transposing tiles (see etha_reshard.hip).
  * A tile holds up to tile_units units and is executed by tile_units / 64 workgroups of 64 work-items.
  * Copies up to cap_bytes into out and stores the full size in *need_bytes.
  */
 int etha_table_read_tiles(const EthaTable* table, int which, void* out, uint64_t cap_bytes, uint64_t* need_bytes);
 /* per-chunk first-tile indices, n_chunks+1 entries each */
 int etha_table_read_ranges(const EthaTable* table, uint32_t* run_begin, uint32_t* row_begin);
+int etha_table_read_trans_ranges(const EthaTable* table, uint32_t* trans_begin);
 
 /*
  * Declare that chunks [first, first+count) are always launched together by etha_unpack_bucket (or

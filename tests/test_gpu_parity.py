@@ -492,3 +492,24 @@ def test_random_batches_gpu(gpu_device, seed):
     for i, spec in enumerate(specs):
         for r, t in gpu_job.target_locals[i].items():
             assert_bit_equal(t, cpu_job.target_locals[i][r], f"seed {seed} {spec.name} rank {r}")
+
+
+@pytest.mark.parametrize("dtype", [torch.int8, torch.bfloat16, torch.float32, torch.float64])
+def test_transposed_parents_go_through_lds(gpu_device, dtype):
+    """Source and target shards that are transposes of their storage ([R, C] views of [C, R] tensors)."""
+    def transposed(kind, t):
+        if t.dim() != 2:
+            return t
+        return torch.zeros(t.shape[1], t.shape[0], dtype=t.dtype, device=t.device).t()
+
+    spec = TensorSpec("w", (260, 330), mesh_of(0, [2]), (Shard(0),), mesh_of(2, [3]), (Shard(1),), dtype, seed=21, dist="bits")
+    gpu_job = ReshardJob([spec], device=gpu_device, bucket_size=1 << 20, keep_globals=True, fill=cpu_fill, local_view=transposed)
+    cpu_job = ReshardJob([spec], device="cpu", bucket_size=1 << 20, keep_globals=True, fill=cpu_fill, local_view=transposed)
+    assert not gpu_job.source_locals[0][0].is_contiguous()
+    gpu_job.run()
+    run_oracle(cpu_job)
+    for r, t in gpu_job.target_locals[0].items():
+        assert_bit_equal(t, cpu_job.target_locals[0][r], f"rank {r}")
+        assert_bit_equal(t, expected_target(spec, cpu_job.globals_[0], r), f"rank {r} closed form")
+    assert gpu_job.wire.plan(gpu_job.send_buckets[0]).send_table.info().n_trans_tiles > 0
+    assert gpu_job.wire.plan(gpu_job.recv_buckets[2]).recv_table.info().n_trans_tiles > 0

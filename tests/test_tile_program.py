@@ -229,3 +229,37 @@ def test_optimized_range_is_a_write_ordered_permutation():
     assert not np.all(np.diff(logical) >= 0)  # bucket order is not write order here
     with pytest.raises(nat.EthaNativeError, match="not been optimized"):
         table.ordered_tiles(0, 2)
+
+
+@pytest.mark.parametrize("dt", [nat.B8, nat.BF16, nat.F32, nat.B64])
+def test_transposed_parent_uses_lds_blocks(dt):
+    """A chunk of a transposed view: the tensor side is contiguous along dim 0, the bucket along dim 1."""
+    rows, cols, es = 150, 97, ES[dt]
+    arena = HostArena(3 * rows * cols * es + 65536)
+    t = arena.alloc(rows * cols * es)   # storage of the [cols, rows] parent; the view is its transpose
+    arena.bytes_at(t, rows * cols * es)[:] = rs.randint(0, 256, rows * cols * es)
+    b = arena.alloc(rows * cols * es)
+    start, cshape, strides = (3, 2), (140, 90), (1, rows)  # view[i, j] = parent[j, i]
+    d = _mk_desc(t, t, t + rows * cols * es, b, b, b + 140 * 90 * es, start, cshape, strides, dt, dt)
+    table = nat.Table.create(d.reshape(1), upload=False)
+    info = table.info()
+    assert info.n_trans_tiles == 3 * 2 and info.n_run_tiles == 0 and info.n_row_tiles == 0  # ceil(140/64) x ceil(90/64)
+    before = arena.bytes_at(t, rows * cols * es).copy()
+    execute(table, arena, "pack")
+    want = np.zeros(140 * 90 * es, dtype=np.uint8)
+    scratch = np.zeros(140 * 90 * es, dtype=np.uint8)
+    oc = co.make_chunk(t, start, cshape, strides, dt, dt, bucket_off=0)
+    assert co.lib().oracle_pack_bucket(oc, 1, want.ctypes.data, scratch.ctypes.data) == 0
+    assert np.array_equal(arena.bytes_at(b, 140 * 90 * es), want)
+    assert np.array_equal(arena.bytes_at(t, rows * cols * es), before)
+    assert arena.writes.max() == 1 and int(arena.writes.sum()) == 140 * 90 * es
+    # and back: unpack into a second transposed parent
+    arena.writes[:] = 0
+    t2 = arena.alloc(rows * cols * es)
+    before2 = arena.bytes_at(t2, rows * cols * es).copy()
+    d2 = _mk_desc(t2, t2, t2 + rows * cols * es, b, b, b + 140 * 90 * es, start, cshape, strides, dt, dt)
+    execute(nat.Table.create(d2.reshape(1), upload=False), arena, "unpack")
+    want2 = before2.copy()
+    oc2 = co.make_chunk(want2.ctypes.data, start, cshape, strides, dt, dt, bucket_off=0)
+    assert co.lib().oracle_unpack_bucket(oc2, 1, want.ctypes.data, scratch.ctypes.data) == 0
+    assert np.array_equal(arena.bytes_at(t2, rows * cols * es), want2)

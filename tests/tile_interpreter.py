@@ -110,6 +110,10 @@ def execute(table, arena, direction: str, first: int = 0, count: int | None = No
         run_tiles, row_tiles = table.tiles()
         run_tiles = run_tiles[run_begin[first] : run_begin[first + count]]
         row_tiles = row_tiles[row_begin[first] : row_begin[first + count]]
+    trans_begin = table.trans_ranges()
+    trans = table.trans_tiles()[trans_begin[first] : trans_begin[first + count]]
+    if len(trans):
+        _transpose_blocks(arena, trans, direction == "unpack")
     assert np.all(run_tiles["n"] <= THREADS) and np.all(row_tiles["n"] <= THREADS)
     assert np.all(run_tiles["n"] > 0) and np.all(row_tiles["n"] > 0)
     rev = direction == "unpack"
@@ -142,6 +146,24 @@ def execute(table, arena, direction: str, first: int = 0, count: int | None = No
             if arena.writes is not None:
                 np.add.at(arena.writes, do.reshape(-1), 1)
             mem[do] = data
+
+
+def _transpose_blocks(arena, trans, rev: bool) -> None:
+    mem = arena.buf[arena.pad : arena.pad + arena.nbytes]
+    for t in trans:
+        es = 1 << int(t["es_log2"])
+        nj, nk = int(t["nj"]), int(t["nk"])
+        assert 0 < nj <= 64 and 0 < nk <= 64
+        j, k = np.meshgrid(np.arange(nj), np.arange(nk), indexing="ij")
+        a = int(t["a"]) + j * es + k * int(t["a_pitch"])
+        b = int(t["b"]) + j * int(t["b_pitch"]) + k * es
+        assert np.all(a % es == 0) and np.all(b % es == 0)
+        src, dst = (b, a) if rev else (a, b)
+        so = arena.offsets(src.reshape(-1), es)[:, None] + np.arange(es)
+        do = arena.offsets(dst.reshape(-1), es)[:, None] + np.arange(es)
+        if arena.writes is not None:
+            np.add.at(arena.writes, do.reshape(-1), 1)
+        mem[do] = mem[so]
 
 
 def _reduce_units(arena, mem, row_tiles, row_idx, a_off, b, ua, ub, dta, dtb, peers):
