@@ -36,8 +36,16 @@ class BucketPool:
         self.segment_bytes = segment_bytes
         self.segments: list[torch.Tensor] = []
         self._cursor = 0  # offset inside the last segment
+        self._free: dict[int, list[Slot]] = {}  # released slots, reused for requests of exactly their size
+
+    def release(self, slot: Slot) -> None:
+        slot.filled = slot.drained = 0
+        self._free.setdefault(slot.nbytes, []).append(slot)
 
     def alloc(self, nbytes: int) -> Slot:
+        free = self._free.get(nbytes)
+        if free:
+            return free.pop()
         need = max(nbytes, 1)
         if need > self.segment_bytes or not self.segments or self._cursor + need > self.segments[-1].numel():
             size = max(self.segment_bytes, need)
@@ -197,6 +205,28 @@ class LoopbackWire:
             plan = TransferPlan(self, list(buckets))
             self._plans[key] = plan
         return plan
+
+    def release(self, buckets: list[Bucket]) -> None:
+        """Forget a bucket list: drop its compiled plan and hand its send slots back to the pool.
+        The caller guarantees that no transfer of these buckets, on either end, is still in flight."""
+        plan = self._plans.pop(tuple(id(b) for b in buckets), None)
+        if plan is None:
+            return
+        for kind, _, _, slot in plan.steps:
+            if slot is None or self.pool is None:
+                continue
+            owned = False
+            for key, entries in list(self._sent.items()):
+                kept = [(s, sizes) for s, sizes in entries if s is not slot]
+                if len(kept) != len(entries):
+                    owned = True
+                    if kept:
+                        self._sent[key] = kept
+                    else:
+                        del self._sent[key]
+            if owned or kind == "pack":
+                if not any(slot is s for s in self.pool._free.get(slot.nbytes, [])):
+                    self.pool.release(slot)
 
     def reset(self) -> None:
         self._plans.clear()

@@ -398,8 +398,10 @@ class TensorBusAgent:
         self.stats["transfers"] += 1
         return True, {"ms": (time.perf_counter() - t0) * 1e3}
 
-    @staticmethod
-    def _release_batch(batch: BatchState) -> None:
+    def _release_batch(self, batch: BatchState) -> None:
+        # receivers first: their plans only reference slots, the senders' plans own them
+        for buckets in list(batch.recv_buckets.values()) + list(batch.send_buckets.values()):
+            self.wire.release(buckets)
         for regs in batch.registrations.values():
             for _, t in regs:
                 if isinstance(t, IpcTensor):

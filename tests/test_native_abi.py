@@ -101,3 +101,18 @@ def test_executor_refuses_cpu_tensors():
                      device="cpu", bucket_size=None)
     with pytest.raises(RuntimeError, match="no CPU path"):
         job.run()
+
+
+def test_ipc_entry_points_reject_bad_arguments_without_a_gpu():
+    import ctypes
+
+    h = nat.IpcHandle()
+    h.size = 2 << 30  # allocations of 2 GiB and more are refused before any HIP call
+    out = ctypes.c_void_p()
+    assert nat.lib().etha_ipc_open(ctypes.byref(h), ctypes.byref(out)) == nat.ERR_UNSUPPORTED
+    assert b"under 2 GiB" in nat.lib().etha_last_error()
+    assert nat.lib().etha_ipc_open(None, ctypes.byref(out)) == nat.ERR_INVALID
+    with pytest.raises(nat.EthaNativeError, match="not returned by etha_ipc_open"):
+        nat.ipc_close(0x1234)
+    nat.ipc_close(0)  # null is a no-op
+    assert nat.lib().etha_arena_create(0, ctypes.byref(out)) == nat.ERR_INVALID

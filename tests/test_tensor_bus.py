@@ -220,3 +220,35 @@ def test_bucket_pool_crosses_a_process_boundary(gpu_device):
         for p in procs:
             if p.is_alive():
                 p.kill()
+
+
+@pytest.mark.gpu
+def test_cleanup_returns_pool_slots(gpu_device, agent_factory):
+    """Registering, transferring and closing the same batch repeatedly must not grow the bucket pool."""
+    agent, naming = agent_factory(2, device=gpu_device)
+    src = torch.arange(4096, dtype=torch.float32, device=gpu_device).reshape(64, 64)
+    tgt = torch.zeros(64, 64, device=gpu_device)
+    clients = {r: _client(naming, r, connection_timeout=5) for r in range(2)}
+
+    def pair(r):
+        clients[r].init_pair("w", "a" if r == 0 else "b", "b" if r == 0 else "a", 1, device_mesh=torch.arange(1),
+                             placements=(Replicate(),))
+
+    run_ranks(pair, range(2))
+    reserved = []
+    for it in range(3):
+        src.add_(1.0)
+        torch.cuda.synchronize()
+
+        def body(r):
+            h = clients[r].register_tensors(f"b{it}", [((src if r == 0 else tgt), "w")], bucket_size=1 << 20)
+            h.transfer("send" if r == 0 else "recv", blocking=True)
+            h.close()
+
+        run_ranks(body, range(2))
+        torch.cuda.synchronize()
+        assert torch.equal(tgt, src)
+        reserved.append((agent.wire.pool.reserved_bytes, agent.wire.pool._cursor, len(agent.wire._plans)))
+    assert reserved[0] == reserved[1] == reserved[2], reserved
+    for c in clients.values():
+        c.close()
