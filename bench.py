@@ -39,6 +39,8 @@ def parse_args():
     ap.add_argument("--workload", default="llama3_8b_fsdp8_to_tp2")
     ap.add_argument("--per-bucket", action="store_true", help="one launch per bucket instead of one per run of buckets")
     ap.add_argument("--fanout", type=int, default=1, help="side streams for per-bucket launches (with --per-bucket)")
+    ap.add_argument("--zero-copy", action="store_true",
+                    help="lend contiguous single-chunk buckets to the consumer instead of packing them")
     ap.add_argument("--graph", action="store_true", help="replay the step from a captured HIP graph (whole step timed)")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--cpu-layers", type=int, default=8, help="layers of the workload the CPU baseline sample covers")
@@ -119,7 +121,7 @@ def main():
     torch.cuda.set_device(dev)
     specs, targets, bucket = workloads.WORKLOADS[args.workload]()
     t0 = time.time()
-    job = ReshardJob(specs, device=dev, bucket_size=bucket, target_ranks=targets)
+    job = ReshardJob(specs, device=dev, bucket_size=bucket, target_ranks=targets, zero_copy=args.zero_copy)
     merge = not args.per_bucket
     # plan (compiles the tile programs) + warm-up
     for _ in range(max(args.warmup, 1)):
@@ -144,7 +146,7 @@ def main():
     pack_read = 0
     for p in send_plans:
         for b in p.buckets:
-            if b.transport.value in ("p2p", "broadcast") and b.is_source:
+            if b.transport.value in ("p2p", "broadcast") and b.is_source and id(b) not in p.lent:
                 for c in b.chunks:
                     peers = c.partial_peers()
                     n = 1
@@ -236,6 +238,7 @@ def main():
             "launch_granularity": "run of buckets" if merge else "bucket",
             "fanout_streams": args.fanout,
             "hip_graph": bool(args.graph),
+            "zero_copy_single_chunk": bool(args.zero_copy),
             **job.counts(),
         },
         "device_ms_per_step": round(dev_ms, 4),

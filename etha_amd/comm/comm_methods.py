@@ -9,7 +9,9 @@ Here a bucket list is compiled once into tile programs and a call enqueues, in b
 * target buckets:  one unpack launch each - ``Bucket.finalize``;
 * LOCAL buckets:   one direct self-copy launch each, or pack + unpack through a private slot when
                    source and destination bytes may overlap;
-* NONE buckets:    nothing - the primary's reduce-pack already read this member's partial.
+* NONE buckets:    nothing - the primary's reduce-pack already read this member's partial;
+* with the wire's ``zero_copy_single_chunk`` option, a single-chunk source bucket whose bytes already lie
+  contiguously in the tensor is lent, not packed: the consumer unpacks straight from the tensor.
 
 Consecutive buckets of the same kind can be merged into one launch (``merge_launches=True``).
 All work goes to one stream, so per-channel FIFO order and "pack before unpack" hold by stream
@@ -27,7 +29,7 @@ from .transfer import Transport
 
 __all__ = ["bucket_comm", "TransferPlan"]
 
-_PACK, _REDUCE, _UNPACK, _SELF = "pack", "reduce_pack", "unpack", "selfcopy"
+_PACK, _REDUCE, _UNPACK, _SELF, _LEND = "pack", "reduce_pack", "unpack", "selfcopy", "lend"
 
 
 class TransferPlan:
@@ -40,6 +42,7 @@ class TransferPlan:
         send, recv, local = DescBuilder(), DescBuilder(), SelfCopyBuilder()
         # steps: (kind, first_chunk, n_chunks, slot or None), in execution order
         self.steps: list[tuple[str, int, int, object]] = []
+        self.lent: set[int] = set()  # ids of source buckets that are consumed straight from their tensor
         send_index: dict[tuple, int] = {}
         recv_index: dict[tuple, int] = {}
         from .loopback import wire_key
@@ -83,6 +86,10 @@ class TransferPlan:
                 idx = send_index.get(key, 0)
                 send_index[key] = idx + 1
                 slot = wire.slot_for_send(bucket, idx, device)
+                if slot.borrowed:  # zero-copy: the consumer reads the tensor itself; nothing to launch
+                    self.steps.append((_LEND, 0, 0, slot))
+                    self.lent.add(id(bucket))
+                    continue
                 first = len(send)
                 reduce = bool(bucket.chunks[0].source_partial_groups)
                 for off, c in zip(bucket.offsets, bucket.chunks):
@@ -125,7 +132,12 @@ class TransferPlan:
     @staticmethod
     def _merge(steps):
         merged: list[list] = []
+        lends = [s[3] for s in steps if s[0] == _LEND]
+        if lends:  # nothing is launched for them; keep them out of the way of merging their neighbours
+            merged.append([_LEND, 0, 0, list(lends)])
         for kind, first, count, slot in steps:
+            if kind == _LEND:
+                continue
             if merged and merged[-1][0] == kind and merged[-1][1] + merged[-1][2] == first:
                 merged[-1][2] += count
                 merged[-1][3].append(slot)
@@ -205,12 +217,16 @@ class TransferPlan:
                             "recv bucket runs before its send bucket was ever packed (a real wire would block here)"
                         )
                 self.recv_table.unpack(first, count, stream)
-            else:
+            elif kind == _SELF:
                 self.local_table.selfcopy(first, count, stream)
-            if kind in (_PACK, _REDUCE):
+            if kind in (_PACK, _REDUCE, _LEND):
                 for s in slots:
                     if s is not None:
                         s.filled += 1
+
+    def lends_tensor_memory(self) -> bool:
+        """True when some send bucket of this plan is consumed straight from its source tensor."""
+        return any(kind == _LEND for kind, _, _, _ in self.steps)
 
     def payload_bytes(self) -> dict[str, int]:
         out = {}

@@ -93,6 +93,8 @@ class Slot:
     hi: int
     filled: int = 0  # number of times a pack has been enqueued into this slot
     drained: int = 0  # number of unpacks enqueued from it (per consumer bookkeeping is the wire's job)
+    borrowed: bool = False  # the slot IS the source tensor's memory (zero-copy single-chunk bucket), not pool memory
+    keepalive: object = None  # the tensor a borrowed slot aliases
 
 
 class DescBuilder:
@@ -188,6 +190,35 @@ def region_hull(tensor, slices: tuple) -> tuple[int, int]:
     if empty:
         return lo, lo
     return lo, lo + (span_el + 1) * es
+
+
+def zero_copy_region(bucket: Bucket):
+    """``(address, storage lo, storage hi, keepalive tensor)`` when the bucket's bytes already exist, in bucket
+    layout, inside its source tensor - else None.
+
+    That is the reference's single-entry path: one chunk, its slice contiguous, no Partial reduce and no
+    cast, so that ``bucket.buffer = chunk.buffer.view(uint8)`` aliases the tensor (``ir.py:238-244``)."""
+    if len(bucket.chunks) != 1:
+        return None
+    c = bucket.chunks[0]
+    t = c.tensor
+    if c.source_partial_groups or t is None or (c.transfer_dtype or t.dtype) != t.dtype or c.nbytes == 0:
+        return None
+    shape, stride = tuple(t.shape), tuple(t.stride())
+    start_el, expect, contiguous = 0, 1, True
+    for d in range(len(shape) - 1, -1, -1):
+        lo, hi = 0, shape[d]
+        if d < len(c.src_slice):
+            lo, hi, _ = c.src_slice[d].indices(shape[d])
+        ext = hi - lo
+        start_el += lo * stride[d]
+        if ext != 1 and stride[d] != expect:
+            contiguous = False
+        expect *= ext
+    if not contiguous:
+        return None
+    lo_b, hi_b = _storage_range(t)
+    return t.data_ptr() + start_el * t.element_size(), lo_b, hi_b, t
 
 
 def local_bucket_needs_staging(bucket: Bucket) -> bool:

@@ -243,7 +243,7 @@ class Bucket:
     def prepare(self, wire=None) -> None:
         """Source bucket: enqueue its pack (or reduce-pack / self-copy) launch.  Target bucket: nothing
         to do, its bytes arrive in the producer's pool slot (``Bucket.prepare``, ``ir.py:229-264``)."""
-        self._plan(wire).run_kinds(("pack", "reduce_pack", "selfcopy"))
+        self._plan(wire).run_kinds(("pack", "reduce_pack", "selfcopy", "lend"))
 
     def launch(self) -> bool:
         """The wire step.  Always ready: the loopback hands the pool slot over in place

@@ -83,6 +83,11 @@ class LoopbackWire:
         # True: bucket lists on host tensors may be *planned* (tile programs compiled against host
         # addresses, for checking them on the CPU); they still cannot be run
         self.host_inspection = host_inspection
+        # True: a single-chunk bucket whose bytes already lie contiguously in its source tensor is not
+        # packed at all - the consumer unpacks straight from the tensor, as the reference's single-entry
+        # path sends straight from it (ir.py:238-244).  The producer must then leave that tensor alone
+        # until the consumer has unpacked: "sent" no longer means "copied".
+        self.zero_copy_single_chunk = False
         self.pool: BucketPool | None = None
         self._sent: dict[tuple, list[tuple[Slot, tuple[int, ...]]]] = defaultdict(list)
         self._plans: dict[tuple, object] = {}
@@ -108,7 +113,17 @@ class LoopbackWire:
             return slot
         if index != len(sent):
             raise RuntimeError(f"{bucket}: send buckets must be planned in order")
-        slot = self._pool_for(device).alloc(bucket.total_bytes)
+        slot = None
+        if self.zero_copy_single_chunk:
+            from .device_plan import zero_copy_region
+
+            region = zero_copy_region(bucket)
+            if region is not None:
+                self._pool_for(device)
+                slot = Slot(ptr=region[0], nbytes=bucket.total_bytes, lo=region[1], hi=region[2], borrowed=True)
+                slot.keepalive = region[3]
+        if slot is None:
+            slot = self._pool_for(device).alloc(bucket.total_bytes)
         sent.append((slot, sizes))
         return slot
 
@@ -144,6 +159,11 @@ class LoopbackWire:
         for key, entries in self._sent.items():
             out = []
             for slot, sizes in entries:
+                if slot.borrowed:  # lives in a source tensor: export that allocation, range = the slot itself
+                    with torch.cuda.device(self.pool.device):
+                        segments.append({"ipc": nat.ipc_export(slot.ptr), "nbytes": slot.nbytes})
+                    out.append({"segment": len(segments) - 1, "offset": 0, "nbytes": slot.nbytes, "sizes": sizes})
+                    continue
                 idx = next(i for i, seg in enumerate(self.pool.segments)
                            if seg.data_ptr() <= slot.ptr and slot.ptr + slot.nbytes <= seg.data_ptr() + seg.numel())
                 out.append({"segment": idx, "offset": slot.ptr - self.pool.segments[idx].data_ptr(),
@@ -224,7 +244,7 @@ class LoopbackWire:
                         self._sent[key] = kept
                     else:
                         del self._sent[key]
-            if owned or kind == "pack":
+            if (owned or kind == "pack") and not slot.borrowed:
                 if not any(slot is s for s in self.pool._free.get(slot.nbytes, [])):
                     self.pool.release(slot)
 

@@ -81,18 +81,22 @@ class _Entry:
     conn: object
     command: object
     started: bool = False
+    result: object = None
 
 
 class TensorBusAgent:
     """Hub agent: serves ``world_size`` agent ranks on one device."""
 
     def __init__(self, world_size: int, path_naming_fn=None, device: str | torch.device = "cuda:0",
-                 heartbeat_interval: float = 0.2):
+                 heartbeat_interval: float = 0.2, zero_copy_single_chunk: bool = False):
         self.world_size = world_size
         self.device = torch.device(device)
         self.path_naming_fn = path_naming_fn or default_path_naming
         self.heartbeat_interval = heartbeat_interval
         self.wire = LoopbackWire(self.device if self.device.type == "cuda" else None)
+        # lent buckets are read from the worker's tensor at receive time, so a send that lends memory only
+        # completes once its receivers have unpacked (the reference's transfers end with a barrier as well)
+        self.wire.zero_copy_single_chunk = zero_copy_single_chunk
         self.pairs: dict[str, PairState] = {}
         self.batches: dict[str, BatchState] = {}
         self._inbox: queue.Queue = queue.Queue()
@@ -375,6 +379,11 @@ class TensorBusAgent:
                 )
             return True, None
         if cmd.transfer_type == "send":
+            if entry.started:  # already launched; this send lends tensor memory and waits for its receivers
+                gen = batch.send_count[rank]
+                if all(batch.recv_count.get(d, gen) >= gen for d in self._peers(buckets, "dst")):
+                    return True, entry.result
+                return False, None
             gen = batch.send_count[rank]
             for d in self._peers(buckets, "dst"):
                 if d in batch.recv_count and batch.recv_count[d] < gen:
@@ -385,6 +394,11 @@ class TensorBusAgent:
             batch.send_count[rank] = gen + 1
             for d in self._peers(buckets, "dst"):
                 batch.owed[d] = max(batch.owed.get(d, 0), gen + 1)
+            if self.wire.plan(buckets).lends_tensor_memory():
+                entry.started = True
+                entry.result = {"ms": (time.perf_counter() - t0) * 1e3}
+                self.stats["transfers"] += 1
+                return False, None
         else:
             gen = batch.recv_count[rank]
             for s in self._peers(buckets, "src"):

@@ -105,6 +105,7 @@ class ReshardJob:
     fill: object = "random"
     wire: LoopbackWire | None = None
     local_view: object = None  # optional ``(kind, tensor) -> view``: re-home a local shard inside another parent
+    zero_copy: bool = False  # lend contiguous single-chunk buckets instead of packing them (see LoopbackWire)
     source_locals: list[dict[int, torch.Tensor]] = field(default_factory=list, init=False)
     target_locals: list[dict[int, torch.Tensor]] = field(default_factory=list, init=False)
     globals_: list[torch.Tensor | None] = field(default_factory=list, init=False)
@@ -115,6 +116,8 @@ class ReshardJob:
         self.device = torch.device(self.device)
         if self.wire is None:
             self.wire = LoopbackWire(self.device)
+        if self.zero_copy:
+            self.wire.zero_copy_single_chunk = True
         send_chunks: dict[int, list] = {}
         recv_chunks: dict[int, list] = {}
         m2m_cache: dict[tuple, object] = {}

@@ -168,7 +168,7 @@ def _pool_specs():
     ]
 
 
-def producer_process(device, conn, rounds):
+def producer_process(device, conn, rounds, zero_copy=False):
     """Owns the source shards and the bucket pool: plans, exports the pool, packs each round."""
     try:
         import torch
@@ -178,9 +178,11 @@ def producer_process(device, conn, rounds):
         from helpers import cpu_fill
 
         setup_ptrace()
-        job = ReshardJob(_pool_specs(), device=device, bucket_size=32 * 1024, fill=cpu_fill)
+        job = ReshardJob(_pool_specs(), device=device, bucket_size=32 * 1024, fill=cpu_fill, zero_copy=zero_copy)
+        lent = 0
         for buckets in job.send_buckets.values():
-            job.wire.plan(buckets)  # assigns the slots
+            lent += len(job.wire.plan(buckets).lent)  # planning assigns the slots
+        assert (lent > 0) == bool(zero_copy)
         conn.send(("manifest", job.wire.export_manifest()))
         for round_ in range(rounds):
             if round_ > 0:

@@ -513,3 +513,32 @@ def test_transposed_parents_go_through_lds(gpu_device, dtype):
         assert_bit_equal(t, expected_target(spec, cpu_job.globals_[0], r), f"rank {r} closed form")
     assert gpu_job.wire.plan(gpu_job.send_buckets[0]).send_table.info().n_trans_tiles > 0
     assert gpu_job.wire.plan(gpu_job.recv_buckets[2]).recv_table.info().n_trans_tiles > 0
+
+
+def test_zero_copy_single_chunk_buckets(gpu_device):
+    """With the wire's zero-copy option, contiguous single-chunk buckets are lent: no pack launch, the
+    consumer unpacks straight from the source shard; everything else is packed as usual."""
+    specs, targets, _ = workloads.llama3_8b_fsdp8_to_tp2(n_layers=2, hidden=256, inter=896, kv=64, vocab=2056)
+    gpu_job = ReshardJob(specs, device=gpu_device, bucket_size=64 * 1024, target_ranks=targets, keep_globals=True,
+                         fill=cpu_fill, zero_copy=True)
+    cpu_job = ReshardJob(specs, device="cpu", bucket_size=64 * 1024, target_ranks=targets, keep_globals=True, fill=cpu_fill)
+    gpu_job.run(merge_launches=True)
+    run_oracle(cpu_job)
+    plans = [gpu_job.wire.plan(b) for b in gpu_job.send_buckets.values()]
+    lent = sum(len(p.lent) for p in plans)
+    packed = sum(1 for p in plans for s in p.steps if s[0] == "pack")
+    assert lent > 0 and packed > 0  # the big embedding / projection chunks are lent, bundled ones are packed
+    for i, spec in enumerate(specs):
+        for r, t in gpu_job.target_locals[i].items():
+            assert_bit_equal(t, cpu_job.target_locals[i][r], f"{spec.name} rank {r}")
+    # a second transfer with new values: lent buckets must deliver the new bytes too
+    for d in gpu_job.source_locals:
+        for t in d.values():
+            t.mul_(-1.0)
+    gpu_job.run(merge_launches=False)
+    for i, spec in enumerate(specs):
+        for r, t in gpu_job.target_locals[i].items():
+            assert_bit_equal(t, -cpu_job.target_locals[i][r], f"{spec.name} rank {r}, second transfer")
+    for p in plans:
+        gpu_job.wire.release(p.buckets)  # lent slots are not pool memory and must not enter its free list
+    assert all(not s.borrowed for free in gpu_job.wire.pool._free.values() for s in free)

@@ -198,7 +198,8 @@ def test_two_process_hipipc_handoff(gpu_device, tmp_path):
 
 
 @pytest.mark.gpu
-def test_bucket_pool_crosses_a_process_boundary(gpu_device):
+@pytest.mark.parametrize("zero_copy", [False, True], ids=["packed", "lent"])
+def test_bucket_pool_crosses_a_process_boundary(gpu_device, zero_copy):
     """The wire step as a same-GPU loopback between two processes: the producer packs into its pool, the
     consumer maps the pool with hipIpcOpenMemHandle and unpacks from it; two rounds with new values."""
     from bus_workers import consumer_process, producer_process
@@ -206,7 +207,7 @@ def test_bucket_pool_crosses_a_process_boundary(gpu_device):
     ctx = mp.get_context("spawn")
     a, b = ctx.Pipe()
     out_q = ctx.Queue()
-    procs = [ctx.Process(target=producer_process, args=(str(gpu_device), a, 2)),
+    procs = [ctx.Process(target=producer_process, args=(str(gpu_device), a, 2, zero_copy)),
              ctx.Process(target=consumer_process, args=(str(gpu_device), b, 2, out_q))]
     try:
         for p in procs:
@@ -252,3 +253,38 @@ def test_cleanup_returns_pool_slots(gpu_device, agent_factory):
     assert reserved[0] == reserved[1] == reserved[2], reserved
     for c in clients.values():
         c.close()
+
+
+@pytest.mark.gpu
+def test_agent_zero_copy_send_completes_only_after_receive(gpu_device, tmp_path):
+    """With lent buckets the receiver reads the worker's tensor itself, so a blocking send may only return
+    once the receiver has unpacked - otherwise the worker could overwrite bytes still to be read."""
+    agent = TensorBusAgent(2, path_naming(str(tmp_path)), device=gpu_device, heartbeat_interval=0.05,
+                           zero_copy_single_chunk=True)
+    agent.start_in_thread()
+    try:
+        naming = path_naming(str(tmp_path))
+        src = torch.arange(4096, dtype=torch.float32, device=gpu_device).reshape(64, 64)
+        tgt = torch.zeros(64, 64, device=gpu_device)
+        clients = {r: _client(naming, r, connection_timeout=5) for r in range(2)}
+
+        def reg(r):
+            clients[r].init_pair("w", "a" if r == 0 else "b", "b" if r == 0 else "a", 1, device_mesh=torch.arange(1),
+                                 placements=(Replicate(),))
+            return clients[r].register_tensors("b", [((src if r == 0 else tgt), "w")], bucket_size=None)
+
+        handlers = run_ranks(reg, range(2))
+        assert agent.wire.plan(agent.batches["b"].send_buckets[0]).lends_tensor_memory()
+        sem = handlers[0].transfer("send", blocking=False)
+        with pytest.raises(Exception):
+            sem.acquire(timeout=0.5)  # nobody has received yet: the send must still be pending
+        handlers[1].transfer("recv", blocking=True, timeout=20)
+        sem.acquire(timeout=20)  # now it completes
+        torch.cuda.synchronize()
+        assert torch.equal(tgt, src)
+        for h in handlers.values():
+            h.close()
+        for c in clients.values():
+            c.close()
+    finally:
+        agent.close()
