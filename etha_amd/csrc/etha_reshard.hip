@@ -91,6 +91,7 @@ constexpr uint32_t kMetaDtbShift = 12;  // 4 bits: ETHA_* dtype, b side
 constexpr uint32_t kMetaCvt = 1u << 16; // converting move (else byte move)
 constexpr uint32_t kMetaVec = 1u << 17; // converting move handles the full vector (else 1 element)
 constexpr uint32_t kMetaSkew = 1u << 18; // byte move of 16-byte units whose a-side address is not 16-byte aligned
+constexpr uint32_t kMetaSkewB = 1u << 19; // ... whose b-side address is not 16-byte aligned
 
 // ---- typed vector access ----------------------------------------------------------------------
 typedef uint32_t u32x2 __attribute__((ext_vector_type(2)));
@@ -197,11 +198,15 @@ template <bool REV>
 __device__ __forceinline__ void move_unit(uint32_t meta, uint64_t a, uint64_t b) {
   const uint64_t src = REV ? b : a, dst = REV ? a : b;
   if (!(meta & kMetaCvt)) {
-    if (meta & kMetaSkew) {  // a side unaligned, b side aligned
-      if (REV)
-        __builtin_nontemporal_store(ld_stream<u32x4>(b), reinterpret_cast<ETHA_GLOBAL u32x4_any*>(a));
+    if (meta & (kMetaSkew | kMetaSkewB)) {  // 16-byte units; the flagged sides may sit at any byte address
+      const bool any_src = (meta & (REV ? kMetaSkewB : kMetaSkew)) != 0;
+      const bool any_dst = (meta & (REV ? kMetaSkew : kMetaSkewB)) != 0;
+      const u32x4 v = any_src ? __builtin_nontemporal_load(reinterpret_cast<const ETHA_GLOBAL u32x4_any*>(src))
+                              : ld_stream<u32x4>(src);
+      if (any_dst)
+        __builtin_nontemporal_store(v, reinterpret_cast<ETHA_GLOBAL u32x4_any*>(dst));
       else
-        st_stream<u32x4>(b, __builtin_nontemporal_load(reinterpret_cast<const ETHA_GLOBAL u32x4_any*>(a)));
+        st_stream<u32x4>(dst, v);
       return;
     }
     switch (meta & 15u) {
@@ -646,8 +651,10 @@ int compile_pair(Builder& bld, uint32_t idx, const Region& A0, const Region& B0,
   int ua_log2, ub_log2;
   uint64_t run_units;
   uint32_t meta = 0;
+  uint64_t mask_a = 0, mask_b = 0;  // OR of every row start (base and outer strides) per side
   {
-    uint64_t mask_a = red.n_peers ? 0 : A0.base, mask_b = B0.base;
+    mask_a = red.n_peers ? 0 : A0.base;
+    mask_b = B0.base;
     for (uint64_t p : align_bases) mask_a |= p + A0.base;  // reduce: A0.base is an offset from each peer base
     for (int i = 0; i < k; i++) {
       mask_a |= (uint64_t)(sa[i] < 0 ? -sa[i] : sa[i]);
@@ -736,8 +743,9 @@ int compile_pair(Builder& bld, uint32_t idx, const Region& A0, const Region& B0,
     return ETHA_OK;
   }
 
-  // 5. tiles.  Long or 256-multiple rows (and single runs) become run tiles; other shapes become
+  // 5. tiles.  Long or tile-multiple rows (and single runs) become run tiles; other shapes become
   //    row tiles over the innermost remaining dim; dims further out are unrolled here.
+  auto emit = [&](uint64_t base_a, uint64_t base_b, uint64_t run_units, uint64_t ua, uint64_t ub, uint32_t meta) -> int {
   const bool use_rows = red.n_peers != 0 || (k > 0 && run_units % kTileThreads != 0 && run_units < 4 * kTileThreads);
   if (run_units > 0xffffffffull && use_rows && k > 0)
     return fail(ETHA_ERR_UNSUPPORTED, "chunk %u: row longer than 2^32 units", idx);
@@ -745,7 +753,7 @@ int compile_pair(Builder& bld, uint32_t idx, const Region& A0, const Region& B0,
   int64_t pos[ETHA_MAX_NDIM] = {0};
   uint64_t off_a = 0, off_b = 0;  // wraps mod 2^64 for negative strides, which is fine
   while (true) {
-    const uint64_t a0 = A0.base + off_a, b0 = B0.base + off_b;
+    const uint64_t a0 = base_a + off_a, b0 = base_b + off_b;
     if (!use_rows) {
       for (uint64_t q = 0; q < run_units; q += kTileThreads) {
         RunTile t;
@@ -800,6 +808,30 @@ int compile_pair(Builder& bld, uint32_t idx, const Region& A0, const Region& B0,
     if (d < 0) break;
   }
   return ETHA_OK;
+  };  // emit
+
+  // Byte moves whose rows are not a whole number of aligned 16-byte units (odd row lengths, short skewed
+  // rows): instead of element-sized units, every row is split into a body of 16-byte units - accessed
+  // unaligned on the sides whose row starts are not 16-byte aligned - and a remainder of < 16 bytes in
+  // narrow units.  Both parts are ordinary tile sets over the same rows.
+  if (!cvt && !red.n_peers && ua_log2 < 4 && run_elems * (uint64_t)esa >= 32) {
+    const uint64_t run_bytes = run_elems * (uint64_t)esa;
+    const uint64_t body_units = run_bytes / 16, rem_bytes = run_bytes % 16;
+    const uint32_t dt_bits = (dta << kMetaDtaShift) | (dtb << kMetaDtbShift);
+    // a row's start is aligned only if base, outer strides AND (for the 2nd, 3rd.. rows of a collapsed run) hold
+    const uint32_t body_meta = dt_bits | (4u << kMetaUaShift) | (4u << kMetaUbShift) | ((mask_a & 15) ? kMetaSkew : 0u) |
+                               ((mask_b & 15) ? kMetaSkewB : 0u);
+    if (!(body_meta & (kMetaSkew | kMetaSkewB)) && rem_bytes == 0)
+      return fail(ETHA_ERR_INVALID, "chunk %u: internal alignment classification error", idx);
+    int rc = emit(A0.base, B0.base, body_units, 16, 16, body_meta);
+    if (rc != ETHA_OK || rem_bytes == 0) return rc;
+    uint64_t m = mask_a | mask_b | rem_bytes | 16;
+    int v = 3;
+    while (v > 0 && (m & ((1ull << v) - 1))) v--;
+    const uint32_t rem_meta = dt_bits | ((uint32_t)v << kMetaUaShift) | ((uint32_t)v << kMetaUbShift);
+    return emit(A0.base + body_units * 16, B0.base + body_units * 16, rem_bytes >> v, 1ull << v, 1ull << v, rem_meta);
+  }
+  return emit(A0.base, B0.base, run_units, ua, ub, meta);
 }
 
 }  // namespace

@@ -120,6 +120,28 @@ def test_skewed_chunks_use_wide_units():
     assert np.all(body["b"] % 16 == 0) and np.all(body["a"] % 16 == 10)
 
 
+def test_odd_row_lengths_use_16_byte_bodies():
+    """Rows of 150 bytes (75 bf16) at a 2-byte-aligned pitch: 9 body units + 3 remainder units per row
+    instead of 75 element units."""
+    rows, cols, es = 200, 75, 2
+    arena = HostArena(4 * rows * 160 * es + 65536)
+    t = arena.alloc(rows * 81 * es)
+    arena.bytes_at(t, rows * 81 * es)[:] = rs.randint(0, 256, rows * 81 * es)
+    b = arena.alloc(rows * cols * es)
+    d = _mk_desc(t, t, t + rows * 81 * es, b, b, b + rows * cols * es, (0, 3), (rows, cols), (81, 1), nat.BF16, nat.BF16)
+    table = nat.Table.create(d.reshape(1), upload=False)
+    run, row = table.tiles()
+    units = int(run["n"].sum()) + int(row["n"].sum())
+    assert units == rows * (9 + 3)
+    execute(table, arena, "pack")
+    want = np.zeros(rows * cols * es, dtype=np.uint8)
+    scratch = np.zeros(rows * cols * es, dtype=np.uint8)
+    oc = co.make_chunk(t, (0, 3), (rows, cols), (81, 1), co.BF16, co.BF16, bucket_off=0)
+    assert co.lib().oracle_pack_bucket(oc, 1, want.ctypes.data, scratch.ctypes.data) == 0
+    assert np.array_equal(arena.bytes_at(b, rows * cols * es), want)
+    assert arena.writes.max() == 1 and int(arena.writes.sum()) == rows * cols * es
+
+
 def test_bucket_ranges_and_many_chunks():
     """Chunk ranges select exactly their own tiles; un-padded prefix-sum offsets inside one bucket."""
     shapes = [(40, 24), (7, 5), (128,), (3, 9, 11), (256, 8)]

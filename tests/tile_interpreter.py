@@ -124,10 +124,10 @@ def execute(table, arena, direction: str, first: int = 0, count: int | None = No
             ua, ub = 1 << (int(m) & 15), 1 << ((int(m) >> 4) & 15)
             dta, dtb = (int(m) >> 8) & 15, (int(m) >> 12) & 15
             cvt, vec = bool(int(m) & (1 << 16)), bool(int(m) & (1 << 17))
-            skew = bool(int(m) & (1 << 18))
-            assert skew or np.all(a[sel] % ua == 0), "misaligned vector access on the a side"
-            assert np.all(b[sel] % ub == 0), "misaligned vector access on the b side"
-            assert not skew or (ua == 16 and ub == 16 and not cvt)
+            skew_a, skew_b = bool(int(m) & (1 << 18)), bool(int(m) & (1 << 19))
+            assert skew_a or np.all(a[sel] % ua == 0), "misaligned vector access on the a side"
+            assert skew_b or np.all(b[sel] % ub == 0), "misaligned vector access on the b side"
+            assert not (skew_a or skew_b) or (ua == 16 and ub == 16 and not cvt)
             reduce = row_idx[sel][0] >= 0 and int(row_tiles["n_peers"][row_idx[sel][0]]) > 0
             if reduce:
                 _reduce_units(arena, mem, row_tiles, row_idx[sel], a[sel], b[sel], ua, ub, dta, dtb, peers)
