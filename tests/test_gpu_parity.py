@@ -324,12 +324,15 @@ def test_moe_experts_and_uneven_vocab_small(gpu_device):
 
 # ---- full size: size-independent properties ------------------------------------------------------------
 
-def test_llama3_8b_full_size_properties(gpu_device):
+@pytest.mark.parametrize("bucket_size", [64 << 20, None, 1 << 20, 1 << 30], ids=["64MiB", "unbucketed", "1MiB", "1GiB"])
+def test_llama3_8b_full_size_properties(gpu_device, bucket_size):
     """Config 2 at its real size: every target shard equals its slice of the global tensor, sources
-    are untouched, and the step is idempotent."""
-    specs, targets, bucket = workloads.llama3_8b_fsdp8_to_tp2()
-    job = ReshardJob(specs, device=gpu_device, bucket_size=bucket, target_ranks=targets, keep_globals=True)
+    are untouched, and the step is idempotent - for the configured 64 MiB buckets and for other bucket sizes."""
+    specs, targets, _ = workloads.llama3_8b_fsdp8_to_tp2()
+    job = ReshardJob(specs, device=gpu_device, bucket_size=bucket_size, target_ranks=targets, keep_globals=True)
     assert job.payload_bytes() == 8_030_519_296 and job.counts()["recv_chunks"] == 1672
+    if bucket_size is None:
+        assert job.counts()["recv_buckets"] == 1672
     src_sums = [{r: t.view(torch.int16).sum(dtype=torch.int64).item() for r, t in d.items()} for d in job.source_locals]
     job.run(merge_launches=True)
     from etha_amd.layout import local_shard, mesh_coord
