@@ -51,6 +51,46 @@ def parse_args():
     return ap.parse_args()
 
 
+def _cheap_fill(spec):  # values do not affect timing; avoid minutes of CPU randn
+    import torch
+
+    n = 1
+    for s in spec.shape:
+        n *= s
+    return (torch.arange(n, dtype=torch.int32) % 251).to(spec.source_dtype).reshape(spec.shape)
+
+
+def _cpu_job(workload: str):
+    """The whole workload staged on the CPU; module-level so that spawned rank processes can build it too."""
+    from etha_amd import workloads
+    from etha_amd.world import ReshardJob
+
+    specs, targets, bucket = workloads.WORKLOADS[workload]()
+    return ReshardJob(specs, device="cpu", bucket_size=bucket, target_ranks=targets, fill=_cheap_fill)
+
+
+def gloo_baseline(workload: str, passes: int = 20):
+    """The same CPU path with one process per rank and gloo isend/irecv/broadcast as the wire: the
+    reference's own CPU way of running a redistribute (its tests/test_communication_cpu.py:25-118)."""
+    from oracle import gloo_redistribute
+
+    job = _cpu_job(workload)
+    ranks = {int(r) for spec in job.specs for mesh in (spec.source_mesh, spec.target_mesh)
+             for r in __import__("numpy").asarray(mesh).reshape(-1)}
+    world = max(ranks) + 1
+    _, seconds, threads = gloo_redistribute.run(_cpu_job, (workload,), world, passes=passes + 1, timeout=300.0)
+    seconds = sorted(seconds[1:])
+    med = seconds[len(seconds) // 2]
+    return {
+        "value": job.payload_bytes() / med / 1e9,
+        "unit": "GB/s",
+        "processes": world,
+        "threads_per_process": threads,
+        "ms_per_transfer": med * 1e3,
+        "sample": f"whole workload, median of {len(seconds)} transfers between barriers",
+    }
+
+
 def cpu_baseline(workload: str, layers: int, seconds: float):
     """The oracle's op-for-op restatement of the reference path, timed on this host's cores."""
     import torch
@@ -66,13 +106,7 @@ def cpu_baseline(workload: str, layers: int, seconds: float):
         specs, targets, bucket = workloads.WORKLOADS[workload]()
         sample = "whole workload"
 
-    def cheap_fill(spec):  # values do not affect timing; avoid minutes of CPU randn
-        n = 1
-        for s in spec.shape:
-            n *= s
-        return (torch.arange(n, dtype=torch.int32) % 251).to(spec.source_dtype).reshape(spec.shape)
-
-    job = ReshardJob(specs, device="cpu", bucket_size=bucket, target_ranks=targets, fill=cheap_fill)
+    job = ReshardJob(specs, device="cpu", bucket_size=bucket, target_ranks=targets, fill=_cheap_fill)
     payload = job.payload_bytes()
 
     def one_pass():
@@ -270,6 +304,8 @@ def main():
         out["calibration_copy"] = {"bytes_read": 1 << 30, "bytes_written": 1 << 30, "launches": 3}
     if not args.no_cpu_baseline:
         out["cpu_baseline"] = cpu_baseline(args.workload, args.cpu_layers, args.cpu_seconds)
+        if args.workload == "single_fp32_shard0_to_shard1":
+            out["cpu_baseline"]["gloo"] = gloo_baseline(args.workload)
     print(json.dumps(out))
 
 

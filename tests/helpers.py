@@ -33,6 +33,12 @@ def mirror_partials(gpu_job: ReshardJob, cpu_job: ReshardJob) -> None:
             t.copy_(g_src[r].cpu())
 
 
+def make_cpu_job(specs, bucket_size, target_ranks=None) -> ReshardJob:
+    """A CPU-resident job with seeded CPU data; module-level so that spawned rank processes can call it."""
+    return ReshardJob(clone_specs(specs), device="cpu", bucket_size=bucket_size, target_ranks=target_ranks,
+                      keep_globals=True, fill=cpu_fill)
+
+
 def run_oracle(cpu_job: ReshardJob) -> None:
     """Execute a CPU-resident job with the oracle's restatement of the reference path."""
     box = reference_path.Mailbox()

@@ -335,7 +335,7 @@ def test_llama3_8b_full_size_properties(gpu_device, bucket_size):
         assert job.counts()["recv_buckets"] == 1672
     src_sums = [{r: t.view(torch.int16).sum(dtype=torch.int64).item() for r, t in d.items()} for d in job.source_locals]
     job.run(merge_launches=True)
-    from etha_amd.layout import local_shard, mesh_coord
+    from etha_amd.layout import local_shard
 
     def check():
         for i, spec in enumerate(specs):
