@@ -352,6 +352,75 @@ def test_llama3_8b_full_size_properties(gpu_device, bucket_size):
     check()
 
 
+def _check_targets_against_global(job, specs, cast=None):
+    import numpy as np
+
+    from oracle.dtensor_layout import local_shard, mesh_coord  # the pinned convention, not the product's planner
+
+    for i, spec in enumerate(specs):
+        mesh = np.asarray(spec.target_mesh)
+        flat = [int(x) for x in mesh.reshape(-1)]
+        for r, got in job.target_locals[i].items():
+            want = local_shard(job.globals_[i], mesh.shape, spec.target_placements, mesh_coord(mesh.shape, flat.index(r)))
+            if cast is not None:
+                want = want.to(cast)
+            assert got.shape == want.shape and got.dtype == want.dtype, spec.name
+            assert torch.equal(got.contiguous().view(torch.uint8), want.contiguous().view(torch.uint8)), (spec.name, r)
+
+
+def test_llama3_8b_fp32_to_bf16_full_size_properties(gpu_device):
+    """Config 2 with fp32 source shards and bf16 targets at full size: every target shard is the RNE
+    bf16 cast of its slice of the fp32 global tensor (torch's device cast is the independent check)."""
+    specs, targets, bucket = workloads.llama3_8b_fsdp8_to_tp2_fp32_to_bf16()
+    job = ReshardJob(specs, device=gpu_device, bucket_size=bucket, target_ranks=targets, keep_globals=True)
+    assert job.payload_bytes() == 8_030_519_296
+    job.run(merge_launches=True)
+    _check_targets_against_global(job, specs, cast=torch.bfloat16)
+
+
+def test_many_small_2d_to_replicate_full_size_properties(gpu_device):
+    """Config 3 at full size: the replicated target equals the global tensor; both launch granularities."""
+    specs, targets, bucket = workloads.many_small_2d_to_replicate()
+    job = ReshardJob(specs, device=gpu_device, bucket_size=bucket, target_ranks=targets, keep_globals=True)
+    assert len(job.send_buckets) == 8  # one channel per source rank
+    for merge in (True, False):
+        for d in job.target_locals:
+            for t in d.values():
+                t.zero_()
+        job.run(merge_launches=merge)
+        _check_targets_against_global(job, specs)
+
+
+def test_partial4_to_shard2_full_size_properties(gpu_device):
+    """Config 4 at full size: the target shard is the fp32 rank-order sum of the four partials, cast once
+    to bf16 - recomputed here with torch device ops (IEEE fp32 adds, RNE cast), so 0 ulp is required
+    where 1 bf16 ulp is allowed; the partials are not modified."""
+    specs, targets, bucket = workloads.partial4_to_shard2()
+    job = ReshardJob(specs, device=gpu_device, bucket_size=bucket, target_ranks=targets)
+    sums = [{r: t.view(torch.int16).sum(dtype=torch.int64).item() for r, t in d.items()} for d in job.source_locals]
+    job.run(merge_launches=True)
+    for i, spec in enumerate(specs):
+        acc = job.source_locals[i][0][:4096].float()
+        for r in (1, 2, 3):
+            acc = acc + job.source_locals[i][r][:4096].float()
+        want = acc.to(torch.bfloat16)
+        got = job.target_locals[i][4]
+        ulp = (got.view(torch.int16).int() - want.view(torch.int16).int()).abs().max().item()
+        assert ulp == 0, (spec.name, ulp)
+        for r, t in job.source_locals[i].items():
+            assert t.view(torch.int16).sum(dtype=torch.int64).item() == sums[i][r], "partial mutated"
+
+
+def test_moe_experts_and_uneven_vocab_full_size_properties(gpu_device):
+    """Config 5 at full size, all four target ranks: every shard (through buckets or the direct
+    same-rank path) equals its slice of the global tensor, uneven 151936-row embedding included."""
+    specs, _, bucket = workloads.moe_experts_and_uneven_vocab()
+    job = ReshardJob(specs, device=gpu_device, bucket_size=bucket, target_ranks=[0, 1, 2, 3], keep_globals=True)
+    assert [t.shape[0] for t in job.source_locals[3].values()] == [25323] * 5 + [25321]
+    job.run(merge_launches=True)
+    _check_targets_against_global(job, specs)
+
+
 def test_per_bucket_launches_on_side_streams(gpu_device):
     """Fan-out over side streams (fork/join with events) gives the same bytes as one stream."""
     specs, targets, _ = workloads.llama3_8b_fsdp8_to_tp2(n_layers=3, hidden=256, inter=896, kv=64, vocab=2056)
