@@ -1,11 +1,11 @@
 // MI355X (gfx950) redistribute hot path: pack / unpack / self-copy / Partial reduce-pack.
 //
 // Design.  These are HBM-bound byte movers.  On MI355X a plain copy runs fastest when every
-// work-item moves exactly one 16-byte vector, workgroups are small (256 work-items = 4 KiB),
+// work-item moves exactly one 16-byte vector, workgroups are one wavefront (64 work-items = 1 KiB),
 // the grid is huge and ordered by address, and both sides use nontemporal accesses; loops and
 // several vectors per work-item lose 10-30 %.  So all chunk geometry (slices, strides, bucket
 // offsets, dtype pairs, alignment classes) is resolved once on the host into a flat
-// device-resident *tile program*: one entry per workgroup holding absolute addresses.  A
+// device-resident *tile program*: one entry per 16 workgroups holding absolute addresses.  A
 // workgroup does one scalar table load, each work-item one vector load and one vector store.  Only
 // chunks whose contiguous dim differs between the two sides (transposes) are staged through LDS.
 //
@@ -34,6 +34,9 @@ namespace {
 #endif
 #ifndef ETHA_BLOCK_THREADS
 #define ETHA_BLOCK_THREADS 64
+#endif
+#ifndef ETHA_SKEW_PEEL_MIN_BYTES
+#define ETHA_SKEW_PEEL_MIN_BYTES (256 * 1024)
 #endif
 // One table entry (tile) describes kTileThreads units; it is executed by kBlocksPerTile workgroups of
 // kBlockThreads work-items (one wavefront each).  Wave-sized workgroups schedule best; the coarser
@@ -230,7 +233,7 @@ __device__ __forceinline__ void move_unit(uint32_t meta, uint64_t a, uint64_t b)
 }
 
 __device__ __forceinline__ void row_position(const RowTile& t, uint32_t tid, uint32_t& r, uint32_t& c) {
-  const uint32_t q = t.c0 + tid;  // c0 < run and tid < 256, so q < 2*run whenever run >= 256
+  const uint32_t q = t.c0 + tid;  // c0 < run and tid < kTileThreads, so q < 2*run whenever run >= kTileThreads
   if (t.run >= kTileThreads) {
     r = q >= t.run ? 1u : 0u;
     c = q - (r ? t.run : 0u);
@@ -689,10 +692,12 @@ int compile_pair(Builder& bld, uint32_t idx, const Region& A0, const Region& B0,
   const uint64_t ua = 1ull << ua_log2, ub = 1ull << ub_log2;
 
   // Skewed byte moves: the two sides disagree on their position inside a 16-byte vector (typically
-  // a chunk that follows an odd-sized one in an un-padded bucket).  Long runs are peeled per run so
+  // a chunk that follows an odd-sized one in an un-padded bucket).  Very long runs are peeled per run so
   // that the b side is 16-byte aligned: a head and a tail of < 16 bytes go through narrow tiles, the
-  // body moves in 16-byte units whose a-side access is unaligned.
-  constexpr uint64_t kSkewMinRunBytes = 512;
+  // body moves in 16-byte units whose a-side access is unaligned.  Peeling costs three tile sets per
+  // run, so it only pays for runs of many tiles (measured: +5 % from 256 KiB up, 20x slower than the
+  // row split below at 512-byte runs); shorter runs take the row split, unaligned on both sides.
+  constexpr uint64_t kSkewMinRunBytes = ETHA_SKEW_PEEL_MIN_BYTES;
   if (!cvt && !red.n_peers && ua_log2 < 4 && run_elems * (uint64_t)esa >= kSkewMinRunBytes) {
     const uint64_t run_bytes = run_elems * (uint64_t)esa;
     const uint32_t dt_bits = (dta << kMetaDtaShift) | (dtb << kMetaDtbShift);

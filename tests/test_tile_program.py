@@ -45,6 +45,8 @@ GEOMETRIES = [
     ((64, 256), None, (0, 128), (64, 128), nat.F16, nat.BF16, 0),
     ((3,), None, (0,), (3,), nat.F32, nat.F32, 0),
     ((40000,), None, (3,), (39990,), nat.BF16, nat.BF16, 0),             # long run, the two sides skewed
+    ((200000,), None, (3,), (199990,), nat.BF16, nat.BF16, 0),           # >= 256 KiB skewed run: peeled per run
+    ((3, 140000), None, (0, 1), (3, 139999), nat.BF16, nat.BF16, 2),     # peeled rows of 279998 bytes
     ((64, 1024), None, (0, 5), (64, 777), nat.BF16, nat.BF16, 2),        # skewed rows of 1554 bytes
     ((9000,), None, (1,), (8990,), nat.B8, nat.B8, 1),                   # byte elements, odd everything
     ((30, 600), None, (0, 1), (30, 599), nat.F32, nat.F32, 4),           # dword-aligned skew
