@@ -93,8 +93,9 @@ constexpr uint32_t kMetaDtaShift = 8;   // 4 bits: ETHA_* dtype, a side
 constexpr uint32_t kMetaDtbShift = 12;  // 4 bits: ETHA_* dtype, b side
 constexpr uint32_t kMetaCvt = 1u << 16; // converting move (else byte move)
 constexpr uint32_t kMetaVec = 1u << 17; // converting move handles the full vector (else 1 element)
-constexpr uint32_t kMetaSkew = 1u << 18; // byte move of 16-byte units whose a-side address is not 16-byte aligned
-constexpr uint32_t kMetaSkewB = 1u << 19; // ... whose b-side address is not 16-byte aligned
+constexpr uint32_t kMetaSkew = 1u << 18;  // a-side addresses are not all multiples of the a-side unit size
+constexpr uint32_t kMetaSkewB = 1u << 19; // same for the b side (both are bookkeeping for checkers: the kernel's
+                                          // accesses are legal at any element-aligned address)
 
 // ---- typed vector access ----------------------------------------------------------------------
 typedef uint32_t u32x2 __attribute__((ext_vector_type(2)));
@@ -111,21 +112,27 @@ template <typename V>
 __device__ __forceinline__ void st_stream(uint64_t addr, V v) {
   __builtin_nontemporal_store(v, reinterpret_cast<ETHA_GLOBAL V*>(addr));
 }
+// The device runs in unaligned-access mode: a 4/8/16-byte access may sit at any byte address and is still
+// one instruction, so vector types are declared with the weakest alignment their use can meet.  The
+// host decides per tile whether addresses are in fact aligned (the fast case) and records it in the
+// meta bits; consecutive work-items cover one contiguous byte range either way.
+typedef u32x4 u32x4_any __attribute__((aligned(1)));
+typedef u32x2 u32x2_any __attribute__((aligned(1)));
+typedef uint32_t u32_any __attribute__((aligned(1)));
+typedef uint16_t u16_any __attribute__((aligned(1)));
 template <typename V>
 __device__ __forceinline__ void copy_as(uint64_t src, uint64_t dst) {
   st_stream<V>(dst, ld_stream<V>(src));
 }
-// 16-byte access at any byte address (the device runs in unaligned-access mode; consecutive
-// work-items still cover one contiguous byte range, so the memory system sees full lines)
-typedef u32x4 u32x4_any __attribute__((aligned(1)));
 
-// N elements of storage type T as one naturally aligned vector.
+// N elements of storage type T as one vector that is only element-aligned.
 template <typename T, int N>
 struct Pack {
   typedef T vec __attribute__((ext_vector_type(N)));
+  typedef vec vec_mem __attribute__((aligned(sizeof(T))));
   vec v;
-  __device__ __forceinline__ void load(uint64_t addr) { v = ld_stream<vec>(addr); }
-  __device__ __forceinline__ void store(uint64_t addr) const { st_stream<vec>(addr, v); }
+  __device__ __forceinline__ void load(uint64_t addr) { v = ld_stream<vec_mem>(addr); }
+  __device__ __forceinline__ void store(uint64_t addr) const { st_stream<vec_mem>(addr, v); }
   __device__ __forceinline__ T get(int i) const { return v[i]; }
   __device__ __forceinline__ void set(int i, T x) { v[i] = x; }
 };
@@ -201,22 +208,11 @@ template <bool REV>
 __device__ __forceinline__ void move_unit(uint32_t meta, uint64_t a, uint64_t b) {
   const uint64_t src = REV ? b : a, dst = REV ? a : b;
   if (!(meta & kMetaCvt)) {
-    if (meta & (kMetaSkew | kMetaSkewB)) {  // 16-byte units; the flagged sides may sit at any byte address
-      const bool any_src = (meta & (REV ? kMetaSkewB : kMetaSkew)) != 0;
-      const bool any_dst = (meta & (REV ? kMetaSkew : kMetaSkewB)) != 0;
-      const u32x4 v = any_src ? __builtin_nontemporal_load(reinterpret_cast<const ETHA_GLOBAL u32x4_any*>(src))
-                              : ld_stream<u32x4>(src);
-      if (any_dst)
-        __builtin_nontemporal_store(v, reinterpret_cast<ETHA_GLOBAL u32x4_any*>(dst));
-      else
-        st_stream<u32x4>(dst, v);
-      return;
-    }
     switch (meta & 15u) {
-      case 4: copy_as<u32x4>(src, dst); break;
-      case 3: copy_as<u32x2>(src, dst); break;
-      case 2: copy_as<uint32_t>(src, dst); break;
-      case 1: copy_as<uint16_t>(src, dst); break;
+      case 4: copy_as<u32x4_any>(src, dst); break;
+      case 3: copy_as<u32x2_any>(src, dst); break;
+      case 2: copy_as<u32_any>(src, dst); break;
+      case 1: copy_as<u16_any>(src, dst); break;
       default: copy_as<uint8_t>(src, dst); break;
     }
     return;
@@ -650,11 +646,17 @@ int compile_pair(Builder& bld, uint32_t idx, const Region& A0, const Region& B0,
     }
   }
 
-  // 4. unit size: the widest vector every row start and the run length allow
+  // 4. unit size.  Lengths decide it, not addresses: the kernel's accesses are legal at any (element-aligned)
+  //    address, so a misaligned side only sets a meta flag.  Byte moves use the widest power of two (<= 16
+  //    bytes) that divides the run; converting and reducing moves use whole vectors of 16 / max(element
+  //    size) elements when the run is a multiple of that, else single elements.  Runs that are not a whole
+  //    number of wide units are split further down into a wide body and a narrow remainder.
   int ua_log2, ub_log2;
   uint64_t run_units;
   uint32_t meta = 0;
   uint64_t mask_a = 0, mask_b = 0;  // OR of every row start (base and outer strides) per side
+  const bool plain = !cvt && !red.n_peers;
+  const int epv_full = 16 / (esa > esb ? esa : esb);  // elements per full vector of a converting move
   {
     mask_a = red.n_peers ? 0 : A0.base;
     mask_b = B0.base;
@@ -663,23 +665,16 @@ int compile_pair(Builder& bld, uint32_t idx, const Region& A0, const Region& B0,
       mask_a |= (uint64_t)(sa[i] < 0 ? -sa[i] : sa[i]);
       mask_b |= (uint64_t)(sb[i] < 0 ? -sb[i] : sb[i]);
     }
-    if (!cvt && !red.n_peers) {
+    if (plain) {
       const uint64_t run_bytes = run_elems * (uint64_t)esa;
-      uint64_t m = mask_a | mask_b | run_bytes;
       int v = 4;
-      while (v > 0 && (m & ((1ull << v) - 1))) v--;
+      while (v > 0 && (run_bytes & ((1ull << v) - 1))) v--;
       ua_log2 = ub_log2 = v;
       run_units = run_bytes >> v;
     } else {
-      const int big = esa > esb ? esa : esb;
-      int epv = 16 / big;
-      const bool vec_ok = (run_elems % (uint64_t)epv == 0) && (mask_a % (uint64_t)(epv * esa) == 0) &&
-                          (mask_b % (uint64_t)(epv * esb) == 0);
-      if (!vec_ok) {
-        epv = 1;
-        if (mask_a % (uint64_t)esa || mask_b % (uint64_t)esb)
-          return fail(ETHA_ERR_INVALID, "chunk %u: element address not aligned to its dtype", idx);
-      }
+      if (mask_a % (uint64_t)esa || mask_b % (uint64_t)esb)
+        return fail(ETHA_ERR_INVALID, "chunk %u: element address not aligned to its dtype", idx);
+      const int epv = run_elems % (uint64_t)epv_full == 0 ? epv_full : 1;
       ua_log2 = log2u((uint64_t)(epv * esa));
       ub_log2 = log2u((uint64_t)(epv * esb));
       run_units = run_elems / (uint64_t)epv;
@@ -687,8 +682,11 @@ int compile_pair(Builder& bld, uint32_t idx, const Region& A0, const Region& B0,
       if (epv > 1) meta |= kMetaVec;
     }
   }
-  meta |= ((uint32_t)ua_log2 << kMetaUaShift) | ((uint32_t)ub_log2 << kMetaUbShift) | (dta << kMetaDtaShift) |
-          (dtb << kMetaDtbShift);
+  const uint32_t dt_bits = (dta << kMetaDtaShift) | (dtb << kMetaDtbShift);
+  auto skew_bits = [&](int ua_l2, int ub_l2) -> uint32_t {
+    return ((mask_a & ((1ull << ua_l2) - 1)) ? kMetaSkew : 0u) | ((mask_b & ((1ull << ub_l2) - 1)) ? kMetaSkewB : 0u);
+  };
+  meta |= ((uint32_t)ua_log2 << kMetaUaShift) | ((uint32_t)ub_log2 << kMetaUbShift) | dt_bits | skew_bits(ua_log2, ub_log2);
   const uint64_t ua = 1ull << ua_log2, ub = 1ull << ub_log2;
 
   // Skewed byte moves: the two sides disagree on their position inside a 16-byte vector (typically
@@ -698,20 +696,20 @@ int compile_pair(Builder& bld, uint32_t idx, const Region& A0, const Region& B0,
   // run, so it only pays for runs of many tiles (measured: +5 % from 256 KiB up, 20x slower than the
   // row split below at 512-byte runs); shorter runs take the row split, unaligned on both sides.
   constexpr uint64_t kSkewMinRunBytes = ETHA_SKEW_PEEL_MIN_BYTES;
-  if (!cvt && !red.n_peers && ua_log2 < 4 && run_elems * (uint64_t)esa >= kSkewMinRunBytes) {
+  if (plain && ((mask_a | mask_b) & 15) && run_elems * (uint64_t)esa >= kSkewMinRunBytes) {
     const uint64_t run_bytes = run_elems * (uint64_t)esa;
-    const uint32_t dt_bits = (dta << kMetaDtaShift) | (dtb << kMetaDtbShift);
     const uint32_t body_meta = dt_bits | (4u << kMetaUaShift) | (4u << kMetaUbShift) | kMetaSkew;
     auto narrow = [&](uint64_t a, uint64_t b, uint64_t bytes) {  // bytes < 16
       if (!bytes) return;
-      uint64_t m = a | b | bytes;
       int v = 3;
-      while (v > 0 && (m & ((1ull << v) - 1))) v--;
+      while (v > 0 && (bytes & ((1ull << v) - 1))) v--;
+      const uint64_t low = (1ull << v) - 1;
       RunTile t;
       t.a = a;
       t.b = b;
       t.n = (uint32_t)(bytes >> v);
-      t.meta = dt_bits | ((uint32_t)v << kMetaUaShift) | ((uint32_t)v << kMetaUbShift);
+      t.meta = dt_bits | ((uint32_t)v << kMetaUaShift) | ((uint32_t)v << kMetaUbShift) | ((a & low) ? kMetaSkew : 0u) |
+               ((b & low) ? kMetaSkewB : 0u);
       bld.run.push_back(t);
     };
     int64_t pos[ETHA_MAX_NDIM] = {0};
@@ -815,26 +813,33 @@ int compile_pair(Builder& bld, uint32_t idx, const Region& A0, const Region& B0,
   return ETHA_OK;
   };  // emit
 
-  // Byte moves whose rows are not a whole number of aligned 16-byte units (odd row lengths, short skewed
-  // rows): instead of element-sized units, every row is split into a body of 16-byte units - accessed
-  // unaligned on the sides whose row starts are not 16-byte aligned - and a remainder of < 16 bytes in
-  // narrow units.  Both parts are ordinary tile sets over the same rows.
-  if (!cvt && !red.n_peers && ua_log2 < 4 && run_elems * (uint64_t)esa >= 32) {
+  // Runs that are not a whole number of wide units: every row is split into a body of wide units (16 bytes
+  // for byte moves, a full vector for converting and reducing moves) and a narrow remainder.  Both parts
+  // are ordinary, densely packed tile sets over the same rows.
+  if (plain && ua_log2 < 4 && run_elems * (uint64_t)esa >= 32) {
     const uint64_t run_bytes = run_elems * (uint64_t)esa;
     const uint64_t body_units = run_bytes / 16, rem_bytes = run_bytes % 16;
-    const uint32_t dt_bits = (dta << kMetaDtaShift) | (dtb << kMetaDtbShift);
-    // a row's start is aligned only if base, outer strides AND (for the 2nd, 3rd.. rows of a collapsed run) hold
-    const uint32_t body_meta = dt_bits | (4u << kMetaUaShift) | (4u << kMetaUbShift) | ((mask_a & 15) ? kMetaSkew : 0u) |
-                               ((mask_b & 15) ? kMetaSkewB : 0u);
-    if (!(body_meta & (kMetaSkew | kMetaSkewB)) && rem_bytes == 0)
-      return fail(ETHA_ERR_INVALID, "chunk %u: internal alignment classification error", idx);
+    const uint32_t body_meta = dt_bits | (4u << kMetaUaShift) | (4u << kMetaUbShift) | skew_bits(4, 4);
     int rc = emit(A0.base, B0.base, body_units, 16, 16, body_meta);
-    if (rc != ETHA_OK || rem_bytes == 0) return rc;
-    uint64_t m = mask_a | mask_b | rem_bytes | 16;
+    if (rc != ETHA_OK) return rc;
     int v = 3;
-    while (v > 0 && (m & ((1ull << v) - 1))) v--;
-    const uint32_t rem_meta = dt_bits | ((uint32_t)v << kMetaUaShift) | ((uint32_t)v << kMetaUbShift);
+    while (v > 0 && (rem_bytes & ((1ull << v) - 1))) v--;
+    // the remainder starts body_units * 16 bytes into each row: same position modulo 16 as the row start
+    const uint32_t rem_meta = dt_bits | ((uint32_t)v << kMetaUaShift) | ((uint32_t)v << kMetaUbShift) | skew_bits(v, v);
     return emit(A0.base + body_units * 16, B0.base + body_units * 16, rem_bytes >> v, 1ull << v, 1ull << v, rem_meta);
+  }
+  if (!plain && !(meta & kMetaVec) && epv_full > 1 && run_elems >= 2 * (uint64_t)epv_full) {
+    const uint64_t body_units = run_elems / (uint64_t)epv_full, rem_elems = run_elems % (uint64_t)epv_full;
+    const int va = log2u((uint64_t)(epv_full * esa)), vb = log2u((uint64_t)(epv_full * esb));
+    const uint32_t body_meta = dt_bits | kMetaCvt | kMetaVec | ((uint32_t)va << kMetaUaShift) | ((uint32_t)vb << kMetaUbShift) |
+                               skew_bits(va, vb);
+    int rc = emit(A0.base, B0.base, body_units, 1ull << va, 1ull << vb, body_meta);
+    if (rc != ETHA_OK) return rc;
+    // element units are always aligned (checked above), so the remainder carries no skew flags
+    const uint32_t rem_meta = dt_bits | kMetaCvt | ((uint32_t)log2u((uint64_t)esa) << kMetaUaShift) |
+                              ((uint32_t)log2u((uint64_t)esb) << kMetaUbShift);
+    return emit(A0.base + body_units * (uint64_t)(epv_full * esa), B0.base + body_units * (uint64_t)(epv_full * esb),
+                rem_elems, (uint64_t)esa, (uint64_t)esb, rem_meta);
   }
   return emit(A0.base, B0.base, run_units, ua, ub, meta);
 }

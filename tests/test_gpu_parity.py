@@ -14,7 +14,7 @@ from etha_amd import workloads
 from etha_amd.comm import Chunk, LoopbackWire, Transport, bucket_comm, chunk_to_bucket_ops
 from etha_amd.world import ReshardJob, TensorSpec
 
-from helpers import (DTYPES, assert_bit_equal, cpu_fill, expected_target, gpu_vs_oracle, load_cases, mesh_of,
+from helpers import (DTYPES, assert_bit_equal, clone_specs, cpu_fill, expected_target, gpu_vs_oracle, load_cases, mesh_of,
                      mirror_partials, parse_placements, run_oracle)
 
 pytestmark = pytest.mark.gpu
@@ -456,6 +456,43 @@ def test_skewed_buckets_large(gpu_device):
     plan = job.wire.plan(job.send_buckets[0])
     run, _ = plan.send_table.tiles()
     assert ((run["meta"] & (1 << 18)) != 0).sum() > 0  # the skew path was really taken
+
+
+@pytest.mark.parametrize("src_dt,tgt_dt,cols", [
+    (torch.float32, torch.bfloat16, 1000),   # full vectors at a 4-byte-aligned fp32 pitch
+    (torch.float32, torch.bfloat16, 1003),   # vector body + 3-element remainder
+    (torch.bfloat16, torch.float16, 91),     # 8-element vectors + remainder, odd pitch
+    (torch.float64, torch.float32, 77),
+    (torch.bfloat16, torch.bfloat16, 12),    # 24-byte rows: 8-byte units at 2-byte-aligned addresses
+    (torch.int8, torch.int8, 6),             # 6-byte rows at odd addresses
+    (torch.bfloat16, torch.bfloat16, 257),   # 514-byte rows: unaligned body + 2-byte remainder
+])
+def test_rows_at_element_aligned_pitch(gpu_device, src_dt, tgt_dt, cols):
+    """Source and target shards live inside parents whose row pitch is one element longer than the row,
+    so row starts are only element-aligned: vector units must still be used and still be exact."""
+    def padded(kind, t):
+        if t.dim() != 2:
+            return t
+        parent = torch.zeros(t.shape[0], t.shape[1] + 1, dtype=t.dtype, device=t.device)
+        return parent[:, : t.shape[1]]
+
+    one = (mesh_of(0, [1]), (Replicate(),), mesh_of(1, [1]), (Replicate(),))
+    specs = [TensorSpec("lead", (5,), *one, src_dt, tgt_dt, seed=1, std=1.0),
+             TensorSpec("rows", (300, cols), *one, src_dt, tgt_dt, seed=2, std=1.0)]
+    gpu_job = ReshardJob(clone_specs(specs), device=gpu_device, bucket_size=1 << 30, keep_globals=True, fill=cpu_fill,
+                         local_view=padded)
+    cpu_job = ReshardJob(clone_specs(specs), device="cpu", bucket_size=1 << 30, keep_globals=True, fill=cpu_fill,
+                         local_view=padded)
+    gpu_job.run()
+    run_oracle(cpu_job)
+    for i, spec in enumerate(specs):
+        assert_bit_equal(gpu_job.target_locals[i][1], cpu_job.target_locals[i][1], spec.name)
+        assert_bit_equal(gpu_job.target_locals[i][1], expected_target(spec, cpu_job.globals_[i], 1), spec.name + " closed form")
+    # element-sized units only where the arithmetic forces them (remainders), never for whole rows
+    plan = gpu_job.wire.plan(gpu_job.send_buckets[0])
+    run, row = plan.send_table.tiles()
+    units = sum(int(t["n"].sum()) for t in (run, row))
+    assert units <= 5 + 300 * (cols // 2 + 8)
 
 
 def test_bucket_protocol_methods(gpu_device):

@@ -50,6 +50,11 @@ GEOMETRIES = [
     ((64, 1024), None, (0, 5), (64, 777), nat.BF16, nat.BF16, 2),        # skewed rows of 1554 bytes
     ((9000,), None, (1,), (8990,), nat.B8, nat.B8, 1),                   # byte elements, odd everything
     ((30, 600), None, (0, 1), (30, 599), nat.F32, nat.F32, 4),           # dword-aligned skew
+    ((64, 1030), None, (0, 3), (64, 1000), nat.F32, nat.BF16, 4),        # vector conversion, fp32 rows only 4-byte aligned
+    ((40, 100), None, (0, 1), (40, 91), nat.BF16, nat.F16, 2),           # 8-element vectors + remainder of 3, skewed
+    ((50, 77), None, (0, 0), (50, 77), nat.F64, nat.F32, 8),             # 2-element vectors + remainder of 1
+    ((64, 13), None, (0, 1), (64, 12), nat.BF16, nat.BF16, 2),           # 24-byte rows at a 2-byte skew: 8-byte units
+    ((64, 7), None, (0, 0), (64, 6), nat.B8, nat.B8, 1),                 # 6-byte rows at odd addresses: 2-byte units
     ((5, 0, 7), None, (0, 0, 0), (5, 0, 7), nat.F32, nat.F32, 0),        # empty chunk
 ]
 

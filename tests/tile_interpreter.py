@@ -127,7 +127,9 @@ def execute(table, arena, direction: str, first: int = 0, count: int | None = No
             skew_a, skew_b = bool(int(m) & (1 << 18)), bool(int(m) & (1 << 19))
             assert skew_a or np.all(a[sel] % ua == 0), "misaligned vector access on the a side"
             assert skew_b or np.all(b[sel] % ub == 0), "misaligned vector access on the b side"
-            assert not (skew_a or skew_b) or (ua == 16 and ub == 16 and not cvt)
+            if cvt:  # typed accesses: every element must sit at a multiple of its size, skewed or not
+                esz = {0: 2, 1: 2, 2: 4, 3: 8}
+                assert np.all(a[sel] % esz[dta] == 0) and np.all(b[sel] % esz[dtb] == 0), "misaligned element"
             reduce = row_idx[sel][0] >= 0 and int(row_tiles["n_peers"][row_idx[sel][0]]) > 0
             if reduce:
                 _reduce_units(arena, mem, row_tiles, row_idx[sel], a[sel], b[sel], ua, ub, dta, dtb, peers)
