@@ -876,7 +876,6 @@ struct EthaTable {
 namespace {
 
 int upload_table(EthaTable* t) {
-
   if (!t->h_run.empty()) {
     const size_t bytes = t->h_run.size() * sizeof(RunTile);
     HIP_TRY(hipMalloc(&t->d_run, bytes));
@@ -1164,18 +1163,18 @@ int etha_table_optimize_range(EthaTable* t, uint32_t first, uint32_t count) {
     return px < py;
   });
   if (t->uploaded) {
-    if (!o.h_run.empty()) {
-      const size_t bytes = o.h_run.size() * sizeof(RunTile);
-      HIP_TRY(hipMalloc(&o.d_run, bytes));
-      HIP_TRY(hipMemcpy(o.d_run, o.h_run.data(), bytes, hipMemcpyHostToDevice));
-      t->device_bytes += bytes;
+    const size_t run_bytes = o.h_run.size() * sizeof(RunTile), row_bytes = o.h_row.size() * sizeof(RowTile);
+    hipError_t e = hipSuccess;
+    if (run_bytes) e = hipMalloc(&o.d_run, run_bytes);
+    if (e == hipSuccess && run_bytes) e = hipMemcpy(o.d_run, o.h_run.data(), run_bytes, hipMemcpyHostToDevice);
+    if (e == hipSuccess && row_bytes) e = hipMalloc(&o.d_row, row_bytes);
+    if (e == hipSuccess && row_bytes) e = hipMemcpy(o.d_row, o.h_row.data(), row_bytes, hipMemcpyHostToDevice);
+    if (e != hipSuccess) {
+      if (o.d_run) (void)hipFree(o.d_run);
+      if (o.d_row) (void)hipFree(o.d_row);
+      return fail(ETHA_ERR_HIP, "uploading the ordered range: %s", hipGetErrorString(e));
     }
-    if (!o.h_row.empty()) {
-      const size_t bytes = o.h_row.size() * sizeof(RowTile);
-      HIP_TRY(hipMalloc(&o.d_row, bytes));
-      HIP_TRY(hipMemcpy(o.d_row, o.h_row.data(), bytes, hipMemcpyHostToDevice));
-      t->device_bytes += bytes;
-    }
+    t->device_bytes += run_bytes + row_bytes;
   }
   t->ordered.emplace(key, std::move(o));
   return ETHA_OK;
@@ -1186,9 +1185,9 @@ int etha_table_read_ordered(const EthaTable* t, uint32_t first, uint32_t count, 
   if (!t || !need_bytes) return fail(ETHA_ERR_INVALID, "null argument");
   auto it = t->ordered.find(std::make_pair(first, count));
   if (it == t->ordered.end()) return fail(ETHA_ERR_INVALID, "range [%u,+%u) has not been optimized", first, count);
+  if (which != 0 && which != 1) return fail(ETHA_ERR_INVALID, "which must be 0 or 1");
   const void* src = which == 0 ? (const void*)it->second.h_run.data() : (const void*)it->second.h_row.data();
   const uint64_t bytes = which == 0 ? it->second.h_run.size() * sizeof(RunTile) : it->second.h_row.size() * sizeof(RowTile);
-  if (which != 0 && which != 1) return fail(ETHA_ERR_INVALID, "which must be 0 or 1");
   *need_bytes = bytes;
   if (out && bytes) memcpy(out, src, bytes < cap_bytes ? bytes : cap_bytes);
   return ETHA_OK;
