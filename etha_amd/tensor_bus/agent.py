@@ -106,6 +106,8 @@ class TensorBusAgent:
         self._state_paths: dict[int, str] = {}
         self._threads: list[threading.Thread] = []
         self._last_heartbeat = 0.0
+        self._last_core: dict | None = None
+        self._unsynced: list[tuple[dict, float]] = []  # (result dict, start time) of transfers enqueued but not synchronised
         self.stats = {"ipc_tensors": 0, "in_process_tensors": 0, "transfers": 0}
         for rank in range(world_size):
             cmd_path, state_path = self.path_naming_fn(rank)
@@ -132,16 +134,19 @@ class TensorBusAgent:
             self._inbox.put(_Entry(rank=rank, conn=conn, command=command))
 
     def _write_state(self, force: bool = False) -> None:
+        """Publish heartbeat and pair/batch state.  ``force`` asks for the current state to be visible on
+        return; files are rewritten only if the state differs from what they hold or the heartbeat is due."""
         now = time.time()
-        if not force and now - self._last_heartbeat < self.heartbeat_interval:
-            return
-        self._last_heartbeat = now
-        state = {
-            "agent:heartbeat": now,
+        core = {
             "pairs": {name: ("matched" if p.matched else "pending") for name, p in self.pairs.items()},
             "batches": {bid: {"transfer_signal": b.transfer_signal} for bid, b in self.batches.items()},
         }
-        blob = json.dumps(state)
+        due = now - self._last_heartbeat >= self.heartbeat_interval
+        if not due and (not force or core == self._last_core):
+            return
+        self._last_heartbeat = now
+        self._last_core = core
+        blob = json.dumps({"agent:heartbeat": now, **core})
         for path in self._state_paths.values():
             tmp = f"{path}.tmp{os.getpid()}"
             with open(tmp, "w") as f:
@@ -170,7 +175,11 @@ class TensorBusAgent:
                 self._pending.append(self._inbox.get_nowait())
             except queue.Empty:
                 break
-        progressed, changed = True, False
+        # Sweep until nothing moves.  Commands that complete are answered only after the sweep: the device
+        # work of every transfer that became ready is enqueued first, then the stream is synchronised once
+        # and the state files are written once, instead of once per rank.
+        finished: list[tuple[_Entry, tuple]] = []
+        progressed = True
         while progressed:
             progressed = False
             for entry in list(self._pending):
@@ -178,17 +187,28 @@ class TensorBusAgent:
                     done, value = self._advance(entry)
                 except Exception as e:  # report to the worker, keep serving
                     logger.exception("agent rank %s: %s failed", entry.rank, type(entry.command).__name__)
-                    self._reply(entry, ("error", (type(e).__name__, str(e))))
+                    finished.append((entry, ("error", (type(e).__name__, str(e)))))
                     self._pending.remove(entry)
                     progressed = True
                     continue
                 if done:
-                    # the state file must show the new state before the worker is released
-                    self._write_state(force=True)
-                    self._reply(entry, ("ok", value))
+                    finished.append((entry, ("ok", value)))
                     self._pending.remove(entry)
-                    progressed = changed = True
-        self._write_state(force=changed)
+                    progressed = True
+        if self._unsynced:
+            # a worker may overwrite its tensors as soon as its send returns, and read them as soon as its
+            # recv returns: both replies wait for the device
+            if self.device.type == "cuda":
+                torch.cuda.current_stream(self.device).synchronize()
+            now = time.perf_counter()
+            for result, t0 in self._unsynced:
+                result["ms"] = (now - t0) * 1e3
+            self._unsynced.clear()
+        if finished:
+            # the state file must show the new state before a worker is released
+            self._write_state(force=True)
+            for entry, message in finished:
+                self._reply(entry, message)
 
     @staticmethod
     def _reply(entry: _Entry, message) -> None:
@@ -389,14 +409,15 @@ class TensorBusAgent:
                 if d in batch.recv_count and batch.recv_count[d] < gen:
                     return False, None  # the previous generation has not been consumed yet
             batch.transfer_signal = True
-            t0 = time.perf_counter()
-            bucket_comm(buckets, wire=self.wire, merge_launches=True)
+            result = {"ms": 0.0}
+            self._unsynced.append((result, time.perf_counter()))
+            bucket_comm(buckets, wire=self.wire, merge_launches=True, synchronize=False)
             batch.send_count[rank] = gen + 1
             for d in self._peers(buckets, "dst"):
                 batch.owed[d] = max(batch.owed.get(d, 0), gen + 1)
             if self.wire.plan(buckets).lends_tensor_memory():
                 entry.started = True
-                entry.result = {"ms": (time.perf_counter() - t0) * 1e3}
+                entry.result = result
                 self.stats["transfers"] += 1
                 return False, None
         else:
@@ -404,13 +425,14 @@ class TensorBusAgent:
             for s in self._peers(buckets, "src"):
                 if batch.send_count.get(s, 0) <= gen:
                     return False, None  # wait for the source's send of this generation
-            t0 = time.perf_counter()
-            bucket_comm(buckets, wire=self.wire, merge_launches=True)
+            result = {"ms": 0.0}
+            self._unsynced.append((result, time.perf_counter()))
+            bucket_comm(buckets, wire=self.wire, merge_launches=True, synchronize=False)
             batch.recv_count[rank] = gen + 1
             if all(batch.recv_count.get(d, 0) >= n for d, n in batch.owed.items()):
                 batch.transfer_signal = False  # every destination of every send so far has received
         self.stats["transfers"] += 1
-        return True, {"ms": (time.perf_counter() - t0) * 1e3}
+        return True, result
 
     def _release_batch(self, batch: BatchState) -> None:
         # receivers first: their plans only reference slots, the senders' plans own them
