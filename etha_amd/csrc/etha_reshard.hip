@@ -35,6 +35,9 @@ namespace {
 #ifndef ETHA_BLOCK_THREADS
 #define ETHA_BLOCK_THREADS 64
 #endif
+#ifndef ETHA_CVT_WIDE_BYTES
+#define ETHA_CVT_WIDE_BYTES 16
+#endif
 #ifndef ETHA_SKEW_PEEL_MIN_BYTES
 #define ETHA_SKEW_PEEL_MIN_BYTES (256 * 1024)
 #endif
@@ -45,6 +48,15 @@ constexpr uint32_t kTileThreads = ETHA_TILE_UNITS;     // units per tile
 constexpr uint32_t kBlockThreads = ETHA_BLOCK_THREADS; // work-items per workgroup
 constexpr uint32_t kBlocksPerTile = kTileThreads / kBlockThreads;
 static_assert(kTileThreads % kBlockThreads == 0 && kBlocksPerTile >= 1, "tile must be a multiple of the workgroup");
+
+// Elements one work-item converts at once: the narrow side moves up to 16 bytes, the wide side up to
+// kCvtWideBytes (one or two 16-byte accesses).
+constexpr int kCvtWideBytes = ETHA_CVT_WIDE_BYTES;
+constexpr int cvt_elems_per_unit(int es_a, int es_b) {
+  const int lo = es_a < es_b ? es_a : es_b, hi = es_a < es_b ? es_b : es_a;
+  const int by_narrow = 16 / lo, by_wide = kCvtWideBytes / hi;
+  return by_narrow < by_wide ? by_narrow : by_wide;
+}
 
 // ---- tile program entries (device-visible, also read back by host-side checkers) -------------
 // A "unit" is what one work-item moves: 2^ua bytes on the a side and 2^ub bytes on the b side
@@ -185,9 +197,7 @@ __device__ __forceinline__ void cvt_n(uint64_t src, uint64_t dst) {
 
 template <typename S, typename D>
 __device__ __forceinline__ void cvt_pair(bool vec, uint64_t src, uint64_t dst) {
-  constexpr int kMaxBytes = sizeof(typename S::bits) > sizeof(typename D::bits) ? sizeof(typename S::bits)
-                                                                                  : sizeof(typename D::bits);
-  constexpr int kN = 16 / kMaxBytes;
+  constexpr int kN = cvt_elems_per_unit(sizeof(typename S::bits), sizeof(typename D::bits));
   if (vec)
     cvt_n<S, D, kN>(src, dst);
   else
@@ -656,7 +666,8 @@ int compile_pair(Builder& bld, uint32_t idx, const Region& A0, const Region& B0,
   uint32_t meta = 0;
   uint64_t mask_a = 0, mask_b = 0;  // OR of every row start (base and outer strides) per side
   const bool plain = !cvt && !red.n_peers;
-  const int epv_full = 16 / (esa > esb ? esa : esb);  // elements per full vector of a converting move
+  // elements per full vector: converting moves may use two accesses on the wide side, reductions one
+  const int epv_full = red.n_peers ? 16 / (esa > esb ? esa : esb) : cvt_elems_per_unit(esa, esb);
   {
     mask_a = red.n_peers ? 0 : A0.base;
     mask_b = B0.base;

@@ -139,7 +139,7 @@ def execute(table, arena, direction: str, first: int = 0, count: int | None = No
             do = arena.offsets(dst, ud)[:, None] + np.arange(ud)
             data = mem[so]
             if cvt:
-                assert vec == (max(us, ud) == 16) or not vec
+                assert not vec or (max(us, ud) in (16, 32) and min(us, ud) <= 16)
                 raw_s, raw_d = _CODE_RAW[ds_], _CODE_RAW[dd]
                 elems = np.ascontiguousarray(data).view(raw_s)
                 data = co.cast(elems, ds_, dd, raw_d).view(np.uint8).reshape(len(so), ud)
