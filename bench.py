@@ -24,8 +24,8 @@ HBM_PEAK_GBS = 8000.0  # MI355X HBM3E, published
 # scaled by what the counter reads for a plain 1 GiB copy; the summary of those runs is
 # profiles/etha_tile_kernel_llama3_8b_fsdp8_to_tp2.txt.  Keyed by (workload, kernel, launch granularity).
 MEASURED_TRAFFIC_BYTES = {
-    ("llama3_8b_fsdp8_to_tp2", "etha_tile_kernel<false>", "run of buckets"): 2043045817,
-    ("llama3_8b_fsdp8_to_tp2", "etha_tile_kernel<true>", "run of buckets"): 16249577507,
+    ("llama3_8b_fsdp8_to_tp2", "etha_tile_kernel<false>", "run of buckets"): 2043040739,
+    ("llama3_8b_fsdp8_to_tp2", "etha_tile_kernel<true>", "run of buckets"): 16249517705,
     # profiles/etha_reduce_kernel_partial4_to_shard2.txt
     ("partial4_to_shard2", "etha_reduce_kernel", "run of buckets"): 5436000000,
 }
