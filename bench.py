@@ -41,6 +41,9 @@ def parse_args():
     ap.add_argument("--fanout", type=int, default=1, help="side streams for per-bucket launches (with --per-bucket)")
     ap.add_argument("--zero-copy", action="store_true",
                     help="lend contiguous single-chunk buckets to the consumer instead of packing them")
+    ap.add_argument("--direct", action="store_true",
+                    help="no bucket buffers: the target side copies straight from the source shards (one pass; "
+                         "not the pack+unpack path the headline is quoted on)")
     ap.add_argument("--graph", action="store_true", help="replay the step from a captured HIP graph (whole step timed)")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--cpu-layers", type=int, default=8, help="layers of the workload the CPU baseline sample covers")
@@ -155,7 +158,8 @@ def main():
     torch.cuda.set_device(dev)
     specs, targets, bucket = workloads.WORKLOADS[args.workload]()
     t0 = time.time()
-    job = ReshardJob(specs, device=dev, bucket_size=bucket, target_ranks=targets, zero_copy=args.zero_copy)
+    job = ReshardJob(specs, device=dev, bucket_size=bucket, target_ranks=targets, zero_copy=args.zero_copy,
+                     direct=args.direct)
     merge = not args.per_bucket
     # plan (compiles the tile programs) + warm-up
     for _ in range(max(args.warmup, 1)):
@@ -168,7 +172,7 @@ def main():
     steps_of = (lambda p: p.merged_steps) if merge else (lambda p: p.steps)
     n_pack = sum(1 for p in send_plans for s in steps_of(p) if s[0] in ("pack", "reduce_pack"))
     n_self = sum(1 for p in send_plans + recv_plans for s in steps_of(p) if s[0] == "selfcopy")
-    n_unpack = sum(1 for p in send_plans + recv_plans for s in steps_of(p) if s[0] == "unpack")
+    n_unpack = sum(1 for p in send_plans + recv_plans for s in steps_of(p) if s[0] in ("unpack", "direct"))
 
     # algorithmic bytes: pack reads the source dtype and writes the wire dtype; unpack reads the wire
     # dtype and writes the target dtype; a reduce-pack reads every member's partial
@@ -196,6 +200,7 @@ def main():
                     n *= d
                 unpack_write += n * c.tensor.element_size()
     unpack_read = sum(table_bytes(p, "recv_table") for p in recv_plans)
+    unpack_read += sum(p.direct_read_bytes for p in recv_plans)  # direct wire: reads the source regions themselves
     # LOCAL chunks run inside the send phase as direct copies: read the source region, write the target
     self_bytes = 0
     for p in send_plans:
@@ -242,7 +247,7 @@ def main():
     dev_ms = pack_avg + unpack_avg
 
     value = S / (step_ms * 1e-3) / 1e9
-    pack_gbs = pack_bytes / (pack_avg * 1e-3) / 1e9
+    pack_gbs = pack_bytes / (pack_avg * 1e-3) / 1e9 if pack_avg > 0 else 0.0
     unpack_gbs = unpack_bytes / (unpack_avg * 1e-3) / 1e9 if unpack_avg > 0 else 0.0
     dominant = "pack" if pack_avg >= unpack_avg else "unpack"
     dom_bytes, dom_ms, dom_launches = (
@@ -251,6 +256,8 @@ def main():
     kernel_name = {"pack": "etha_tile_kernel<false>", "unpack": "etha_tile_kernel<true>"}[dominant]
     if dominant == "pack" and any(s[0] == "reduce_pack" for p in send_plans for s in steps_of(p)):
         kernel_name = "etha_reduce_kernel"
+    if dominant == "unpack" and args.direct:
+        kernel_name = "etha_tile_kernel<false>"  # the direct copy runs source region -> target region
     achieved = dom_bytes / (dom_ms * 1e-3) / 1e9
     out = {
         "metric": "effective reshard GB/s (pack+unpack, 1 GPU) and % of HBM peak",
@@ -273,6 +280,7 @@ def main():
             "fanout_streams": args.fanout,
             "hip_graph": bool(args.graph),
             "zero_copy_single_chunk": bool(args.zero_copy),
+            "direct_same_device": bool(args.direct),
             **job.counts(),
         },
         "device_ms_per_step": round(dev_ms, 4),
@@ -287,8 +295,9 @@ def main():
             "peak": HBM_PEAK_GBS,
             "unit": "GB/s",
             "frac": round(achieved / HBM_PEAK_GBS, 4),
-            "traffic": MEASURED_TRAFFIC_BYTES.get(
-                (args.workload, kernel_name, "run of buckets" if merge else "bucket")),
+            # measured for the default configuration only
+            "traffic": None if (args.zero_copy or args.direct or args.graph or args.fanout > 1) else
+            MEASURED_TRAFFIC_BYTES.get((args.workload, kernel_name, "run of buckets" if merge else "bucket")),
             "bytes_per_launch": dom_bytes // dom_launches,
             "avg_launch_ms": round(dom_ms / dom_launches, 5),
             "launches_per_step": dom_launches,

@@ -11,7 +11,9 @@ Here a bucket list is compiled once into tile programs and a call enqueues, in b
                    source and destination bytes may overlap;
 * NONE buckets:    nothing - the primary's reduce-pack already read this member's partial;
 * with the wire's ``zero_copy_single_chunk`` option, a single-chunk source bucket whose bytes already lie
-  contiguously in the tensor is lent, not packed: the consumer unpacks straight from the tensor.
+  contiguously in the tensor is lent, not packed: the consumer unpacks straight from the tensor;
+* with the wire's ``direct_same_device`` option no plain bucket is packed at all: the target bucket's
+  launch copies from the producer's chunk regions into its own tensors in one pass.
 
 Consecutive buckets of the same kind can be merged into one launch (``merge_launches=True``).
 All work goes to one stream, so per-channel FIFO order and "pack before unpack" hold by stream
@@ -29,7 +31,7 @@ from .transfer import Transport
 
 __all__ = ["bucket_comm", "TransferPlan"]
 
-_PACK, _REDUCE, _UNPACK, _SELF, _LEND = "pack", "reduce_pack", "unpack", "selfcopy", "lend"
+_PACK, _REDUCE, _UNPACK, _SELF, _LEND, _DIRECT = "pack", "reduce_pack", "unpack", "selfcopy", "lend", "direct"
 
 
 class TransferPlan:
@@ -43,6 +45,7 @@ class TransferPlan:
         # steps: (kind, first_chunk, n_chunks, slot or None), in execution order
         self.steps: list[tuple[str, int, int, object]] = []
         self.lent: set[int] = set()  # ids of source buckets that are consumed straight from their tensor
+        self.direct_read_bytes = 0  # bytes the direct steps read from producers' tensors (source dtype)
         send_index: dict[tuple, int] = {}
         recv_index: dict[tuple, int] = {}
         from .loopback import wire_key
@@ -99,6 +102,17 @@ class TransferPlan:
                 idx = recv_index.get(key, 0)
                 recv_index[key] = idx + 1
                 slot = wire.slot_for_recv(bucket, idx)
+                if slot.sources is not None:  # direct wire: copy from the producer's regions, no bucket
+                    first = len(local)
+                    for c, (src_t, src_slice, wire_dtype) in zip(bucket.chunks, slot.sources):
+                        if wire_dtype not in (src_t.dtype, c.tensor.dtype):
+                            raise NotImplementedError(
+                                f"{bucket}: wire dtype {wire_dtype} differs from both tensor dtypes; one direct "
+                                "conversion cannot reproduce the two roundings")
+                        local.add_pair(src_t, src_slice, c.tensor, c.dst_slice, c.chunk_shape)
+                        self.direct_read_bytes += c.nbytes // wire_dtype.itemsize * src_t.element_size()
+                    self.steps.append((_DIRECT, first, len(bucket.chunks), slot))
+                    continue
                 first = len(recv)
                 for off, c in zip(bucket.offsets, bucket.chunks):
                     recv.add_chunk(c, c.tensor, c.dst_slice, slot, off, reduce=False)
@@ -126,7 +140,7 @@ class TransferPlan:
         for kind, first, count, slots in self.merged_steps:
             if len(slots) > 1 and kind == _UNPACK:
                 self.recv_table.optimize_range(first, count)
-            elif len(slots) > 1 and kind == _SELF:
+            elif len(slots) > 1 and kind in (_SELF, _DIRECT):
                 self.local_table.optimize_range(first, count)
 
     @staticmethod
@@ -218,6 +232,13 @@ class TransferPlan:
                         )
                 self.recv_table.unpack(first, count, stream)
             elif kind == _SELF:
+                self.local_table.selfcopy(first, count, stream)
+            elif kind == _DIRECT:
+                for s in slots:
+                    if s is not None and s.filled == 0:
+                        raise RuntimeError(
+                            "recv bucket runs before its send bucket was ever sent (a real wire would block here)"
+                        )
                 self.local_table.selfcopy(first, count, stream)
             if kind in (_PACK, _REDUCE, _LEND):
                 for s in slots:

@@ -93,8 +93,11 @@ class Slot:
     hi: int
     filled: int = 0  # number of times a pack has been enqueued into this slot
     drained: int = 0  # number of unpacks enqueued from it (per consumer bookkeeping is the wire's job)
-    borrowed: bool = False  # the slot IS the source tensor's memory (zero-copy single-chunk bucket), not pool memory
-    keepalive: object = None  # the tensor a borrowed slot aliases
+    borrowed: bool = False  # the slot is source-tensor memory (zero-copy single-chunk bucket, direct wire), not pool memory
+    keepalive: object = None  # the tensor(s) a borrowed slot aliases
+    # direct wire: per chunk of the send bucket ``(source tensor, src_slice, wire dtype)``; the consumer copies
+    # from these regions straight into its own tensors and no bucket buffer exists (ptr is 0)
+    sources: list | None = None
 
 
 class DescBuilder:
@@ -152,16 +155,20 @@ class SelfCopyBuilder:
 
     def add_chunk(self, chunk: Chunk) -> None:
         src_t = chunk.src_tensor if chunk.src_tensor is not None else chunk.tensor
+        self.add_pair(src_t, chunk.src_slice, chunk.tensor, chunk.dst_slice, chunk.chunk_shape)
+
+    def add_pair(self, src_t, src_slice: tuple, dst_t, dst_slice: tuple, chunk_shape: tuple) -> None:
+        """Copy ``src_t[src_slice]`` to ``dst_t[dst_slice]`` (same shape), converting between their dtypes."""
         a = np.zeros((), dtype=nat.CHUNK_DESC)
         b = np.zeros((), dtype=nat.CHUNK_DESC)
-        fill_region(a, src_t, chunk.src_slice, chunk.chunk_shape)
-        fill_region(b, chunk.tensor, chunk.dst_slice, chunk.chunk_shape)
-        check_cast(src_t.dtype, chunk.tensor.dtype)
+        fill_region(a, src_t, src_slice, chunk_shape)
+        fill_region(b, dst_t, dst_slice, chunk_shape)
+        check_cast(src_t.dtype, dst_t.dtype)
         a["wire_dtype"] = a["tensor_dtype"]
         b["wire_dtype"] = b["tensor_dtype"]
         self.src.append(a)
         self.dst.append(b)
-        self.keepalive += [src_t, chunk.tensor]
+        self.keepalive += [src_t, dst_t]
 
     def build(self, upload: bool = True) -> nat.Table | None:
         if not self.src:

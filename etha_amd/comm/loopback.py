@@ -88,6 +88,12 @@ class LoopbackWire:
         # path sends straight from it (ir.py:238-244).  The producer must then leave that tensor alone
         # until the consumer has unpacked: "sent" no longer means "copied".
         self.zero_copy_single_chunk = False
+        # True: no bucket buffers at all for plain (non-Partial) buckets.  Producer and consumer tensors are
+        # on one device, so the consumer's launch reads the producer's chunk regions and writes its own:
+        # one pass (read source dtype, write target dtype) instead of pack + unpack, and no pool memory.
+        # This is what a pull over a peer mapping does between GPUs, minus the link.  Like a lent bucket,
+        # a "sent" tensor must be left alone until the consumer has run.  Only within one process.
+        self.direct_same_device = False
         self.pool: BucketPool | None = None
         self._sent: dict[tuple, list[tuple[Slot, tuple[int, ...]]]] = defaultdict(list)
         self._plans: dict[tuple, object] = {}
@@ -114,7 +120,12 @@ class LoopbackWire:
         if index != len(sent):
             raise RuntimeError(f"{bucket}: send buckets must be planned in order")
         slot = None
-        if self.zero_copy_single_chunk:
+        if self.direct_same_device and not any(c.source_partial_groups for c in bucket.chunks):
+            self._pool_for(device)
+            slot = Slot(ptr=0, nbytes=bucket.total_bytes, lo=0, hi=0, borrowed=True)
+            slot.sources = [(c.tensor, c.src_slice, c.transfer_dtype or c.tensor.dtype) for c in bucket.chunks]
+            slot.keepalive = [c.tensor for c in bucket.chunks]
+        if slot is None and self.zero_copy_single_chunk:
             from .device_plan import zero_copy_region
 
             region = zero_copy_region(bucket)
@@ -159,6 +170,8 @@ class LoopbackWire:
         for key, entries in self._sent.items():
             out = []
             for slot, sizes in entries:
+                if slot.sources is not None:
+                    raise NotImplementedError("a direct wire has no bucket buffers to export; it works inside one process")
                 if slot.borrowed:  # lives in a source tensor: export that allocation, range = the slot itself
                     with torch.cuda.device(self.pool.device):
                         segments.append({"ipc": nat.ipc_export(slot.ptr), "nbytes": slot.nbytes})

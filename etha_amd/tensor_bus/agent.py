@@ -88,7 +88,8 @@ class TensorBusAgent:
     """Hub agent: serves ``world_size`` agent ranks on one device."""
 
     def __init__(self, world_size: int, path_naming_fn=None, device: str | torch.device = "cuda:0",
-                 heartbeat_interval: float = 0.2, zero_copy_single_chunk: bool = False):
+                 heartbeat_interval: float = 0.2, zero_copy_single_chunk: bool = False,
+                 direct_same_device: bool = False):
         self.world_size = world_size
         self.device = torch.device(device)
         self.path_naming_fn = path_naming_fn or default_path_naming
@@ -97,6 +98,8 @@ class TensorBusAgent:
         # lent buckets are read from the worker's tensor at receive time, so a send that lends memory only
         # completes once its receivers have unpacked (the reference's transfers end with a barrier as well)
         self.wire.zero_copy_single_chunk = zero_copy_single_chunk
+        # no bucket buffers for plain buckets: a recv copies straight from the sending worker's tensors
+        self.wire.direct_same_device = direct_same_device
         self.pairs: dict[str, PairState] = {}
         self.batches: dict[str, BatchState] = {}
         self._inbox: queue.Queue = queue.Queue()
@@ -107,6 +110,7 @@ class TensorBusAgent:
         self._threads: list[threading.Thread] = []
         self._last_heartbeat = 0.0
         self._last_core: dict | None = None
+        self._moved = False  # set by a command that changed shared state without completing
         self._unsynced: list[tuple[dict, float]] = []  # (result dict, start time) of transfers enqueued but not synchronised
         self.stats = {"ipc_tensors": 0, "in_process_tensors": 0, "transfers": 0}
         for rank in range(world_size):
@@ -181,7 +185,7 @@ class TensorBusAgent:
         finished: list[tuple[_Entry, tuple]] = []
         progressed = True
         while progressed:
-            progressed = False
+            progressed, self._moved = False, False
             for entry in list(self._pending):
                 try:
                     done, value = self._advance(entry)
@@ -195,6 +199,9 @@ class TensorBusAgent:
                     finished.append((entry, ("ok", value)))
                     self._pending.remove(entry)
                     progressed = True
+            # a command that changed shared state without completing (a send that lends its tensors and now
+            # waits for its receivers) may have unblocked commands examined earlier in this pass
+            progressed = progressed or self._moved
         if self._unsynced:
             # a worker may overwrite its tensors as soon as its send returns, and read them as soon as its
             # recv returns: both replies wait for the device
@@ -419,6 +426,7 @@ class TensorBusAgent:
                 entry.started = True
                 entry.result = result
                 self.stats["transfers"] += 1
+                self._moved = True
                 return False, None
         else:
             gen = batch.recv_count[rank]

@@ -1,6 +1,6 @@
 """End-to-end timing of ``handler.transfer`` through the tensor bus on one GPU.
 
-    python -m etha_amd.tensor_bus.bench_transfer [--workload NAME] [--steps K] [--warmup W] [--zero-copy]
+    python -m etha_amd.tensor_bus.bench_transfer [--workload NAME] [--steps K] [--warmup W] [--zero-copy | --direct]
 
 Three processes share the GPU, as in a deployment on one device: this process runs the hub agent,
 a "trainer" worker process holds every source rank's shards and a "inference" worker process
@@ -125,6 +125,7 @@ def main() -> None:
     ap.add_argument("--steps", type=int, default=10)
     ap.add_argument("--warmup", type=int, default=2)
     ap.add_argument("--zero-copy", action="store_true", help="lend contiguous single-chunk buckets (agent option)")
+    ap.add_argument("--direct", action="store_true", help="no bucket buffers: receivers copy from the senders' tensors")
     ap.add_argument("--device", default="cuda:0")
     args = ap.parse_args()
 
@@ -146,7 +147,8 @@ def main() -> None:
         sys.exit(2)
     world = 1 + max(int(r) for s in specs for m in (s.source_mesh, s.target_mesh) for r in np.asarray(m).reshape(-1))
     tmpdir = tempfile.mkdtemp(prefix="etha_bus_")
-    agent = TensorBusAgent(world, _naming(tmpdir), device=args.device, zero_copy_single_chunk=args.zero_copy)
+    agent = TensorBusAgent(world, _naming(tmpdir), device=args.device, zero_copy_single_chunk=args.zero_copy,
+                           direct_same_device=args.direct)
     agent.start_in_thread()
     ctx = mp.get_context("spawn")
     out_q = ctx.Queue()
@@ -188,7 +190,8 @@ def main() -> None:
         "value": payload / med / 1e9, "unit": "GB/s", "ms_per_transfer": med * 1e3, "min_ms": lat[0] * 1e3,
         "steps": args.steps, "warmup": args.warmup, "payload_bytes": payload,
         "config": {"workload": args.workload, "source_ranks": len(results["trainer"]["ranks"]),
-                   "target_ranks": len(results["inference"]["ranks"]), "zero_copy_single_chunk": args.zero_copy},
+                   "target_ranks": len(results["inference"]["ranks"]), "zero_copy_single_chunk": args.zero_copy,
+                   "direct_same_device": args.direct},
         "agent": agent_stats,
     }))
 

@@ -106,6 +106,7 @@ class ReshardJob:
     wire: LoopbackWire | None = None
     local_view: object = None  # optional ``(kind, tensor) -> view``: re-home a local shard inside another parent
     zero_copy: bool = False  # lend contiguous single-chunk buckets instead of packing them (see LoopbackWire)
+    direct: bool = False  # no bucket buffers for plain buckets: targets copy straight from the sources (see LoopbackWire)
     source_locals: list[dict[int, torch.Tensor]] = field(default_factory=list, init=False)
     target_locals: list[dict[int, torch.Tensor]] = field(default_factory=list, init=False)
     globals_: list[torch.Tensor | None] = field(default_factory=list, init=False)
@@ -118,6 +119,8 @@ class ReshardJob:
             self.wire = LoopbackWire(self.device)
         if self.zero_copy:
             self.wire.zero_copy_single_chunk = True
+        if self.direct:
+            self.wire.direct_same_device = True
         send_chunks: dict[int, list] = {}
         recv_chunks: dict[int, list] = {}
         m2m_cache: dict[tuple, object] = {}

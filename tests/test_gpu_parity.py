@@ -651,3 +651,50 @@ def test_zero_copy_single_chunk_buckets(gpu_device):
     for p in plans:
         gpu_job.wire.release(p.buckets)  # lent slots are not pool memory and must not enter its free list
     assert all(not s.borrowed for free in gpu_job.wire.pool._free.values() for s in free)
+
+
+def test_direct_same_device_wire(gpu_device):
+    """With the direct wire no plain bucket is packed: the target bucket's launch copies from the producer's
+    regions in one pass.  Same results as the bucket path for P2P, BROADCAST, LOCAL, converting and strided
+    layouts; Partial sources still go through reduce-pack + unpack; no pool memory for the plain buckets."""
+    src = mesh_of(0, (2, 2))
+    specs = [
+        TensorSpec("a", (64, 48), src, (Shard(0), Shard(1)), mesh_of(4, (2,)), (Replicate(),), torch.float32, seed=1),
+        TensorSpec("b", (32, 40), src, (Shard(1), Shard(0)), mesh_of(1, (4,)), (Shard(0),), torch.float32, seed=2),
+        TensorSpec("c", (24, 16), src, (Replicate(), Shard(0)), mesh_of(4, (2,)), (Replicate(),), torch.float32,
+                   torch.bfloat16, seed=3),
+        TensorSpec("d", (8, 128), src, (Shard(0), Shard(1)), mesh_of(4, (2, 2)), (Shard(1), Replicate()),
+                   torch.bfloat16, torch.float32, seed=4),
+        TensorSpec("p", (64, 32), mesh_of(0, (4,)), (Partial(),), mesh_of(4, (2,)), (Shard(0),), torch.bfloat16, seed=5),
+    ]
+    for bucket_size in (1, 4096, 1 << 20):
+        for merge in (False, True):
+            gpu_job = ReshardJob(clone_specs(specs), device=gpu_device, bucket_size=bucket_size, keep_globals=True,
+                                 fill=cpu_fill, direct=True)
+            cpu_job = ReshardJob(clone_specs(specs), device="cpu", bucket_size=bucket_size, keep_globals=True, fill=cpu_fill)
+            mirror_partials(gpu_job, cpu_job)
+            before = [{r: t.clone() for r, t in d.items()} for d in gpu_job.source_locals]
+            gpu_job.run(merge_launches=merge)
+            gpu_job.run(merge_launches=merge)  # plan once, transfer twice
+            run_oracle(cpu_job)
+            for i, spec in enumerate(specs):
+                for r, t in gpu_job.target_locals[i].items():
+                    assert_bit_equal(t, cpu_job.target_locals[i][r], f"{spec.name} rank {r} bucket {bucket_size} merge {merge}")
+                for r, t in gpu_job.source_locals[i].items():
+                    if not any(t is x for x in gpu_job.target_locals[i].values()):
+                        assert_bit_equal(t, before[i][r], f"{spec.name} source {r} mutated")
+            kinds = {s[0] for bs in list(gpu_job.send_buckets.values()) + list(gpu_job.recv_buckets.values())
+                     for s in gpu_job.wire.plan(bs).steps}
+            assert "direct" in kinds and "lend" in kinds and "reduce_pack" in kinds
+            plain_packs = [s for bs in gpu_job.send_buckets.values() for s in gpu_job.wire.plan(bs).steps if s[0] == "pack"]
+            assert not plain_packs  # (staged self-copies would pack; this layout has none)
+    with pytest.raises(NotImplementedError):
+        gpu_job.wire.export_manifest()
+
+
+def test_direct_wire_full_size_llama(gpu_device):
+    specs, targets, bucket = workloads.llama3_8b_fsdp8_to_tp2()
+    job = ReshardJob(specs, device=gpu_device, bucket_size=bucket, target_ranks=targets, keep_globals=True, direct=True)
+    job.run(merge_launches=True)
+    _check_targets_against_global(job, specs)
+    assert job.wire.pool is None or job.wire.pool.reserved_bytes == 0
