@@ -8,7 +8,8 @@ holds every target rank's shards (one thread per rank in both).  Workers registe
 hipIPC once (``register_tensors``) and then repeat ``transfer("send")`` / ``transfer("recv")``.
 One step is timed on the host wall clock from the moment the first source rank issues its send to
 the moment the last target rank's blocking recv returns, so it includes the command round trips,
-the agent's launches and the device work.  Prints ONE JSON line.
+the agent's launches and the device work.  After the last step every same-dtype tensor is verified by a
+checksum of checksums (raw bits summed over all target ranks against all source ranks).  Prints ONE JSON line.
 
 All target ranks of the workload take part (a pair needs its whole mesh), so the payload is every
 target rank's share, not the single share ``bench.py`` measures.
@@ -114,7 +115,14 @@ def _worker(role: str, workload: str, tmpdir: str, device: str, steps: int, warm
             out_q.put((role, "error", errors[0]))
             return
         nbytes = sum(t.numel() * t.element_size() for r in my_ranks for t, _ in shards[r])
-        out_q.put((role, "ok", {"stamps": stamps, "bytes": nbytes, "ranks": my_ranks}))
+        # checksum per logical tensor over every rank of this side: the raw bits summed as integers
+        raw = {1: torch.uint8, 2: torch.int16, 4: torch.int32, 8: torch.int64}
+        sums = [0] * len(specs)
+        for r in my_ranks:
+            for i, (t, _) in enumerate(shards[r]):
+                if t.numel():
+                    sums[i] += int(t.contiguous().view(raw[t.element_size()]).sum(dtype=torch.int64).item())
+        out_q.put((role, "ok", {"stamps": stamps, "bytes": nbytes, "ranks": my_ranks, "checksums": sums}))
     except BaseException:
         out_q.put((role, "error", traceback.format_exc()))
 
@@ -176,6 +184,23 @@ def main() -> None:
                 p.kill()
         agent_stats = dict(agent.stats)
         agent.close()
+    # checksum of checksums: a same-dtype tensor's bits, summed over all target ranks, equal the sum over all
+    # source ranks times the number of copies the target layout holds of each element (per copy the source holds)
+    from torch.distributed.tensor.placement_types import Partial, Replicate
+
+    def copies(mesh, placements):
+        shape = np.asarray(mesh).shape
+        return int(np.prod([n for n, p in zip(shape, placements) if isinstance(p, Replicate)] or [1]))
+
+    verified = 0
+    for i, s in enumerate(specs):
+        if (s.target_dtype or s.source_dtype) != s.source_dtype or any(isinstance(p, Partial) for p in s.source_placements):
+            continue
+        want = results["trainer"]["checksums"][i] * copies(s.target_mesh, s.target_placements)
+        got = results["inference"]["checksums"][i] * copies(s.source_mesh, s.source_placements)
+        if want != got:
+            raise RuntimeError(f"{s.name}: checksum over the target ranks differs from the source ranks' ({got} vs {want})")
+        verified += 1
     send, recv = results["trainer"]["stamps"], results["inference"]["stamps"]
     lat = []
     for k in range(args.warmup, args.warmup + args.steps):
@@ -192,7 +217,7 @@ def main() -> None:
         "config": {"workload": args.workload, "source_ranks": len(results["trainer"]["ranks"]),
                    "target_ranks": len(results["inference"]["ranks"]), "zero_copy_single_chunk": args.zero_copy,
                    "direct_same_device": args.direct},
-        "agent": agent_stats,
+        "agent": agent_stats, "tensors_verified_by_checksum": verified,
     }))
 
 
