@@ -125,14 +125,15 @@ def execute(table, arena, direction: str, first: int = 0, count: int | None = No
             dta, dtb = (int(m) >> 8) & 15, (int(m) >> 12) & 15
             cvt, vec = bool(int(m) & (1 << 16)), bool(int(m) & (1 << 17))
             skew_a, skew_b = bool(int(m) & (1 << 18)), bool(int(m) & (1 << 19))
-            assert skew_a or np.all(a[sel] % ua == 0), "misaligned vector access on the a side"
+            reduce = row_idx[sel][0] >= 0 and int(row_tiles["n_peers"][row_idx[sel][0]]) > 0
+            # (for reduce tiles the a side is an offset from each peer's base: checked against the real addresses below)
+            assert reduce or skew_a or np.all(a[sel] % ua == 0), "misaligned vector access on the a side"
             assert skew_b or np.all(b[sel] % ub == 0), "misaligned vector access on the b side"
-            if cvt:  # typed accesses: every element must sit at a multiple of its size, skewed or not
+            if cvt and not reduce:  # typed accesses: every element must sit at a multiple of its size, skewed or not
                 esz = {0: 2, 1: 2, 2: 4, 3: 8}
                 assert np.all(a[sel] % esz[dta] == 0) and np.all(b[sel] % esz[dtb] == 0), "misaligned element"
-            reduce = row_idx[sel][0] >= 0 and int(row_tiles["n_peers"][row_idx[sel][0]]) > 0
             if reduce:
-                _reduce_units(arena, mem, row_tiles, row_idx[sel], a[sel], b[sel], ua, ub, dta, dtb, peers)
+                _reduce_units(arena, mem, row_tiles, row_idx[sel], a[sel], b[sel], ua, ub, dta, dtb, peers, skew_a)
                 continue
             src, dst, us, ud, ds_, dd = (b[sel], a[sel], ub, ua, dtb, dta) if rev else (a[sel], b[sel], ua, ub, dta, dtb)
             so = arena.offsets(src, us)[:, None] + np.arange(us)
@@ -168,7 +169,7 @@ def _transpose_blocks(arena, trans, rev: bool) -> None:
         mem[do] = mem[so]
 
 
-def _reduce_units(arena, mem, row_tiles, row_idx, a_off, b, ua, ub, dta, dtb, peers):
+def _reduce_units(arena, mem, row_tiles, row_idx, a_off, b, ua, ub, dta, dtb, peers, skew_a=False):
     es = {0: 2, 1: 2, 2: 4, 3: 8}[dta]
     n_el = ua // es
     for ti in np.unique(row_idx):
@@ -183,6 +184,8 @@ def _reduce_units(arena, mem, row_tiles, row_idx, a_off, b, ua, ub, dta, dtb, pe
         # gather each peer's units into a contiguous staging array, then let the C oracle combine them
         staged = []
         for base in bases:
+            assert skew_a or np.all((base + offs) % ua == 0), "misaligned vector access on a peer"
+            assert np.all((base + offs) % es == 0), "misaligned element on a peer"
             so = arena.offsets(base + offs, ua)[:, None] + np.arange(ua)
             staged.append(np.ascontiguousarray(mem[so]).reshape(-1).copy())
         ch = co.make_chunk(0, (0,), (n_units * n_el,), (1,), dta, dtb, peers=[s.ctypes.data for s in staged], op=op)
