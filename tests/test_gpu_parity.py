@@ -593,14 +593,16 @@ def test_random_batches_gpu(gpu_device, seed):
             wide = torch.zeros(shape, dtype=t.dtype, device=t.device)
             return wide[..., 1 : 1 + t.shape[-1]]
     merge = bool(rng.integers(2))
-    gpu_job = ReshardJob(specs, device=gpu_device, bucket_size=bucket_size, keep_globals=True, fill=cpu_fill, local_view=view)
+    mode = ["buckets", "buckets", "zero_copy", "direct"][int(rng.integers(4))]  # wire options must not change results
+    gpu_job = ReshardJob(specs, device=gpu_device, bucket_size=bucket_size, keep_globals=True, fill=cpu_fill, local_view=view,
+                         zero_copy=mode == "zero_copy", direct=mode == "direct")
     cpu_job = ReshardJob(specs, device="cpu", bucket_size=bucket_size, keep_globals=True, fill=cpu_fill, local_view=view)
     mirror_partials(gpu_job, cpu_job)
     gpu_job.run(merge_launches=merge)
     run_oracle(cpu_job)
     for i, spec in enumerate(specs):
         for r, t in gpu_job.target_locals[i].items():
-            assert_bit_equal(t, cpu_job.target_locals[i][r], f"seed {seed} {spec.name} rank {r}")
+            assert_bit_equal(t, cpu_job.target_locals[i][r], f"seed {seed} ({mode}) {spec.name} rank {r}")
 
 
 @pytest.mark.parametrize("dtype", [torch.int8, torch.bfloat16, torch.float32, torch.float64])
