@@ -172,7 +172,7 @@ def main():
     steps_of = (lambda p: p.merged_steps) if merge else (lambda p: p.steps)
     n_pack = sum(1 for p in send_plans for s in steps_of(p) if s[0] in ("pack", "reduce_pack"))
     n_self = sum(1 for p in send_plans + recv_plans for s in steps_of(p) if s[0] == "selfcopy")
-    n_unpack = sum(1 for p in send_plans + recv_plans for s in steps_of(p) if s[0] in ("unpack", "direct"))
+    n_unpack = sum(1 for p in send_plans + recv_plans for s in steps_of(p) if s[0] in ("unpack", "direct", "direct_reduce"))
 
     # algorithmic bytes: pack reads the source dtype and writes the wire dtype; unpack reads the wire
     # dtype and writes the target dtype; a reduce-pack reads every member's partial
@@ -258,6 +258,8 @@ def main():
         kernel_name = "etha_reduce_kernel"
     if dominant == "unpack" and args.direct:
         kernel_name = "etha_tile_kernel<false>"  # the direct copy runs source region -> target region
+        if any(s[0] == "direct_reduce" for p in recv_plans for s in steps_of(p)):
+            kernel_name = "etha_reduce_kernel"
     achieved = dom_bytes / (dom_ms * 1e-3) / 1e9
     out = {
         "metric": "effective reshard GB/s (pack+unpack, 1 GPU) and % of HBM peak",

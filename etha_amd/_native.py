@@ -14,7 +14,7 @@ import numpy as np
 from .build import LIB_PATH
 
 ETHA_MAX_NDIM = 8
-ABI_VERSION = 2
+ABI_VERSION = 3
 
 # element type codes (include/etha_reshard.h)
 F16, BF16, F32, F64, B8, B16, B32, B64 = range(8)
@@ -59,7 +59,7 @@ ROW_TILE = np.dtype(
         ("peer_first", "<u4"),
         ("n_peers", "<u4"),
         ("reduce_op", "<u4"),
-        ("pad", "<u4"),
+        ("via", "<u4"),
     ]
 )
 TRANS_TILE = np.dtype([("a", "<u8"), ("b", "<u8"), ("a_pitch", "<i8"), ("b_pitch", "<i8"), ("nj", "<u4"), ("nk", "<u4"),
@@ -98,6 +98,7 @@ _SIGNATURES = {
     "etha_last_error": (c_char_p, []),
     "etha_table_create": (c_int, [c_void_p, c_uint32, c_void_p, c_uint32, c_int, POINTER(c_void_p)]),
     "etha_selfcopy_table_create": (c_int, [c_void_p, c_void_p, c_uint32, c_int, POINTER(c_void_p)]),
+    "etha_direct_table_create": (c_int, [c_void_p, c_void_p, c_uint32, c_void_p, c_uint32, c_int, POINTER(c_void_p)]),
     "etha_table_destroy": (c_int, [c_void_p]),
     "etha_table_info": (c_int, [c_void_p, POINTER(TableInfo)]),
     "etha_table_read_tiles": (c_int, [c_void_p, c_int, c_void_p, c_uint64, POINTER(c_uint64)]),
@@ -168,14 +169,22 @@ class Table:
         return cls(out.value)
 
     @classmethod
-    def create_selfcopy(cls, src: np.ndarray, dst: np.ndarray, upload: bool = True) -> "Table":
+    def create_selfcopy(cls, src: np.ndarray, dst: np.ndarray, upload: bool = True,
+                        partial_ptrs: np.ndarray | None = None) -> "Table":
+        """Region-to-region table.  With ``partial_ptrs`` some sources may be Partial (``etha_direct_table_create``)."""
         src = np.ascontiguousarray(src, dtype=CHUNK_DESC)
         dst = np.ascontiguousarray(dst, dtype=CHUNK_DESC)
         if len(src) != len(dst):
             raise ValueError("src and dst descriptor arrays differ in length")
         out = c_void_p()
-        rc = lib().etha_selfcopy_table_create(src.ctypes.data, dst.ctypes.data, len(src), int(upload), byref(out))
-        _check("etha_selfcopy_table_create", rc)
+        if partial_ptrs is not None and len(partial_ptrs):
+            partial_ptrs = np.ascontiguousarray(partial_ptrs, dtype=np.uint64)
+            rc = lib().etha_direct_table_create(src.ctypes.data, dst.ctypes.data, len(src), partial_ptrs.ctypes.data,
+                                                len(partial_ptrs), int(upload), byref(out))
+            _check("etha_direct_table_create", rc)
+        else:
+            rc = lib().etha_selfcopy_table_create(src.ctypes.data, dst.ctypes.data, len(src), int(upload), byref(out))
+            _check("etha_selfcopy_table_create", rc)
         return cls(out.value)
 
     def info(self) -> TableInfo:

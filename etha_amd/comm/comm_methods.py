@@ -12,8 +12,8 @@ Here a bucket list is compiled once into tile programs and a call enqueues, in b
 * NONE buckets:    nothing - the primary's reduce-pack already read this member's partial;
 * with the wire's ``zero_copy_single_chunk`` option, a single-chunk source bucket whose bytes already lie
   contiguously in the tensor is lent, not packed: the consumer unpacks straight from the tensor;
-* with the wire's ``direct_same_device`` option no plain bucket is packed at all: the target bucket's
-  launch copies from the producer's chunk regions into its own tensors in one pass.
+* with the wire's ``direct_same_device`` option no bucket is packed at all: the target bucket's launch
+  copies (for a Partial source: reduces) from the producer's chunk regions into its own tensors in one pass.
 
 Consecutive buckets of the same kind can be merged into one launch (``merge_launches=True``).
 All work goes to one stream, so per-channel FIFO order and "pack before unpack" hold by stream
@@ -31,7 +31,8 @@ from .transfer import Transport
 
 __all__ = ["bucket_comm", "TransferPlan"]
 
-_PACK, _REDUCE, _UNPACK, _SELF, _LEND, _DIRECT = "pack", "reduce_pack", "unpack", "selfcopy", "lend", "direct"
+_PACK, _REDUCE, _UNPACK, _SELF, _LEND, _DIRECT, _DIRECT_REDUCE = (
+    "pack", "reduce_pack", "unpack", "selfcopy", "lend", "direct", "direct_reduce")
 
 
 class TransferPlan:
@@ -104,14 +105,17 @@ class TransferPlan:
                 slot = wire.slot_for_recv(bucket, idx)
                 if slot.sources is not None:  # direct wire: copy from the producer's regions, no bucket
                     first = len(local)
-                    for c, (src_t, src_slice, wire_dtype) in zip(bucket.chunks, slot.sources):
-                        if wire_dtype not in (src_t.dtype, c.tensor.dtype):
+                    reduce = slot.sources[0][3] is not None  # buckets never mix Partial and plain chunks
+                    for c, (src_t, src_slice, wire_dtype, peers) in zip(bucket.chunks, slot.sources):
+                        if peers is None and wire_dtype not in (src_t.dtype, c.tensor.dtype):
                             raise NotImplementedError(
                                 f"{bucket}: wire dtype {wire_dtype} differs from both tensor dtypes; one direct "
                                 "conversion cannot reproduce the two roundings")
-                        local.add_pair(src_t, src_slice, c.tensor, c.dst_slice, c.chunk_shape)
-                        self.direct_read_bytes += c.nbytes // wire_dtype.itemsize * src_t.element_size()
-                    self.steps.append((_DIRECT, first, len(bucket.chunks), slot))
+                        local.add_pair(src_t, src_slice, c.tensor, c.dst_slice, c.chunk_shape, peers=peers,
+                                       wire_dtype=wire_dtype)
+                        members = len(peers[0]) if peers is not None else 1
+                        self.direct_read_bytes += c.nbytes // wire_dtype.itemsize * src_t.element_size() * members
+                    self.steps.append((_DIRECT_REDUCE if reduce else _DIRECT, first, len(bucket.chunks), slot))
                     continue
                 first = len(recv)
                 for off, c in zip(bucket.offsets, bucket.chunks):
@@ -233,7 +237,7 @@ class TransferPlan:
                 self.recv_table.unpack(first, count, stream)
             elif kind == _SELF:
                 self.local_table.selfcopy(first, count, stream)
-            elif kind == _DIRECT:
+            elif kind in (_DIRECT, _DIRECT_REDUCE):
                 for s in slots:
                     if s is not None and s.filled == 0:
                         raise RuntimeError(

@@ -95,8 +95,8 @@ class Slot:
     drained: int = 0  # number of unpacks enqueued from it (per consumer bookkeeping is the wire's job)
     borrowed: bool = False  # the slot is source-tensor memory (zero-copy single-chunk bucket, direct wire), not pool memory
     keepalive: object = None  # the tensor(s) a borrowed slot aliases
-    # direct wire: per chunk of the send bucket ``(source tensor, src_slice, wire dtype)``; the consumer copies
-    # from these regions straight into its own tensors and no bucket buffer exists (ptr is 0)
+    # direct wire: per chunk of the send bucket ``(source tensor, src_slice, wire dtype, Partial peers or None)``;
+    # the consumer copies from these regions straight into its own tensors and no bucket buffer exists (ptr is 0)
     sources: list | None = None
 
 
@@ -145,9 +145,12 @@ class DescBuilder:
 
 
 class SelfCopyBuilder:
+    """Accumulates region-to-region rows: LOCAL chunks, and the chunks of a direct (bucket-less) wire."""
+
     def __init__(self) -> None:
         self.src: list[np.ndarray] = []
         self.dst: list[np.ndarray] = []
+        self.partial_ptrs: list[int] = []
         self.keepalive: list[torch.Tensor] = []
 
     def __len__(self) -> int:
@@ -157,8 +160,11 @@ class SelfCopyBuilder:
         src_t = chunk.src_tensor if chunk.src_tensor is not None else chunk.tensor
         self.add_pair(src_t, chunk.src_slice, chunk.tensor, chunk.dst_slice, chunk.chunk_shape)
 
-    def add_pair(self, src_t, src_slice: tuple, dst_t, dst_slice: tuple, chunk_shape: tuple) -> None:
-        """Copy ``src_t[src_slice]`` to ``dst_t[dst_slice]`` (same shape), converting between their dtypes."""
+    def add_pair(self, src_t, src_slice: tuple, dst_t, dst_slice: tuple, chunk_shape: tuple, peers=None,
+                 wire_dtype: torch.dtype | None = None) -> None:
+        """Copy ``src_t[src_slice]`` to ``dst_t[dst_slice]`` (same shape), converting between their dtypes.
+        ``peers = (tensors, op)`` makes the source a Partial one: the members' slices are combined, rounded to
+        ``wire_dtype`` and then converted, as the bucket path would."""
         a = np.zeros((), dtype=nat.CHUNK_DESC)
         b = np.zeros((), dtype=nat.CHUNK_DESC)
         fill_region(a, src_t, src_slice, chunk_shape)
@@ -166,6 +172,22 @@ class SelfCopyBuilder:
         check_cast(src_t.dtype, dst_t.dtype)
         a["wire_dtype"] = a["tensor_dtype"]
         b["wire_dtype"] = b["tensor_dtype"]
+        if peers is not None:
+            tensors, op = peers
+            wire = wire_dtype or src_t.dtype
+            check_cast(src_t.dtype, wire)
+            check_cast(wire, dst_t.dtype)
+            for t in tensors:
+                if t.dtype != src_t.dtype or tuple(t.shape) != tuple(src_t.shape) or t.stride() != src_t.stride():
+                    raise NotImplementedError("Partial peers must share dtype, shape and strides")
+                if t.device != src_t.device:
+                    raise NotImplementedError("Partial peers must live on the same device")
+            a["wire_dtype"] = dtype_code(wire)
+            a["n_partials"] = len(tensors)
+            a["partial_first"] = len(self.partial_ptrs)
+            a["reduce_op"] = nat.REDUCE_OPS[op]
+            self.partial_ptrs.extend(t.data_ptr() for t in tensors)
+            self.keepalive.extend(tensors)
         self.src.append(a)
         self.dst.append(b)
         self.keepalive += [src_t, dst_t]
@@ -173,7 +195,8 @@ class SelfCopyBuilder:
     def build(self, upload: bool = True) -> nat.Table | None:
         if not self.src:
             return None
-        return nat.Table.create_selfcopy(np.stack(self.src), np.stack(self.dst), upload=upload)
+        ptrs = np.asarray(self.partial_ptrs, dtype=np.uint64) if self.partial_ptrs else None
+        return nat.Table.create_selfcopy(np.stack(self.src), np.stack(self.dst), upload=upload, partial_ptrs=ptrs)
 
 
 def region_hull(tensor, slices: tuple) -> tuple[int, int]:

@@ -256,4 +256,4 @@ class Bucket:
     def finalize(self, wire=None) -> None:
         """Target bucket (and staged self-copy): enqueue its unpack launch (``Bucket.finalize``,
         ``ir.py:300-310``)."""
-        self._plan(wire).run_kinds(("unpack", "direct"))
+        self._plan(wire).run_kinds(("unpack", "direct", "direct_reduce"))

@@ -88,8 +88,8 @@ class LoopbackWire:
         # path sends straight from it (ir.py:238-244).  The producer must then leave that tensor alone
         # until the consumer has unpacked: "sent" no longer means "copied".
         self.zero_copy_single_chunk = False
-        # True: no bucket buffers at all for plain (non-Partial) buckets.  Producer and consumer tensors are
-        # on one device, so the consumer's launch reads the producer's chunk regions and writes its own:
+        # True: no bucket buffers at all.  Producer and consumer tensors are on one device, so the consumer's
+        # launch reads the producer's chunk regions (every member's, for a Partial source) and writes its own:
         # one pass (read source dtype, write target dtype) instead of pack + unpack, and no pool memory.
         # This is what a pull over a peer mapping does between GPUs, minus the link.  Like a lent bucket,
         # a "sent" tensor must be left alone until the consumer has run.  Only within one process.
@@ -120,10 +120,11 @@ class LoopbackWire:
         if index != len(sent):
             raise RuntimeError(f"{bucket}: send buckets must be planned in order")
         slot = None
-        if self.direct_same_device and not any(c.source_partial_groups for c in bucket.chunks):
+        if self.direct_same_device:
             self._pool_for(device)
             slot = Slot(ptr=0, nbytes=bucket.total_bytes, lo=0, hi=0, borrowed=True)
-            slot.sources = [(c.tensor, c.src_slice, c.transfer_dtype or c.tensor.dtype) for c in bucket.chunks]
+            slot.sources = [(c.tensor, c.src_slice, c.transfer_dtype or c.tensor.dtype, c.partial_peers())
+                            for c in bucket.chunks]
             slot.keepalive = [c.tensor for c in bucket.chunks]
         if slot is None and self.zero_copy_single_chunk:
             from .device_plan import zero_copy_region

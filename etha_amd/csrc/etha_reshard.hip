@@ -82,7 +82,7 @@ struct RowTile {     // walks rows of `run` units; covers units [c0, c0+n) count
   uint32_t peer_first;  // reduce tiles: index of the first peer base in the peers array
   uint32_t n_peers;     // 0 = plain tile
   uint32_t reduce_op;
-  uint32_t pad;
+  uint32_t via;         // reduce tiles: 0, or 1 + ETHA_* dtype the result is rounded to before the b-side dtype
 };
 static_assert(sizeof(RowTile) == 64, "RowTile layout");
 
@@ -346,10 +346,21 @@ struct LoadF32 {
   }
 };
 
+// A reduction that writes a tensor directly (no bucket in between) still rounds the way the bucket path
+// does: accumulator -> wire dtype -> tensor dtype.  `via` names the wire dtype when it differs from the
+// b-side dtype (0 = no intermediate rounding).
+__device__ __forceinline__ float round_via(uint32_t via, float r) {
+  switch (via) {
+    case 1 + ETHA_F16: return to_f32(TagF16(), from_f32(TagF16(), r));
+    case 1 + ETHA_BF16: return to_f32(TagBF16(), from_f32(TagBF16(), r));
+    default: return r;
+  }
+}
+
 // f16/bf16/f32 partials: fp32 accumulation, peers combined strictly in list (= rank) order.
 template <typename S, typename D, int N>
-__device__ __forceinline__ void reduce_f32(const uint64_t* __restrict__ peers, uint32_t np, uint32_t op, uint64_t a_off,
-                                           uint64_t dst) {
+__device__ __forceinline__ void reduce_f32(const uint64_t* __restrict__ peers, uint32_t np, uint32_t op, uint32_t via,
+                                           uint64_t a_off, uint64_t dst) {
   float acc[N];
   LoadF32<S, N>::run(peers[0] + a_off, acc);
   uint32_t p = 1;
@@ -373,15 +384,15 @@ __device__ __forceinline__ void reduce_f32(const uint64_t* __restrict__ peers, u
   for (int i = 0; i < N; i++) {
     float r = acc[i];
     if (op == ETHA_AVG) r = r / cnt;
-    out.set(i, from_f32(D(), r));
+    out.set(i, from_f32(D(), round_via(via, r)));
   }
   out.store(dst);
 }
 
 // f64 partials: f64 accumulation; result converted like a plain f64 -> D move.
 template <typename D, int N>
-__device__ __forceinline__ void reduce_f64(const uint64_t* __restrict__ peers, uint32_t np, uint32_t op, uint64_t a_off,
-                                           uint64_t dst) {
+__device__ __forceinline__ void reduce_f64(const uint64_t* __restrict__ peers, uint32_t np, uint32_t op, uint32_t via,
+                                           uint64_t a_off, uint64_t dst) {
   double acc[N];
   {
     Pack<uint64_t, N> in;
@@ -400,44 +411,44 @@ __device__ __forceinline__ void reduce_f64(const uint64_t* __restrict__ peers, u
   for (int i = 0; i < N; i++) {
     double r = acc[i];
     if (op == ETHA_AVG) r = r / (double)np;
-    if (sizeof(typename D::bits) == 8)
+    if (sizeof(typename D::bits) == 8 && via == 0)
       out.set(i, (typename D::bits)__builtin_bit_cast(uint64_t, r));
     else {
       float rf = (float)r;
       asm volatile("" : "+v"(rf));  // two roundings, as in the plain f64 -> D move
-      out.set(i, from_f32(D(), rf));
+      out.set(i, from_f32(D(), round_via(via, rf)));
     }
   }
   out.store(dst);
 }
 
 template <typename S, typename D>
-__device__ __forceinline__ void reduce_pair(bool vec, const uint64_t* peers, uint32_t np, uint32_t op, uint64_t a_off,
-                                            uint64_t dst) {
+__device__ __forceinline__ void reduce_pair(bool vec, const uint64_t* peers, uint32_t np, uint32_t op, uint32_t via,
+                                            uint64_t a_off, uint64_t dst) {
   constexpr int kMaxBytes = sizeof(typename S::bits) > sizeof(typename D::bits) ? sizeof(typename S::bits)
                                                                                   : sizeof(typename D::bits);
   constexpr int kN = 16 / kMaxBytes;
   if (sizeof(typename S::bits) == 8) {
     if (vec)
-      reduce_f64<D, kN>(peers, np, op, a_off, dst);
+      reduce_f64<D, kN>(peers, np, op, via, a_off, dst);
     else
-      reduce_f64<D, 1>(peers, np, op, a_off, dst);
+      reduce_f64<D, 1>(peers, np, op, via, a_off, dst);
   } else {
     if (vec)
-      reduce_f32<S, D, kN>(peers, np, op, a_off, dst);
+      reduce_f32<S, D, kN>(peers, np, op, via, a_off, dst);
     else
-      reduce_f32<S, D, 1>(peers, np, op, a_off, dst);
+      reduce_f32<S, D, 1>(peers, np, op, via, a_off, dst);
   }
 }
 
 template <typename S>
 __device__ __forceinline__ void reduce_from(uint32_t dd, bool vec, const uint64_t* peers, uint32_t np, uint32_t op,
-                                            uint64_t a_off, uint64_t dst) {
+                                            uint32_t via, uint64_t a_off, uint64_t dst) {
   switch (dd) {
-    case ETHA_F16: reduce_pair<S, TagF16>(vec, peers, np, op, a_off, dst); break;
-    case ETHA_BF16: reduce_pair<S, TagBF16>(vec, peers, np, op, a_off, dst); break;
-    case ETHA_F32: reduce_pair<S, TagF32>(vec, peers, np, op, a_off, dst); break;
-    default: reduce_pair<S, TagF64>(vec, peers, np, op, a_off, dst); break;
+    case ETHA_F16: reduce_pair<S, TagF16>(vec, peers, np, op, via, a_off, dst); break;
+    case ETHA_BF16: reduce_pair<S, TagBF16>(vec, peers, np, op, via, a_off, dst); break;
+    case ETHA_F32: reduce_pair<S, TagF32>(vec, peers, np, op, via, a_off, dst); break;
+    default: reduce_pair<S, TagF64>(vec, peers, np, op, via, a_off, dst); break;
   }
 }
 
@@ -455,10 +466,10 @@ __global__ __launch_bounds__(ETHA_BLOCK_THREADS) void etha_reduce_kernel(const R
   const bool vec = (meta & kMetaVec) != 0;
   const uint32_t dd = (meta >> kMetaDtbShift) & 15u;
   switch ((meta >> kMetaDtaShift) & 15u) {
-    case ETHA_F16: reduce_from<TagF16>(dd, vec, peers, t.n_peers, t.reduce_op, a_off, dst); break;
-    case ETHA_BF16: reduce_from<TagBF16>(dd, vec, peers, t.n_peers, t.reduce_op, a_off, dst); break;
-    case ETHA_F32: reduce_from<TagF32>(dd, vec, peers, t.n_peers, t.reduce_op, a_off, dst); break;
-    default: reduce_from<TagF64>(dd, vec, peers, t.n_peers, t.reduce_op, a_off, dst); break;
+    case ETHA_F16: reduce_from<TagF16>(dd, vec, peers, t.n_peers, t.reduce_op, t.via, a_off, dst); break;
+    case ETHA_BF16: reduce_from<TagBF16>(dd, vec, peers, t.n_peers, t.reduce_op, t.via, a_off, dst); break;
+    case ETHA_F32: reduce_from<TagF32>(dd, vec, peers, t.n_peers, t.reduce_op, t.via, a_off, dst); break;
+    default: reduce_from<TagF64>(dd, vec, peers, t.n_peers, t.reduce_op, t.via, a_off, dst); break;
   }
 }
 
@@ -570,7 +581,7 @@ struct Builder {
 constexpr uint64_t kMaxTiles = 0x7fff0000ull / kBlocksPerTile;  // grid.x limit with margin
 
 struct ReduceSpec {
-  uint32_t n_peers = 0, peer_first = 0, op = 0;
+  uint32_t n_peers = 0, peer_first = 0, op = 0, via = 0;
 };
 
 // Emit tiles moving region A (dtype dta) to/from region B (dtype dtb); both have the same shape.
@@ -804,6 +815,7 @@ int compile_pair(Builder& bld, uint32_t idx, const Region& A0, const Region& B0,
         t.peer_first = red.peer_first;
         t.n_peers = red.n_peers;
         t.reduce_op = red.op;
+        t.via = red.via;
         bld.row.push_back(t);
       }
     }
@@ -1072,8 +1084,8 @@ int etha_table_create(const EthaChunkDesc* descs, uint32_t n_chunks, const uint6
   return finish_table(bld, t, upload, out);
 }
 
-int etha_selfcopy_table_create(const EthaChunkDesc* src, const EthaChunkDesc* dst, uint32_t n_chunks, int upload,
-                               EthaTable** out) {
+int etha_direct_table_create(const EthaChunkDesc* src, const EthaChunkDesc* dst, uint32_t n_chunks,
+                             const uint64_t* partial_ptrs, uint32_t n_partial_ptrs, int upload, EthaTable** out) {
   if (!out) return fail(ETHA_ERR_INVALID, "null out");
   *out = nullptr;
   if (n_chunks && (!src || !dst)) return fail(ETHA_ERR_INVALID, "null descriptor array");
@@ -1083,15 +1095,45 @@ int etha_selfcopy_table_create(const EthaChunkDesc* src, const EthaChunkDesc* ds
     bld.run_begin.push_back((uint32_t)bld.run.size());
     bld.row_begin.push_back((uint32_t)bld.row.size());
     bld.trans_begin.push_back((uint32_t)bld.trans.size());
-    if (src[i].n_partials || dst[i].n_partials)
-      return fail(ETHA_ERR_UNSUPPORTED, "chunk %u: self-copy of a Partial source is not implemented", i);
+    if (dst[i].n_partials) return fail(ETHA_ERR_INVALID, "chunk %u: a destination cannot be Partial", i);
     Region A, B;
-    int rc = tensor_region(src[i], i, src[i].tensor_ptr, false, &A);
-    if (rc != ETHA_OK) return rc;
+    ReduceSpec red;
+    std::vector<uint64_t> peer_bases;
+    const EthaChunkDesc& d = src[i];
+    int rc;
+    if (d.n_partials) {
+      if (d.reduce_op > ETHA_PRODUCT) return fail(ETHA_ERR_INVALID, "chunk %u: unknown reduce_op %u", i, d.reduce_op);
+      if (!partial_ptrs || (uint64_t)d.partial_first + d.n_partials > n_partial_ptrs)
+        return fail(ETHA_ERR_INVALID, "chunk %u: partial pointer range outside partial_ptrs", i);
+      if (dtype_size(d.wire_dtype) == 0) return fail(ETHA_ERR_INVALID, "chunk %u: unknown wire_dtype %u", i, d.wire_dtype);
+      EthaChunkDesc dz = d;
+      dz.tensor_lo = dz.tensor_hi = 0;  // the single lo/hi pair cannot describe several peers
+      for (uint32_t p = 0; p < d.n_partials; p++) {
+        Region tmp;
+        rc = tensor_region(dz, i, partial_ptrs[d.partial_first + p], false, &tmp);
+        if (rc != ETHA_OK) return rc;
+        peer_bases.push_back(partial_ptrs[d.partial_first + p]);
+      }
+      rc = tensor_region(dz, i, 0, true, &A);  // offsets relative to a peer base
+      if (rc != ETHA_OK) return rc;
+      red.n_peers = d.n_partials;
+      red.peer_first = d.partial_first;
+      red.op = d.reduce_op;
+      // the bucket path rounds the accumulator to the wire dtype first; keep that rounding when it is not the last one
+      if (d.wire_dtype != dst[i].tensor_dtype) {
+        if (!is_float(d.wire_dtype))
+          return fail(ETHA_ERR_UNSUPPORTED, "chunk %u: Partial reduce needs a floating wire dtype", i);
+        red.via = 1 + d.wire_dtype;
+      }
+      bld.is_reduce[i] = 1;
+    } else {
+      rc = tensor_region(d, i, d.tensor_ptr, false, &A);
+      if (rc != ETHA_OK) return rc;
+    }
     rc = tensor_region(dst[i], i, dst[i].tensor_ptr, false, &B);
     if (rc != ETHA_OK) return rc;
     bld.payload_bytes += region_numel(A) * (uint64_t)dtype_size(dst[i].tensor_dtype);
-    rc = compile_pair(bld, i, A, B, src[i].tensor_dtype, dst[i].tensor_dtype, ReduceSpec(), {});
+    rc = compile_pair(bld, i, A, B, d.tensor_dtype, dst[i].tensor_dtype, red, peer_bases);
     if (rc != ETHA_OK) return rc;
   }
   bld.run_begin.push_back((uint32_t)bld.run.size());
@@ -1101,7 +1143,15 @@ int etha_selfcopy_table_create(const EthaChunkDesc* src, const EthaChunkDesc* ds
   if (!t) return fail(ETHA_ERR_NOMEM, "out of host memory");
   t->kind = 1;
   t->n_chunks = n_chunks;
+  if (partial_ptrs && n_partial_ptrs) t->h_peers.assign(partial_ptrs, partial_ptrs + n_partial_ptrs);
   return finish_table(bld, t, upload, out);
+}
+
+int etha_selfcopy_table_create(const EthaChunkDesc* src, const EthaChunkDesc* dst, uint32_t n_chunks, int upload,
+                               EthaTable** out) {
+  for (uint32_t i = 0; src && i < n_chunks; i++)
+    if (src[i].n_partials) return fail(ETHA_ERR_UNSUPPORTED, "chunk %u: a same-rank copy has no Partial source", i);
+  return etha_direct_table_create(src, dst, n_chunks, nullptr, 0, upload, out);
 }
 
 int etha_table_destroy(EthaTable* table) {
@@ -1236,7 +1286,15 @@ int etha_reduce_pack_bucket(const EthaTable* t, uint32_t first, uint32_t count, 
 int etha_selfcopy_bucket(const EthaTable* t, uint32_t first, uint32_t count, void* stream) {
   const int rc = check_range(t, first, count, 1);
   if (rc != ETHA_OK) return rc;
-  return launch_tiles<false>(t, first, count, stream);
+  const uint32_t n_reduce = t->reduce_prefix[first + count] - t->reduce_prefix[first];
+  if (n_reduce == 0) return launch_tiles<false>(t, first, count, stream);
+  if (n_reduce != count) return fail(ETHA_ERR_INVALID, "range mixes Partial and plain chunks; launch them separately");
+  const uint32_t w0 = t->row_begin[first], w1 = t->row_begin[first + count];
+  if (w1 == w0) return ETHA_OK;
+  hipLaunchKernelGGL(etha_reduce_kernel, dim3((w1 - w0) * kBlocksPerTile), dim3(kBlockThreads), 0, (hipStream_t)stream,
+                     t->d_row + w0, t->d_peers);
+  HIP_TRY(hipGetLastError());
+  return ETHA_OK;
 }
 
 int etha_arena_create(uint64_t nbytes, void** out_ptr) {

@@ -31,7 +31,7 @@
 extern "C" {
 #endif
 
-#define ETHA_ABI_VERSION 2
+#define ETHA_ABI_VERSION 3
 #define ETHA_MAX_NDIM 8
 
 /* status codes */
@@ -120,6 +120,19 @@ int etha_table_create(const EthaChunkDesc* descs, uint32_t n_chunks, const uint6
 int etha_selfcopy_table_create(const EthaChunkDesc* src, const EthaChunkDesc* dst, uint32_t n_chunks, int upload,
                                EthaTable** out);
 
+/*
+ * Region-to-region copies where producer and consumer tensors sit on one device and no bucket buffer is wanted:
+ * src region i is copied (converted) straight into dst region i.  A src with n_partials > 0 is a Partial
+ * source: its peers (partial_ptrs, as in etha_table_create) are combined as in etha_reduce_pack_bucket and the
+ * result is rounded to src.wire_dtype and then converted to dst.tensor_dtype, the two roundings of the bucket
+ * path (Chunk.prepare's cast to transfer_dtype, ir.py:125-126, then Chunk.finalize's cast, ir.py:137-138).
+ * For plain chunks wire_dtype is ignored.  Run with etha_selfcopy_bucket; a launched range must be all plain or
+ * all Partial chunks.  etha_selfcopy_table_create is this function without Partial sources.
+ * No counterpart in the reference (its buckets always cross a process group).
+ */
+int etha_direct_table_create(const EthaChunkDesc* src, const EthaChunkDesc* dst, uint32_t n_chunks,
+                             const uint64_t* partial_ptrs, uint32_t n_partial_ptrs, int upload, EthaTable** out);
+
 int etha_table_destroy(EthaTable* table);
 int etha_table_info(const EthaTable* table, EthaTableInfo* out);
 
@@ -171,7 +184,7 @@ int etha_unpack_bucket(const EthaTable* table, uint32_t first, uint32_t count, v
  */
 int etha_reduce_pack_bucket(const EthaTable* table, uint32_t first, uint32_t count, void* stream);
 
-/* Run chunks [first, first+count) of a self-copy table.  One kernel launch. */
+/* Run chunks [first, first+count) of a self-copy or direct table.  One kernel launch. */
 int etha_selfcopy_bucket(const EthaTable* table, uint32_t first, uint32_t count, void* stream);
 
 /*

@@ -657,8 +657,8 @@ def test_zero_copy_single_chunk_buckets(gpu_device):
 
 def test_direct_same_device_wire(gpu_device):
     """With the direct wire no plain bucket is packed: the target bucket's launch copies from the producer's
-    regions in one pass.  Same results as the bucket path for P2P, BROADCAST, LOCAL, converting and strided
-    layouts; Partial sources still go through reduce-pack + unpack; no pool memory for the plain buckets."""
+    regions in one pass - for a Partial source it reduces every member's region.  Same results as the bucket
+    path for P2P, BROADCAST, LOCAL, converting, strided and Partial layouts; no pool memory."""
     src = mesh_of(0, (2, 2))
     specs = [
         TensorSpec("a", (64, 48), src, (Shard(0), Shard(1)), mesh_of(4, (2,)), (Replicate(),), torch.float32, seed=1),
@@ -668,6 +668,11 @@ def test_direct_same_device_wire(gpu_device):
         TensorSpec("d", (8, 128), src, (Shard(0), Shard(1)), mesh_of(4, (2, 2)), (Shard(1), Replicate()),
                    torch.bfloat16, torch.float32, seed=4),
         TensorSpec("p", (64, 32), mesh_of(0, (4,)), (Partial(),), mesh_of(4, (2,)), (Shard(0),), torch.bfloat16, seed=5),
+        # bf16 partials into an fp32 target: the sum is still rounded to the bf16 wire dtype before widening
+        TensorSpec("pw", (48, 20), mesh_of(0, (4,)), (Partial("avg"),), mesh_of(4, (2,)), (Shard(1),), torch.bfloat16,
+                   torch.float32, seed=6),
+        TensorSpec("pn", (16, 24), mesh_of(0, (2, 2)), (Partial(), Shard(0)), mesh_of(4, (2,)), (Replicate(),), torch.float32,
+                   torch.bfloat16, seed=7),
     ]
     for bucket_size in (1, 4096, 1 << 20):
         for merge in (False, True):
@@ -687,9 +692,9 @@ def test_direct_same_device_wire(gpu_device):
                         assert_bit_equal(t, before[i][r], f"{spec.name} source {r} mutated")
             kinds = {s[0] for bs in list(gpu_job.send_buckets.values()) + list(gpu_job.recv_buckets.values())
                      for s in gpu_job.wire.plan(bs).steps}
-            assert "direct" in kinds and "lend" in kinds and "reduce_pack" in kinds
-            plain_packs = [s for bs in gpu_job.send_buckets.values() for s in gpu_job.wire.plan(bs).steps if s[0] == "pack"]
-            assert not plain_packs  # (staged self-copies would pack; this layout has none)
+            assert {"direct", "direct_reduce", "lend"} <= kinds
+            assert not kinds & {"pack", "reduce_pack", "unpack"}  # (staged self-copies would pack; this layout has none)
+            assert gpu_job.wire.pool is None or gpu_job.wire.pool.reserved_bytes == 0
     with pytest.raises(NotImplementedError):
         gpu_job.wire.export_manifest()
 

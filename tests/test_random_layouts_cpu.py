@@ -101,8 +101,20 @@ def _interpret(job, merged: bool):
                 execute(p.recv_table, mem, "unpack", first, count, ordered=merged and len(slots) > 1)
             elif kind in ("selfcopy", "direct"):
                 execute(p.local_table, mem, "selfcopy", first, count, ordered=merged and len(slots) > 1)
+            elif kind == "direct_reduce":
+                execute(p.local_table, mem, "selfcopy", first, count, peers=_direct_peers_of(p))
             else:
                 assert kind == "lend"  # nothing runs for a lent bucket
+
+
+def _direct_peers_of(plan):
+    """Peer pointers of a plan's direct-reduce chunks, in the order the plan registered them."""
+    ptrs = []
+    for kind, _, _, slot in plan.steps:
+        if kind == "direct_reduce":
+            for _, _, _, peers in slot.sources:
+                ptrs.extend(t.data_ptr() for t in peers[0])
+    return np.asarray(ptrs, dtype=np.uint64) if ptrs else None
 
 
 def _peers_of(plan):

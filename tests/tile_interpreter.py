@@ -179,7 +179,9 @@ def _reduce_units(arena, mem, row_tiles, row_idx, a_off, b, ua, ub, dta, dtb, pe
         op = {0: "sum", 1: "avg", 2: "max", 3: "min", 4: "product"}[int(t["reduce_op"])]
         offs = a_off[sel]
         n_units = len(offs)
-        out = np.zeros(n_units * n_el, dtype=_CODE_RAW[dtb])
+        via = int(t["via"])  # 0, or 1 + the dtype the result is rounded to before the b-side dtype
+        out_dt = via - 1 if via else dtb
+        out = np.zeros(n_units * n_el, dtype=_CODE_RAW[out_dt])
         scratch = np.zeros(n_units * n_el, dtype=np.float64)
         # gather each peer's units into a contiguous staging array, then let the C oracle combine them
         staged = []
@@ -188,8 +190,10 @@ def _reduce_units(arena, mem, row_tiles, row_idx, a_off, b, ua, ub, dta, dtb, pe
             assert np.all((base + offs) % es == 0), "misaligned element on a peer"
             so = arena.offsets(base + offs, ua)[:, None] + np.arange(ua)
             staged.append(np.ascontiguousarray(mem[so]).reshape(-1).copy())
-        ch = co.make_chunk(0, (0,), (n_units * n_el,), (1,), dta, dtb, peers=[s.ctypes.data for s in staged], op=op)
+        ch = co.make_chunk(0, (0,), (n_units * n_el,), (1,), dta, out_dt, peers=[s.ctypes.data for s in staged], op=op)
         assert co.lib().oracle_reduce(ch, out.ctypes.data, scratch.ctypes.data) == 0
+        if via:
+            out = co.cast(out, out_dt, dtb, _CODE_RAW[dtb])
         do = arena.offsets(b[sel], ub)[:, None] + np.arange(ub)
         if arena.writes is not None:
             np.add.at(arena.writes, do.reshape(-1), 1)
