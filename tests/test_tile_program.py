@@ -292,3 +292,65 @@ def test_transposed_parent_uses_lds_blocks(dt):
     oc2 = co.make_chunk(want2.ctypes.data, start, cshape, strides, dt, dt, bucket_off=0)
     assert co.lib().oracle_unpack_bucket(oc2, 1, want.ctypes.data, scratch.ctypes.data) == 0
     assert np.array_equal(arena.bytes_at(t2, rows * cols * es), want2)
+
+
+@pytest.mark.parametrize("tdt,wdt,ddt", [(nat.BF16, nat.BF16, nat.BF16), (nat.BF16, nat.BF16, nat.F32),
+                                         (nat.F32, nat.BF16, nat.BF16), (nat.F16, nat.F16, nat.BF16),
+                                         (nat.F64, nat.F32, nat.F32)])
+def test_direct_reduce_tiles_round_through_the_wire_dtype(tdt, wdt, ddt):
+    """A Partial source reduced straight into a (strided) target region: the result must equal reduce-pack to
+    the wire dtype followed by an unpack conversion to the target dtype - two roundings, not one."""
+    pshape, start, cshape = (20, 72), (2, 8), (16, 40)
+    dshape, dstart = (16, 100), (0, 30)
+    es, ws, ds = ES[tdt], ES[wdt], ES[ddt]
+    pn, cn, dn = int(np.prod(pshape)), int(np.prod(cshape)), int(np.prod(dshape))
+    n_peers = 3
+    arena = HostArena(n_peers * pn * es + dn * ds + 16384)
+    raw_of = {2: np.uint16, 4: np.uint32, 8: np.uint64}
+    peers = []
+    for p in range(n_peers):
+        addr = arena.alloc(pn * es)
+        vals = rs.randn(pn).astype(np.float64)
+        arena.bytes_at(addr, pn * es)[:] = co.cast(vals.view(np.uint64), co.F64, tdt, raw_of[es]).view(np.uint8)
+        peers.append(addr)
+    d_addr = arena.alloc(dn * ds)
+    arena.bytes_at(d_addr, dn * ds)[:] = 0xAB
+    src = _mk_desc(0, 0, 0, 0, 0, 0, start, cshape, [pshape[1], 1], tdt, wdt)
+    src["n_partials"], src["partial_first"], src["reduce_op"] = n_peers, 0, nat.REDUCE_OPS["sum"]
+    dst = _mk_desc(d_addr, d_addr, d_addr + dn * ds, 0, 0, 0, dstart, cshape, [dshape[1], 1], ddt, ddt)
+    ptrs = np.asarray(peers, dtype=np.uint64)
+    table = nat.Table.create_selfcopy(src.reshape(1), dst.reshape(1), upload=False, partial_ptrs=ptrs)
+    run, row = table.tiles()
+    assert len(run) == 0 and np.all(row["n_peers"] == n_peers)
+    assert np.all(row["via"] == (0 if wdt == ddt else 1 + wdt))
+    execute(table, arena, "selfcopy", peers=ptrs)
+    # expectation: the oracle's reduce-pack into a bucket of the wire dtype, then an element-wise cast
+    bucket = np.zeros(cn * ws, dtype=np.uint8)
+    scratch = np.zeros(cn * 8, dtype=np.uint8)
+    oc = co.make_chunk(0, start, cshape, [pshape[1], 1], tdt, wdt, peers=peers, op="sum")
+    assert co.lib().oracle_pack_bucket(oc, 1, bucket.ctypes.data, scratch.ctypes.data) == 0
+    want = co.cast(bucket.view(raw_of[ws]), wdt, ddt, raw_of[ds]).reshape(cshape)
+    got = arena.bytes_at(d_addr, dn * ds).view(raw_of[ds]).reshape(dshape)
+    assert np.array_equal(got[dstart[0] : dstart[0] + cshape[0], dstart[1] : dstart[1] + cshape[1]], want)
+    inside = np.zeros(dshape, dtype=bool)
+    inside[dstart[0] : dstart[0] + cshape[0], dstart[1] : dstart[1] + cshape[1]] = True
+    fill = np.frombuffer(bytes([0xAB]) * ds, dtype=raw_of[ds])[0]
+    assert np.all(got[~inside] == fill), "bytes outside the destination region were written"
+
+
+def test_direct_table_rejects_partial_destinations_and_selfcopy_rejects_partial_sources():
+    arena = HostArena(8192)
+    t = arena.alloc(1024)
+    src = _mk_desc(t, t, t + 1024, 0, 0, 0, (0,), (16,), (1,), nat.F32, nat.F32)
+    dst = _mk_desc(t, t, t + 1024, 0, 0, 0, (32,), (16,), (1,), nat.F32, nat.F32)
+    bad_dst = dst.copy()
+    bad_dst["n_partials"] = 2
+    ptrs = np.asarray([t, t], dtype=np.uint64)
+    with pytest.raises(nat.EthaNativeError, match="destination cannot be Partial"):
+        nat.Table.create_selfcopy(src.reshape(1), bad_dst.reshape(1), upload=False, partial_ptrs=ptrs)
+    bad_src = src.copy()
+    bad_src["n_partials"] = 2
+    with pytest.raises(nat.EthaNativeError, match="no Partial source"):
+        nat.Table.create_selfcopy(bad_src.reshape(1), dst.reshape(1), upload=False)
+    with pytest.raises(nat.EthaNativeError, match="outside partial_ptrs"):
+        nat.Table.create_selfcopy(bad_src.reshape(1), dst.reshape(1), upload=False, partial_ptrs=ptrs[:1])
