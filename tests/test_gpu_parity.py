@@ -705,3 +705,20 @@ def test_direct_wire_full_size_llama(gpu_device):
     job.run(merge_launches=True)
     _check_targets_against_global(job, specs)
     assert job.wire.pool is None or job.wire.pool.reserved_bytes == 0
+
+
+def test_direct_table_launch_refuses_mixed_ranges(gpu_device):
+    """A launched range of a direct table is all plain or all Partial chunks (they run in different kernels)."""
+    from etha_amd._native import EthaNativeError
+
+    one = (mesh_of(0, (2,)), mesh_of(2, (1,)))
+    specs = [TensorSpec("a", (8, 16), one[0], (Shard(0),), one[1], (Replicate(),), torch.float32, seed=1),
+             TensorSpec("p", (8, 16), one[0], (Partial(),), one[1], (Replicate(),), torch.float32, seed=2)]
+    job = ReshardJob(specs, device=gpu_device, bucket_size=1, direct=True)
+    job.run()
+    plan = job.wire.plan(job.recv_buckets[2])
+    kinds = [s[0] for s in plan.steps]
+    assert "direct" in kinds and "direct_reduce" in kinds
+    total = sum(s[2] for s in plan.steps)
+    with pytest.raises(EthaNativeError, match="mixes Partial and plain"):
+        plan.local_table.selfcopy(0, total)
