@@ -100,6 +100,14 @@ class Slot:
     sources: list | None = None
 
 
+def _rows_to_array(rows: list[np.ndarray]) -> np.ndarray:
+    """One descriptor array from 0-d rows (np.stack spends most of its time promoting the struct dtype)."""
+    out = np.empty(len(rows), dtype=nat.CHUNK_DESC)
+    for i, r in enumerate(rows):
+        out[i] = r
+    return out
+
+
 class DescBuilder:
     """Accumulates descriptor rows bucket by bucket and remembers each bucket's chunk range."""
 
@@ -139,7 +147,7 @@ class DescBuilder:
     def build(self, upload: bool = True) -> nat.Table | None:
         if not self.rows:
             return None
-        descs = np.stack(self.rows)
+        descs = _rows_to_array(self.rows)
         ptrs = np.asarray(self.partial_ptrs, dtype=np.uint64) if self.partial_ptrs else None
         return nat.Table.create(descs, ptrs, upload=upload)
 
@@ -196,7 +204,8 @@ class SelfCopyBuilder:
         if not self.src:
             return None
         ptrs = np.asarray(self.partial_ptrs, dtype=np.uint64) if self.partial_ptrs else None
-        return nat.Table.create_selfcopy(np.stack(self.src), np.stack(self.dst), upload=upload, partial_ptrs=ptrs)
+        return nat.Table.create_selfcopy(_rows_to_array(self.src), _rows_to_array(self.dst), upload=upload,
+                                         partial_ptrs=ptrs)
 
 
 def region_hull(tensor, slices: tuple) -> tuple[int, int]:
