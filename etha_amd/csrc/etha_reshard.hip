@@ -584,160 +584,181 @@ struct ReduceSpec {
   uint32_t n_peers = 0, peer_first = 0, op = 0, via = 0;
 };
 
-// Emit tiles moving region A (dtype dta) to/from region B (dtype dtb); both have the same shape.
-// For reduce chunks A.base is 0 and tile addresses on the a side are offsets from the peer bases;
-// `align_bases` then lists the peers' real bases for the alignment decision.
-int compile_pair(Builder& bld, uint32_t idx, const Region& A0, const Region& B0, uint32_t dta, uint32_t dtb,
-                 const ReduceSpec& red, const std::vector<uint64_t>& align_bases) {
-  const int esa = dtype_size(dta), esb = dtype_size(dtb);
-  if (A0.nd != B0.nd) return fail(ETHA_ERR_INVALID, "chunk %u: rank mismatch", idx);
-  for (int i = 0; i < A0.nd; i++)
-    if (A0.shape[i] != B0.shape[i]) return fail(ETHA_ERR_INVALID, "chunk %u: shape mismatch in dim %d", idx, i);
-  const bool cvt = dta != dtb;
-  if (cvt && !(is_float(dta) && is_float(dtb)))
-    return fail(ETHA_ERR_UNSUPPORTED, "chunk %u: conversion %u -> %u is only implemented between floating types", idx,
-                dta, dtb);
-  if (red.n_peers && !is_float(dta))
-    return fail(ETHA_ERR_UNSUPPORTED, "chunk %u: Partial reduce needs a floating tensor dtype", idx);
-  if (region_numel(A0) == 0) return ETHA_OK;
+// Compiles one chunk: emits the tiles that move region A (dtype dta) to/from region B (dtype dtb); both
+// regions have the same shape.  For reduce chunks A.base is 0 and tile addresses on the a side are offsets
+// from the peer bases; `align_bases` then lists the peers' real bases for the alignment bookkeeping.
+class PairCompiler {
+ public:
+  PairCompiler(Builder& bld, uint32_t idx, const Region& A, const Region& B, uint32_t dta, uint32_t dtb,
+               const ReduceSpec& red, const std::vector<uint64_t>& align_bases)
+      : bld_(bld), idx_(idx), A_(A), B_(B), dta_(dta), dtb_(dtb), esa_(dtype_size(dta)), esb_(dtype_size(dtb)),
+        red_(red), align_bases_(align_bases), cvt_(dta != dtb), plain_(dta == dtb && red.n_peers == 0),
+        dt_bits_((dta << kMetaDtaShift) | (dtb << kMetaDtbShift)) {}
 
-  // 1. drop size-1 dims, 2. merge dims that are contiguous on both sides
-  int64_t n[ETHA_MAX_NDIM], sa[ETHA_MAX_NDIM], sb[ETHA_MAX_NDIM];
-  int k = 0;
-  for (int i = 0; i < A0.nd; i++) {
-    if (A0.shape[i] == 1) continue;
-    if (k > 0 && sa[k - 1] == A0.shape[i] * A0.stride[i] && sb[k - 1] == A0.shape[i] * B0.stride[i]) {
-      n[k - 1] *= A0.shape[i];
-      sa[k - 1] = A0.stride[i];
-      sb[k - 1] = B0.stride[i];
-    } else {
-      n[k] = A0.shape[i];
-      sa[k] = A0.stride[i];
-      sb[k] = B0.stride[i];
-      k++;
-    }
+  int compile() {
+    if (A_.nd != B_.nd) return fail(ETHA_ERR_INVALID, "chunk %u: rank mismatch", idx_);
+    for (int i = 0; i < A_.nd; i++)
+      if (A_.shape[i] != B_.shape[i]) return fail(ETHA_ERR_INVALID, "chunk %u: shape mismatch in dim %d", idx_, i);
+    if (cvt_ && !(is_float(dta_) && is_float(dtb_)))
+      return fail(ETHA_ERR_UNSUPPORTED, "chunk %u: conversion %u -> %u is only implemented between floating types", idx_,
+                  dta_, dtb_);
+    if (red_.n_peers && !is_float(dta_))
+      return fail(ETHA_ERR_UNSUPPORTED, "chunk %u: Partial reduce needs a floating tensor dtype", idx_);
+    if (region_numel(A_) == 0) return ETHA_OK;
+    collapse_dims();
+    bool done = false;
+    int rc = try_transposing(&done);
+    if (rc != ETHA_OK || done) return rc;
+    collect_alignment();
+    if (!plain_ && (mask_a_ % (uint64_t)esa_ || mask_b_ % (uint64_t)esb_))
+      return fail(ETHA_ERR_INVALID, "chunk %u: element address not aligned to its dtype", idx_);
+    return plain_ ? compile_byte_move() : compile_typed_move();
   }
-  // 3. innermost contiguous run (in elements)
-  uint64_t run_elems = 1;
-  if (k > 0 && sa[k - 1] == esa && sb[k - 1] == esb) {
-    run_elems = (uint64_t)n[k - 1];
-    k--;
-  }
-  // 3b. transposing chunk: no common contiguous dim, but the a side is contiguous along some other dim j
-  //     while the b side is contiguous along the innermost one.  Such chunks go through the LDS-staged
-  //     transposing kernel in blocks of 64 x 64 elements; all other dims are unrolled here.
-  if (run_elems == 1 && !cvt && !red.n_peers && k >= 2 && sb[k - 1] == esb && sa[k - 1] != esa) {
-    int j = -1;
-    for (int i = 0; i < k - 1; i++)
-      if (sa[i] == esa && n[i] >= 8) j = i;
-    if (j >= 0 && n[k - 1] >= 8 && (A0.base % (uint64_t)esa) == 0 && (B0.base % (uint64_t)esb) == 0) {
-      const int kk = k - 1;
-      int64_t pos[ETHA_MAX_NDIM] = {0};
-      uint64_t off_a = 0, off_b = 0;
-      while (true) {
-        for (int64_t j0 = 0; j0 < n[j]; j0 += kTransDim)
-          for (int64_t k0 = 0; k0 < n[kk]; k0 += kTransDim) {
-            TransTile t;
-            memset(&t, 0, sizeof(t));
-            t.a = A0.base + off_a + (uint64_t)(j0 * sa[j]) + (uint64_t)(k0 * sa[kk]);
-            t.b = B0.base + off_b + (uint64_t)(j0 * sb[j]) + (uint64_t)(k0 * sb[kk]);
-            t.a_pitch = sa[kk];
-            t.b_pitch = sb[j];
-            t.nj = (uint32_t)(n[j] - j0 < kTransDim ? n[j] - j0 : kTransDim);
-            t.nk = (uint32_t)(n[kk] - k0 < kTransDim ? n[kk] - k0 : kTransDim);
-            t.es_log2 = (uint32_t)log2u((uint64_t)esa);
-            bld.trans.push_back(t);
-          }
-        if (bld.trans.size() > kMaxTiles)
-          return fail(ETHA_ERR_UNSUPPORTED, "tile program too large (> %llu tiles)", (unsigned long long)kMaxTiles);
-        int d = k - 1;
-        for (; d >= 0; d--) {
-          if (d == j || d == kk) continue;
-          pos[d]++;
-          off_a += (uint64_t)sa[d];
-          off_b += (uint64_t)sb[d];
-          if (pos[d] < n[d]) break;
-          off_a -= (uint64_t)(sa[d] * n[d]);
-          off_b -= (uint64_t)(sb[d] * n[d]);
-          pos[d] = 0;
-        }
-        if (d < 0) break;
+
+ private:
+  // 1. drop size-1 dims, 2. merge dims that are contiguous on both sides, 3. split off the innermost
+  //    contiguous run (in elements).  Afterwards dims [0, k_) are the outer dims, strides in bytes.
+  void collapse_dims() {
+    k_ = 0;
+    for (int i = 0; i < A_.nd; i++) {
+      if (A_.shape[i] == 1) continue;
+      if (k_ > 0 && sa_[k_ - 1] == A_.shape[i] * A_.stride[i] && sb_[k_ - 1] == A_.shape[i] * B_.stride[i]) {
+        n_[k_ - 1] *= A_.shape[i];
+        sa_[k_ - 1] = A_.stride[i];
+        sb_[k_ - 1] = B_.stride[i];
+      } else {
+        n_[k_] = A_.shape[i];
+        sa_[k_] = A_.stride[i];
+        sb_[k_] = B_.stride[i];
+        k_++;
       }
-      return ETHA_OK;
+    }
+    run_elems_ = 1;
+    if (k_ > 0 && sa_[k_ - 1] == esa_ && sb_[k_ - 1] == esb_) {
+      run_elems_ = (uint64_t)n_[k_ - 1];
+      k_--;
     }
   }
 
-  // 4. unit size.  Lengths decide it, not addresses: the kernel's accesses are legal at any (element-aligned)
-  //    address, so a misaligned side only sets a meta flag.  Byte moves use the widest power of two (<= 16
-  //    bytes) that divides the run; converting and reducing moves use whole vectors of 16 / max(element
-  //    size) elements when the run is a multiple of that, else single elements.  Runs that are not a whole
-  //    number of wide units are split further down into a wide body and a narrow remainder.
-  int ua_log2, ub_log2;
-  uint64_t run_units;
-  uint32_t meta = 0;
-  uint64_t mask_a = 0, mask_b = 0;  // OR of every row start (base and outer strides) per side
-  const bool plain = !cvt && !red.n_peers;
-  // elements per full vector: converting moves may use two accesses on the wide side, reductions one
-  const int epv_full = red.n_peers ? 16 / (esa > esb ? esa : esb) : cvt_elems_per_unit(esa, esb);
-  {
-    mask_a = red.n_peers ? 0 : A0.base;
-    mask_b = B0.base;
-    for (uint64_t p : align_bases) mask_a |= p + A0.base;  // reduce: A0.base is an offset from each peer base
-    for (int i = 0; i < k; i++) {
-      mask_a |= (uint64_t)(sa[i] < 0 ? -sa[i] : sa[i]);
-      mask_b |= (uint64_t)(sb[i] < 0 ? -sb[i] : sb[i]);
+  // Odometer over dims [0, dims) except `skip0` / `skip1`: advances pos and the two byte offsets; false at the end.
+  bool next_position(int dims, int64_t* pos, uint64_t* off_a, uint64_t* off_b, int skip0 = -1, int skip1 = -1) const {
+    for (int d = dims - 1; d >= 0; d--) {
+      if (d == skip0 || d == skip1) continue;
+      pos[d]++;
+      *off_a += (uint64_t)sa_[d];  // wraps mod 2^64 for negative strides, which is fine
+      *off_b += (uint64_t)sb_[d];
+      if (pos[d] < n_[d]) return true;
+      *off_a -= (uint64_t)(sa_[d] * n_[d]);
+      *off_b -= (uint64_t)(sb_[d] * n_[d]);
+      pos[d] = 0;
     }
-    if (plain) {
-      const uint64_t run_bytes = run_elems * (uint64_t)esa;
-      int v = 4;
-      while (v > 0 && (run_bytes & ((1ull << v) - 1))) v--;
-      ua_log2 = ub_log2 = v;
-      run_units = run_bytes >> v;
-    } else {
-      if (mask_a % (uint64_t)esa || mask_b % (uint64_t)esb)
-        return fail(ETHA_ERR_INVALID, "chunk %u: element address not aligned to its dtype", idx);
-      const int epv = run_elems % (uint64_t)epv_full == 0 ? epv_full : 1;
-      ua_log2 = log2u((uint64_t)(epv * esa));
-      ub_log2 = log2u((uint64_t)(epv * esb));
-      run_units = run_elems / (uint64_t)epv;
-      meta |= kMetaCvt;
-      if (epv > 1) meta |= kMetaVec;
+    return false;
+  }
+
+  int check_size() const {
+    if (bld_.run.size() + bld_.row.size() > kMaxTiles || bld_.trans.size() > kMaxTiles)
+      return fail(ETHA_ERR_UNSUPPORTED, "tile program too large (> %llu tiles)", (unsigned long long)kMaxTiles);
+    return ETHA_OK;
+  }
+
+  // Transposing chunk: no common contiguous dim, but the a side is contiguous along some other dim j while
+  // the b side is contiguous along the innermost one.  Such chunks go through the LDS-staged transposing
+  // kernel in blocks of 64 x 64 elements; all other dims are unrolled here.
+  int try_transposing(bool* done) {
+    *done = false;
+    if (!(run_elems_ == 1 && plain_ && k_ >= 2 && sb_[k_ - 1] == esb_ && sa_[k_ - 1] != esa_)) return ETHA_OK;
+    int j = -1;
+    for (int i = 0; i < k_ - 1; i++)
+      if (sa_[i] == esa_ && n_[i] >= 8) j = i;
+    const int kk = k_ - 1;
+    if (j < 0 || n_[kk] < 8 || (A_.base % (uint64_t)esa_) != 0 || (B_.base % (uint64_t)esb_) != 0) return ETHA_OK;
+    int64_t pos[ETHA_MAX_NDIM] = {0};
+    uint64_t off_a = 0, off_b = 0;
+    do {
+      for (int64_t j0 = 0; j0 < n_[j]; j0 += kTransDim)
+        for (int64_t k0 = 0; k0 < n_[kk]; k0 += kTransDim) {
+          TransTile t;
+          memset(&t, 0, sizeof(t));
+          t.a = A_.base + off_a + (uint64_t)(j0 * sa_[j]) + (uint64_t)(k0 * sa_[kk]);
+          t.b = B_.base + off_b + (uint64_t)(j0 * sb_[j]) + (uint64_t)(k0 * sb_[kk]);
+          t.a_pitch = sa_[kk];
+          t.b_pitch = sb_[j];
+          t.nj = (uint32_t)(n_[j] - j0 < kTransDim ? n_[j] - j0 : kTransDim);
+          t.nk = (uint32_t)(n_[kk] - k0 < kTransDim ? n_[kk] - k0 : kTransDim);
+          t.es_log2 = (uint32_t)log2u((uint64_t)esa_);
+          bld_.trans.push_back(t);
+        }
+      const int rc = check_size();
+      if (rc != ETHA_OK) return rc;
+    } while (next_position(k_, pos, &off_a, &off_b, j, kk));
+    *done = true;
+    return ETHA_OK;
+  }
+
+  // OR of every row start (base and outer strides) per side.  Lengths decide unit sizes, not addresses: the
+  // kernel's accesses are legal at any (element-aligned) address, so a misaligned side only sets a meta flag.
+  void collect_alignment() {
+    mask_a_ = red_.n_peers ? 0 : A_.base;
+    mask_b_ = B_.base;
+    for (uint64_t p : align_bases_) mask_a_ |= p + A_.base;  // reduce: A_.base is an offset from each peer base
+    for (int i = 0; i < k_; i++) {
+      mask_a_ |= (uint64_t)(sa_[i] < 0 ? -sa_[i] : sa_[i]);
+      mask_b_ |= (uint64_t)(sb_[i] < 0 ? -sb_[i] : sb_[i]);
     }
   }
-  const uint32_t dt_bits = (dta << kMetaDtaShift) | (dtb << kMetaDtbShift);
-  auto skew_bits = [&](int ua_l2, int ub_l2) -> uint32_t {
-    return ((mask_a & ((1ull << ua_l2) - 1)) ? kMetaSkew : 0u) | ((mask_b & ((1ull << ub_l2) - 1)) ? kMetaSkewB : 0u);
-  };
-  meta |= ((uint32_t)ua_log2 << kMetaUaShift) | ((uint32_t)ub_log2 << kMetaUbShift) | dt_bits | skew_bits(ua_log2, ub_log2);
-  const uint64_t ua = 1ull << ua_log2, ub = 1ull << ub_log2;
+  uint32_t skew_bits(int ua_log2, int ub_log2) const {
+    return ((mask_a_ & ((1ull << ua_log2) - 1)) ? kMetaSkew : 0u) | ((mask_b_ & ((1ull << ub_log2) - 1)) ? kMetaSkewB : 0u);
+  }
+  static uint32_t unit_bits(int ua_log2, int ub_log2) {
+    return ((uint32_t)ua_log2 << kMetaUaShift) | ((uint32_t)ub_log2 << kMetaUbShift);
+  }
+  static int widest_unit_log2(uint64_t bytes, int cap_log2) {  // widest power of two (<= 2^cap) dividing `bytes`
+    int v = cap_log2;
+    while (v > 0 && (bytes & ((1ull << v) - 1))) v--;
+    return v;
+  }
 
-  // Skewed byte moves: the two sides disagree on their position inside a 16-byte vector (typically
-  // a chunk that follows an odd-sized one in an un-padded bucket).  Very long runs are peeled per run so
-  // that the b side is 16-byte aligned: a head and a tail of < 16 bytes go through narrow tiles, the
-  // body moves in 16-byte units whose a-side access is unaligned.  Peeling costs three tile sets per
-  // run, so it only pays for runs of many tiles (measured: +5 % from 256 KiB up, 20x slower than the
-  // row split below at 512-byte runs); shorter runs take the row split, unaligned on both sides.
-  constexpr uint64_t kSkewMinRunBytes = ETHA_SKEW_PEEL_MIN_BYTES;
-  if (plain && ((mask_a | mask_b) & 15) && run_elems * (uint64_t)esa >= kSkewMinRunBytes) {
-    const uint64_t run_bytes = run_elems * (uint64_t)esa;
-    const uint32_t body_meta = dt_bits | (4u << kMetaUaShift) | (4u << kMetaUbShift) | kMetaSkew;
+  // Byte moves (same dtype, no reduce): the widest power of two <= 16 bytes that divides the run.
+  int compile_byte_move() {
+    const uint64_t run_bytes = run_elems_ * (uint64_t)esa_;
+    // Skewed byte moves: the two sides disagree on their position inside a 16-byte vector (typically a chunk
+    // that follows an odd-sized one in an un-padded bucket).  Very long runs are peeled per run so that the
+    // b side is 16-byte aligned: a head and a tail of < 16 bytes go through narrow tiles, the body moves in
+    // 16-byte units whose a-side access is unaligned.  Peeling costs three tile sets per run, so it only
+    // pays for runs of many tiles (measured: +5 % from 256 KiB up, 20x slower than the row split below at
+    // 512-byte runs); shorter runs take the row split, unaligned on both sides.
+    if (((mask_a_ | mask_b_) & 15) && run_bytes >= (uint64_t)ETHA_SKEW_PEEL_MIN_BYTES) return peel_runs(run_bytes);
+    const int v = widest_unit_log2(run_bytes, 4);
+    if (v == 4 || run_bytes < 32)
+      return emit(A_.base, B_.base, run_bytes >> v, 1ull << v, 1ull << v, dt_bits_ | unit_bits(v, v) | skew_bits(v, v));
+    // Rows that are not a whole number of 16-byte units: a body of 16-byte units and a remainder of < 16
+    // bytes in narrow units, both ordinary, densely packed tile sets over the same rows.
+    const uint64_t body_units = run_bytes / 16, rem_bytes = run_bytes % 16;
+    int rc = emit(A_.base, B_.base, body_units, 16, 16, dt_bits_ | unit_bits(4, 4) | skew_bits(4, 4));
+    if (rc != ETHA_OK) return rc;
+    const int r = widest_unit_log2(rem_bytes, 3);
+    // the remainder starts body_units * 16 bytes into each row: same position modulo 16 as the row start
+    return emit(A_.base + body_units * 16, B_.base + body_units * 16, rem_bytes >> r, 1ull << r, 1ull << r,
+                dt_bits_ | unit_bits(r, r) | skew_bits(r, r));
+  }
+
+  int peel_runs(uint64_t run_bytes) {
+    const uint32_t body_meta = dt_bits_ | unit_bits(4, 4) | kMetaSkew;
     auto narrow = [&](uint64_t a, uint64_t b, uint64_t bytes) {  // bytes < 16
       if (!bytes) return;
-      int v = 3;
-      while (v > 0 && (bytes & ((1ull << v) - 1))) v--;
+      const int v = widest_unit_log2(bytes, 3);
       const uint64_t low = (1ull << v) - 1;
       RunTile t;
       t.a = a;
       t.b = b;
       t.n = (uint32_t)(bytes >> v);
-      t.meta = dt_bits | ((uint32_t)v << kMetaUaShift) | ((uint32_t)v << kMetaUbShift) | ((a & low) ? kMetaSkew : 0u) |
-               ((b & low) ? kMetaSkewB : 0u);
-      bld.run.push_back(t);
+      t.meta = dt_bits_ | unit_bits(v, v) | ((a & low) ? kMetaSkew : 0u) | ((b & low) ? kMetaSkewB : 0u);
+      bld_.run.push_back(t);
     };
     int64_t pos[ETHA_MAX_NDIM] = {0};
     uint64_t off_a = 0, off_b = 0;
-    while (true) {
-      const uint64_t a0 = A0.base + off_a, b0 = B0.base + off_b;
+    do {
+      const uint64_t a0 = A_.base + off_a, b0 = B_.base + off_b;
       const uint64_t head = (16 - (b0 & 15)) & 15;
       const uint64_t body_units = (run_bytes - head) / 16;
       const uint64_t tail = run_bytes - head - body_units * 16;
@@ -748,123 +769,114 @@ int compile_pair(Builder& bld, uint32_t idx, const Region& A0, const Region& B0,
         t.b = b0 + head + q * 16;
         t.n = (uint32_t)(body_units - q < kTileThreads ? body_units - q : kTileThreads);
         t.meta = body_meta;
-        bld.run.push_back(t);
+        bld_.run.push_back(t);
       }
       narrow(a0 + head + body_units * 16, b0 + head + body_units * 16, tail);
-      if (bld.run.size() + bld.row.size() > kMaxTiles)
-        return fail(ETHA_ERR_UNSUPPORTED, "tile program too large (> %llu tiles)", (unsigned long long)kMaxTiles);
-      int d = k - 1;
-      for (; d >= 0; d--) {
-        pos[d]++;
-        off_a += (uint64_t)sa[d];
-        off_b += (uint64_t)sb[d];
-        if (pos[d] < n[d]) break;
-        off_a -= (uint64_t)(sa[d] * n[d]);
-        off_b -= (uint64_t)(sb[d] * n[d]);
-        pos[d] = 0;
-      }
-      if (d < 0) break;
-    }
+      const int rc = check_size();
+      if (rc != ETHA_OK) return rc;
+    } while (next_position(k_, pos, &off_a, &off_b));
     return ETHA_OK;
   }
 
-  // 5. tiles.  Long or tile-multiple rows (and single runs) become run tiles; other shapes become
-  //    row tiles over the innermost remaining dim; dims further out are unrolled here.
-  auto emit = [&](uint64_t base_a, uint64_t base_b, uint64_t run_units, uint64_t ua, uint64_t ub, uint32_t meta) -> int {
-  const bool use_rows = red.n_peers != 0 || (k > 0 && run_units % kTileThreads != 0 && run_units < 4 * kTileThreads);
-  if (run_units > 0xffffffffull && use_rows && k > 0)
-    return fail(ETHA_ERR_UNSUPPORTED, "chunk %u: row longer than 2^32 units", idx);
-  const int outer = use_rows && k > 0 ? k - 1 : k;  // dims unrolled on the host
-  int64_t pos[ETHA_MAX_NDIM] = {0};
-  uint64_t off_a = 0, off_b = 0;  // wraps mod 2^64 for negative strides, which is fine
-  while (true) {
-    const uint64_t a0 = base_a + off_a, b0 = base_b + off_b;
-    if (!use_rows) {
-      for (uint64_t q = 0; q < run_units; q += kTileThreads) {
-        RunTile t;
-        t.a = a0 + q * ua;
-        t.b = b0 + q * ub;
-        t.n = (uint32_t)(run_units - q < kTileThreads ? run_units - q : kTileThreads);
-        t.meta = meta;
-        bld.run.push_back(t);
-      }
-    } else {
-      const uint64_t rows = k > 0 ? (uint64_t)n[k - 1] : 1;
-      const int64_t pa = k > 0 ? sa[k - 1] : 0, pb = k > 0 ? sb[k - 1] : 0;
-      const uint64_t total = rows * run_units;
-      for (uint64_t q = 0; q < total; q += kTileThreads) {
-        RowTile t;
-        memset(&t, 0, sizeof(t));
-        const uint64_t left = total - q;
-        t.n = (uint32_t)(left < kTileThreads ? left : kTileThreads);
-        t.meta = meta;
-        if (rows == 1) {  // one (possibly very long) run: address the tile directly
+  // Converting and reducing moves: whole vectors of `epv` elements (the narrow side moves up to 16 bytes;
+  // converting moves may use two accesses on the wide side, reductions one) when the run is a multiple of
+  // that; else a body of whole vectors plus a remainder of single elements; short runs single elements.
+  int compile_typed_move() {
+    const int epv = red_.n_peers ? 16 / (esa_ > esb_ ? esa_ : esb_) : cvt_elems_per_unit(esa_, esb_);
+    const int ea = log2u((uint64_t)esa_), eb = log2u((uint64_t)esb_);
+    const int va = log2u((uint64_t)(epv * esa_)), vb = log2u((uint64_t)(epv * esb_));
+    const uint32_t vec_meta = dt_bits_ | kMetaCvt | kMetaVec | unit_bits(va, vb) | skew_bits(va, vb);
+    // element units are always aligned (checked by the caller), so they carry no skew flags
+    const uint32_t elem_meta = dt_bits_ | kMetaCvt | unit_bits(ea, eb);
+    if (epv > 1 && run_elems_ % (uint64_t)epv == 0)
+      return emit(A_.base, B_.base, run_elems_ / (uint64_t)epv, 1ull << va, 1ull << vb, vec_meta);
+    if (epv > 1 && run_elems_ >= 2 * (uint64_t)epv) {
+      const uint64_t body_units = run_elems_ / (uint64_t)epv, rem_elems = run_elems_ % (uint64_t)epv;
+      const int rc = emit(A_.base, B_.base, body_units, 1ull << va, 1ull << vb, vec_meta);
+      if (rc != ETHA_OK) return rc;
+      return emit(A_.base + body_units * (uint64_t)(epv * esa_), B_.base + body_units * (uint64_t)(epv * esb_), rem_elems,
+                  (uint64_t)esa_, (uint64_t)esb_, elem_meta);
+    }
+    return emit(A_.base, B_.base, run_elems_, (uint64_t)esa_, (uint64_t)esb_, elem_meta);
+  }
+
+  // Tiles for rows of `run_units` units starting at base_a / base_b.  Long or tile-multiple rows (and
+  // single runs) become run tiles; other shapes become row tiles over the innermost remaining dim; dims
+  // further out are unrolled here.  Reduce chunks always use row tiles (they carry the peer list).
+  int emit(uint64_t base_a, uint64_t base_b, uint64_t run_units, uint64_t ua, uint64_t ub, uint32_t meta) {
+    const bool use_rows = red_.n_peers != 0 || (k_ > 0 && run_units % kTileThreads != 0 && run_units < 4 * kTileThreads);
+    if (run_units > 0xffffffffull && use_rows && k_ > 0)
+      return fail(ETHA_ERR_UNSUPPORTED, "chunk %u: row longer than 2^32 units", idx_);
+    const int outer = use_rows && k_ > 0 ? k_ - 1 : k_;  // dims unrolled on the host
+    int64_t pos[ETHA_MAX_NDIM] = {0};
+    uint64_t off_a = 0, off_b = 0;
+    do {
+      const uint64_t a0 = base_a + off_a, b0 = base_b + off_b;
+      if (!use_rows) {
+        for (uint64_t q = 0; q < run_units; q += kTileThreads) {
+          RunTile t;
           t.a = a0 + q * ua;
           t.b = b0 + q * ub;
-          t.run = kTileThreads;
-          t.c0 = 0;
-        } else {
-          const uint64_t r0 = q / run_units, c0 = q % run_units;
-          t.a = a0 + (uint64_t)((int64_t)r0 * pa);
-          t.b = b0 + (uint64_t)((int64_t)r0 * pb);
-          t.a_pitch = pa;
-          t.b_pitch = pb;
-          t.run = (uint32_t)run_units;
-          t.c0 = (uint32_t)c0;
+          t.n = (uint32_t)(run_units - q < kTileThreads ? run_units - q : kTileThreads);
+          t.meta = meta;
+          bld_.run.push_back(t);
         }
-        t.peer_first = red.peer_first;
-        t.n_peers = red.n_peers;
-        t.reduce_op = red.op;
-        t.via = red.via;
-        bld.row.push_back(t);
+      } else {
+        const uint64_t rows = k_ > 0 ? (uint64_t)n_[k_ - 1] : 1;
+        const int64_t pa = k_ > 0 ? sa_[k_ - 1] : 0, pb = k_ > 0 ? sb_[k_ - 1] : 0;
+        const uint64_t total = rows * run_units;
+        for (uint64_t q = 0; q < total; q += kTileThreads) {
+          RowTile t;
+          memset(&t, 0, sizeof(t));
+          const uint64_t left = total - q;
+          t.n = (uint32_t)(left < kTileThreads ? left : kTileThreads);
+          t.meta = meta;
+          if (rows == 1) {  // one (possibly very long) run: address the tile directly
+            t.a = a0 + q * ua;
+            t.b = b0 + q * ub;
+            t.run = kTileThreads;
+            t.c0 = 0;
+          } else {
+            const uint64_t r0 = q / run_units, c0 = q % run_units;
+            t.a = a0 + (uint64_t)((int64_t)r0 * pa);
+            t.b = b0 + (uint64_t)((int64_t)r0 * pb);
+            t.a_pitch = pa;
+            t.b_pitch = pb;
+            t.run = (uint32_t)run_units;
+            t.c0 = (uint32_t)c0;
+          }
+          t.peer_first = red_.peer_first;
+          t.n_peers = red_.n_peers;
+          t.reduce_op = red_.op;
+          t.via = red_.via;
+          bld_.row.push_back(t);
+        }
       }
-    }
-    if (bld.run.size() + bld.row.size() > kMaxTiles)
-      return fail(ETHA_ERR_UNSUPPORTED, "tile program too large (> %llu tiles)", (unsigned long long)kMaxTiles);
-    int d = outer - 1;
-    for (; d >= 0; d--) {
-      pos[d]++;
-      off_a += (uint64_t)sa[d];
-      off_b += (uint64_t)sb[d];
-      if (pos[d] < n[d]) break;
-      off_a -= (uint64_t)(sa[d] * n[d]);
-      off_b -= (uint64_t)(sb[d] * n[d]);
-      pos[d] = 0;
-    }
-    if (d < 0) break;
+      const int rc = check_size();
+      if (rc != ETHA_OK) return rc;
+    } while (next_position(outer, pos, &off_a, &off_b));
+    return ETHA_OK;
   }
-  return ETHA_OK;
-  };  // emit
 
-  // Runs that are not a whole number of wide units: every row is split into a body of wide units (16 bytes
-  // for byte moves, a full vector for converting and reducing moves) and a narrow remainder.  Both parts
-  // are ordinary, densely packed tile sets over the same rows.
-  if (plain && ua_log2 < 4 && run_elems * (uint64_t)esa >= 32) {
-    const uint64_t run_bytes = run_elems * (uint64_t)esa;
-    const uint64_t body_units = run_bytes / 16, rem_bytes = run_bytes % 16;
-    const uint32_t body_meta = dt_bits | (4u << kMetaUaShift) | (4u << kMetaUbShift) | skew_bits(4, 4);
-    int rc = emit(A0.base, B0.base, body_units, 16, 16, body_meta);
-    if (rc != ETHA_OK) return rc;
-    int v = 3;
-    while (v > 0 && (rem_bytes & ((1ull << v) - 1))) v--;
-    // the remainder starts body_units * 16 bytes into each row: same position modulo 16 as the row start
-    const uint32_t rem_meta = dt_bits | ((uint32_t)v << kMetaUaShift) | ((uint32_t)v << kMetaUbShift) | skew_bits(v, v);
-    return emit(A0.base + body_units * 16, B0.base + body_units * 16, rem_bytes >> v, 1ull << v, 1ull << v, rem_meta);
-  }
-  if (!plain && !(meta & kMetaVec) && epv_full > 1 && run_elems >= 2 * (uint64_t)epv_full) {
-    const uint64_t body_units = run_elems / (uint64_t)epv_full, rem_elems = run_elems % (uint64_t)epv_full;
-    const int va = log2u((uint64_t)(epv_full * esa)), vb = log2u((uint64_t)(epv_full * esb));
-    const uint32_t body_meta = dt_bits | kMetaCvt | kMetaVec | ((uint32_t)va << kMetaUaShift) | ((uint32_t)vb << kMetaUbShift) |
-                               skew_bits(va, vb);
-    int rc = emit(A0.base, B0.base, body_units, 1ull << va, 1ull << vb, body_meta);
-    if (rc != ETHA_OK) return rc;
-    // element units are always aligned (checked above), so the remainder carries no skew flags
-    const uint32_t rem_meta = dt_bits | kMetaCvt | ((uint32_t)log2u((uint64_t)esa) << kMetaUaShift) |
-                              ((uint32_t)log2u((uint64_t)esb) << kMetaUbShift);
-    return emit(A0.base + body_units * (uint64_t)(epv_full * esa), B0.base + body_units * (uint64_t)(epv_full * esb),
-                rem_elems, (uint64_t)esa, (uint64_t)esb, rem_meta);
-  }
-  return emit(A0.base, B0.base, run_units, ua, ub, meta);
+  Builder& bld_;
+  const uint32_t idx_;
+  const Region& A_;
+  const Region& B_;
+  const uint32_t dta_, dtb_;
+  const int esa_, esb_;
+  const ReduceSpec& red_;
+  const std::vector<uint64_t>& align_bases_;
+  const bool cvt_, plain_;
+  const uint32_t dt_bits_;
+  int k_ = 0;                                              // outer dims left after collapsing
+  int64_t n_[ETHA_MAX_NDIM], sa_[ETHA_MAX_NDIM], sb_[ETHA_MAX_NDIM];  // their extents and byte strides
+  uint64_t run_elems_ = 1;                                 // innermost contiguous run, in elements
+  uint64_t mask_a_ = 0, mask_b_ = 0;
+};
+
+int compile_pair(Builder& bld, uint32_t idx, const Region& A, const Region& B, uint32_t dta, uint32_t dtb,
+                 const ReduceSpec& red, const std::vector<uint64_t>& align_bases) {
+  return PairCompiler(bld, idx, A, B, dta, dtb, red, align_bases).compile();
 }
 
 }  // namespace
