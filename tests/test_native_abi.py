@@ -116,3 +116,24 @@ def test_ipc_entry_points_reject_bad_arguments_without_a_gpu():
         nat.ipc_close(0x1234)
     nat.ipc_close(0)  # null is a no-op
     assert nat.lib().etha_arena_create(0, ctypes.byref(out)) == nat.ERR_INVALID
+
+
+def test_missing_library_fails_loudly(tmp_path):
+    """No fallback: with the library absent, the first use of the product raises and names the build step."""
+    import subprocess
+    import sys
+
+    root = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+    code = (
+        "import torch\n"
+        "from torch.distributed.tensor.placement_types import Shard\n"
+        "from etha_amd.world import ReshardJob, TensorSpec\n"
+        "from etha_amd.comm import LoopbackWire\n"
+        "spec = TensorSpec('w', (8, 8), [0, 1], (Shard(0),), [2], (Shard(1),), torch.float32)\n"
+        "job = ReshardJob([spec], device='cpu', wire=LoopbackWire('cpu', host_inspection=True))\n"
+        "job.wire.plan(job.send_buckets[0])\n"
+    )
+    env = dict(os.environ, ETHA_AMD_LIB=str(tmp_path / "absent.so"), PYTHONPATH=root)
+    proc = subprocess.run([sys.executable, "-c", code], capture_output=True, text=True, env=env, timeout=120)
+    assert proc.returncode != 0
+    assert "is missing: the HIP extension is not built" in proc.stderr and "no CPU fallback" in proc.stderr
