@@ -164,6 +164,7 @@ class TensorBusAgent:
 
     def start_in_thread(self) -> threading.Thread:
         t = threading.Thread(target=self.run, daemon=True, name="etha-agent")
+        self._serve_thread = t
         t.start()
         return t
 
@@ -231,6 +232,9 @@ class TensorBusAgent:
 
     def close(self) -> None:
         self._stop.set()
+        serving = getattr(self, "_serve_thread", None)
+        if serving is not None and serving is not threading.current_thread():
+            serving.join(timeout=5.0)  # let the current sweep finish before its plans are released
         for q in self._queues.values():
             q.close()
         for b in list(self.batches.values()):
