@@ -780,7 +780,8 @@ class PairCompiler {
 
   // Converting and reducing moves: whole vectors of `epv` elements (the narrow side moves up to 16 bytes;
   // converting moves may use two accesses on the wide side, reductions one) when the run is a multiple of
-  // that; else a body of whole vectors plus a remainder of single elements; short runs single elements.
+  // that; else a body of whole vectors plus a remainder of single elements; runs shorter than one vector
+  // single elements.
   int compile_typed_move() {
     const int epv = red_.n_peers ? 16 / (esa_ > esb_ ? esa_ : esb_) : cvt_elems_per_unit(esa_, esb_);
     const int ea = log2u((uint64_t)esa_), eb = log2u((uint64_t)esb_);
@@ -790,7 +791,7 @@ class PairCompiler {
     const uint32_t elem_meta = dt_bits_ | kMetaCvt | unit_bits(ea, eb);
     if (epv > 1 && run_elems_ % (uint64_t)epv == 0)
       return emit(A_.base, B_.base, run_elems_ / (uint64_t)epv, 1ull << va, 1ull << vb, vec_meta);
-    if (epv > 1 && run_elems_ >= 2 * (uint64_t)epv) {
+    if (epv > 1 && run_elems_ > (uint64_t)epv) {
       const uint64_t body_units = run_elems_ / (uint64_t)epv, rem_elems = run_elems_ % (uint64_t)epv;
       const int rc = emit(A_.base, B_.base, body_units, 1ull << va, 1ull << vb, vec_meta);
       if (rc != ETHA_OK) return rc;
