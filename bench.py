@@ -46,6 +46,9 @@ def parse_args():
                          "not the pack+unpack path the headline is quoted on)")
     ap.add_argument("--graph", action="store_true", help="replay the step from a captured HIP graph (whole step timed)")
     ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--no-per-bucket-leg", action="store_true",
+                    help="skip the extra one-launch-per-bucket measurement after the timed region (use under a "
+                         "profiler, so that per-kernel statistics cover the timed configuration only)")
     ap.add_argument("--cpu-layers", type=int, default=8, help="layers of the workload the CPU baseline sample covers")
     ap.add_argument("--cpu-seconds", type=float, default=15.0, help="CPU work the baseline leg is bounded to")
     ap.add_argument("--calibration-copy", action="store_true",
@@ -306,6 +309,25 @@ def main():
         },
         "setup_s": round(setup_s, 1),
     }
+    if merge and graph is None and args.fanout == 1 and not args.no_per_bucket_leg:
+        # the strict form of the same step, one launch per bucket, for comparison (not the headline)
+        n_strict = sum(1 for p in send_plans + recv_plans for s in p.steps if s[0] != "lend")
+        for _ in range(2):
+            job.run(merge_launches=False)
+        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        reps = max(3, min(args.steps, 10))
+        e0.record(stream)
+        for _ in range(reps):
+            job.run(merge_launches=False, synchronize=False)
+        e1.record(stream)
+        torch.cuda.synchronize()
+        strict_ms = e0.elapsed_time(e1) / reps
+        out["one_launch_per_bucket"] = {
+            "device_ms_per_step": round(strict_ms, 4),
+            "pct_of_hbm_peak": round(100.0 * (pack_bytes + unpack_bytes) / (strict_ms * 1e-3) / 1e9 / HBM_PEAK_GBS, 2),
+            "launches_per_step": n_strict,
+            "effective_GB/s": round(S / (strict_ms * 1e-3) / 1e9, 1),
+        }
     if args.calibration_copy:
         a = torch.empty(1 << 30, dtype=torch.uint8, device=dev).fill_(1)
         b = torch.empty(1 << 30, dtype=torch.uint8, device=dev)
