@@ -111,7 +111,7 @@ class TensorBusAgent:
         self._last_heartbeat = 0.0
         self._last_core: dict | None = None
         self._moved = False  # set by a command that changed shared state without completing
-        self._unsynced: list[tuple[dict, float]] = []  # (result dict, start time) of transfers enqueued but not synchronised
+        self._unsynced: list[tuple[dict, float, str]] = []  # (result, start time, label) of transfers enqueued, not yet synchronised
         self.stats = {"ipc_tensors": 0, "in_process_tensors": 0, "transfers": 0}
         for rank in range(world_size):
             cmd_path, state_path = self.path_naming_fn(rank)
@@ -209,8 +209,9 @@ class TensorBusAgent:
             if self.device.type == "cuda":
                 torch.cuda.current_stream(self.device).synchronize()
             now = time.perf_counter()
-            for result, t0 in self._unsynced:
+            for result, t0, label in self._unsynced:
                 result["ms"] = (now - t0) * 1e3
+                logger.info("%s: %.3f ms (enqueue to device completion)", label, result["ms"])
             self._unsynced.clear()
         if finished:
             # the state file must show the new state before a worker is released
@@ -421,7 +422,7 @@ class TensorBusAgent:
                     return False, None  # the previous generation has not been consumed yet
             batch.transfer_signal = True
             result = {"ms": 0.0}
-            self._unsynced.append((result, time.perf_counter()))
+            self._unsynced.append((result, time.perf_counter(), f"batch {cmd.batch_id} rank {rank} send #{gen}"))
             bucket_comm(buckets, wire=self.wire, merge_launches=True, synchronize=False)
             batch.send_count[rank] = gen + 1
             for d in self._peers(buckets, "dst"):
@@ -438,7 +439,7 @@ class TensorBusAgent:
                 if batch.send_count.get(s, 0) <= gen:
                     return False, None  # wait for the source's send of this generation
             result = {"ms": 0.0}
-            self._unsynced.append((result, time.perf_counter()))
+            self._unsynced.append((result, time.perf_counter(), f"batch {cmd.batch_id} rank {rank} recv #{gen}"))
             bucket_comm(buckets, wire=self.wire, merge_launches=True, synchronize=False)
             batch.recv_count[rank] = gen + 1
             if all(batch.recv_count.get(d, 0) >= n for d, n in batch.owed.items()):
