@@ -722,3 +722,26 @@ def test_direct_table_launch_refuses_mixed_ranges(gpu_device):
     total = sum(s[2] for s in plan.steps)
     with pytest.raises(EthaNativeError, match="mixes Partial and plain"):
         plan.local_table.selfcopy(0, total)
+
+
+def test_large_resident_set_70b_shapes(gpu_device):
+    """Llama-3-70B shapes, 40 layers: 70 GB of source shards resident, a 36 GB share through 37 pool segments.
+    Every checked target shard equals its slice of the reassembled source (sizes well past 32-bit offsets)."""
+    free, _ = torch.cuda.mem_get_info(gpu_device)
+    if free < 180 << 30:
+        pytest.skip("needs about 150 GB of free device memory")
+    specs, targets, bucket = workloads.llama3_8b_fsdp8_to_tp2(n_layers=40, hidden=8192, inter=28672, kv=1024, vocab=128256)
+    job = ReshardJob(specs, device=gpu_device, bucket_size=bucket, target_ranks=targets)
+    assert job.payload_bytes() == 36_328_177_664
+    job.run(merge_launches=True)
+    from oracle.dtensor_layout import local_shard
+
+    for i, spec in enumerate(specs):
+        if i % 9 not in (0, 5) and i != len(specs) - 1:  # embeddings, o_proj / down_proj of every layer, lm_head
+            continue
+        glob = torch.cat([job.source_locals[i][r] for r in range(8)], dim=0)
+        want = local_shard(glob, (2,), spec.target_placements, (0,))
+        assert torch.equal(job.target_locals[i][8].view(torch.int16), want.contiguous().view(torch.int16)), spec.name
+        del glob, want
+    del job
+    torch.cuda.empty_cache()  # hand the 150 GB back before the multi-process tests start
