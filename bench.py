@@ -151,8 +151,10 @@ def main():
     import torch
 
     from etha_amd import _native, workloads
+    from etha_amd.build import ensure_built
     from etha_amd.world import ReshardJob
 
+    ensure_built()  # loads what is built; compiles only if nothing is
     _native.lib()
     if not torch.cuda.is_available():
         print("bench.py needs a GPU: the hot path has no CPU fallback", file=sys.stderr)

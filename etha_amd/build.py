@@ -49,5 +49,11 @@ def build_library(verbose: bool = False, defines: tuple[str, ...] = (), out_path
     return out_path
 
 
+def ensure_built() -> str:
+    """Build the library only if none is there (test / benchmark harnesses; the product itself never builds:
+    ``etha_amd._native.lib()`` raises when the library is missing)."""
+    return LIB_PATH if os.path.exists(LIB_PATH) else build_library()
+
+
 if __name__ == "__main__":
     print(build_library(verbose=True))

@@ -12,6 +12,13 @@ def pytest_configure(config):
     config.addinivalue_line("markers", "gpu: needs a real MI355X (run with -m gpu)")
 
 
+def pytest_sessionstart(session):
+    """Load what is built; compile the HIP library (hipcc cross-compiles without a GPU) only if none is there."""
+    from etha_amd.build import ensure_built
+
+    ensure_built()
+
+
 @pytest.fixture(scope="session")
 def gpu_device():
     import torch
