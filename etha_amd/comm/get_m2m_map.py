@@ -60,6 +60,49 @@ def get_shard_shape(mesh_shape, placements, tensor_ndim: int) -> list[int]:
     return shards
 
 
+def _fine_shape(mesh_shape, placements, tensor_ndim: int) -> list[int]:
+    """Finest granularity a layout cuts each tensor dim into: a strided shard cuts ``split_factor`` times finer."""
+    fine = [1] * tensor_ndim
+    for size, p in zip(mesh_shape, placements):
+        if _is_strided(p):
+            fine[p.dim] *= int(size) * int(p.split_factor)
+        elif _is_shard(p):
+            fine[p.dim] *= int(size)
+    return fine
+
+
+def _whole_cells(idx: np.ndarray, ratio: int) -> bool:
+    """Is a rank's list of fine cells a sequence of whole coarse cells (``ratio`` fine cells each)?"""
+    if ratio == 1:
+        return True
+    if len(idx) % ratio:
+        return False
+    rows = idx.reshape(-1, ratio)
+    return bool(np.all(rows[:, 0] % ratio == 0) and np.all(rows == rows[:, :1] + np.arange(ratio)))
+
+
+def _cell_grid(src_shape, src_pl, src_shards, tgt_shape, tgt_pl, tgt_shards, ndim: int) -> list[int]:
+    """Cells per tensor dim: the coarsest grid on which every rank of both sides holds whole cells.
+
+    The reference uses ``lcm(source shards, target shards)`` (``get_m2m_map.py:155-172``), which is enough
+    when strided shards appear in their usual pairing (split factor = size of a later ``Shard`` mesh dim on
+    the same tensor dim).  A strided shard with any other split factor scatters a rank's pieces more finely;
+    then the dim is gridded by the lcm of both sides' finest cuts.
+    """
+    coarse = [math.lcm(s, t) for s, t in zip(src_shards, tgt_shards)]
+    fine = [math.lcm(math.lcm(a, b), c) for a, b, c in
+            zip(_fine_shape(src_shape, src_pl, ndim), _fine_shape(tgt_shape, tgt_pl, ndim), coarse)]
+    if fine == coarse:
+        return coarse
+    ok = [True] * ndim
+    for shape, pl in ((src_shape, src_pl), (tgt_shape, tgt_pl)):
+        for pos in range(int(np.prod(shape))):
+            idx = local_shard_indices(fine, shape, pl, np.unravel_index(pos, tuple(shape)))
+            for d in range(ndim):
+                ok[d] = ok[d] and _whole_cells(idx[d], fine[d] // coarse[d])
+    return [c if good else f for c, f, good in zip(coarse, fine, ok)]
+
+
 def _chunk(arr: np.ndarray, parts: int) -> list[np.ndarray]:
     """``torch.chunk`` on an index vector, padded with empty pieces up to ``parts``."""
     step = -(-len(arr) // parts) if len(arr) else 0
@@ -163,7 +206,7 @@ def get_m2m_map(
     ndim = max(_get_tensor_ndim(eff_source), _get_tensor_ndim(target_placements))
     src_shards = get_shard_shape(src_mesh.shape, eff_source, ndim)
     tgt_shards = get_shard_shape(tgt_mesh.shape, target_placements, ndim)
-    grid = [math.lcm(s, t) for s, t in zip(src_shards, tgt_shards)]
+    grid = _cell_grid(src_mesh.shape, eff_source, src_shards, tgt_mesh.shape, target_placements, tgt_shards, ndim)
     source_num_slicers = [g // s for g, s in zip(grid, src_shards)]
     target_num_slicers = [g // t for g, t in zip(grid, tgt_shards)]
 

@@ -37,6 +37,26 @@ def _layouts():
     add([2, 2], ["SS0/2", "S0"], [8, 8])
     add([2, 3], ["S1", "S0"], [7, 10])
     add([4], ["S0"], [3, 5])  # more ranks than rows: empty shards
+    # random layouts with strided shards of arbitrary split factors (also unpaired ones), even sizes
+    rng = np.random.RandomState(7)
+    for _ in range(40):
+        ndim = int(rng.randint(1, 4))
+        mesh = [int(rng.choice([1, 2, 3, 4])) for _ in range(int(rng.randint(1, 4)))]
+        while int(np.prod(mesh)) > 8:
+            mesh[int(rng.randint(len(mesh)))] = 1
+        codes, mult = [], [1] * ndim
+        for n in mesh:
+            kind, d = rng.choice(["S", "SS", "R"]), int(rng.randint(ndim))
+            if kind == "S":
+                codes.append(f"S{d}")
+                mult[d] *= n
+            elif kind == "SS":
+                sf = int(rng.choice([2, 3]))
+                codes.append(f"SS{d}/{sf}")
+                mult[d] *= n * sf
+            else:
+                codes.append("R")
+        add(mesh, codes, [m * int(rng.randint(1, 4)) for m in mult])
     return out
 
 

@@ -159,3 +159,23 @@ def test_partial_and_plain_tensors_bucket_alike_on_both_ends():
     recv_b = [b for b in chunk_to_bucket_ops(recv, 1 << 30) if b.src_rank == 0]
     assert [[c.nbytes for c in b.chunks] for b in send_b] == [[c.nbytes for c in b.chunks] for b in recv_b]
     assert len(send_b) == 2 and recv_b[1].chunks[0].source_partial_signature == (((0, 1), "sum"),)
+
+
+def test_strided_shard_grids():
+    """A strided shard in its usual pairing (split factor = size of the later Shard mesh dim on the same tensor
+    dim) keeps the reference's lcm-of-shard-counts grid; any other split factor scatters a rank's pieces more
+    finely and the dim is gridded by the finest cut."""
+    from torch.distributed.tensor.placement_types import _StridedShard
+
+    # the reference's own table: target (R, _StridedShard(1, 2), R, Shard(1)) on mesh (1,2,1,2) - paired
+    src = np.arange(4).reshape(2, 2, 1, 1)
+    tgt = np.arange(4, 8).reshape(1, 2, 1, 2)
+    m = get_m2m_map(src, (Replicate(), Replicate(), Shard(0), Shard(1)), tgt,
+                    (Replicate(), _StridedShard(1, split_factor=2), Replicate(), Shard(1)))
+    assert m.source_num_slicers == [1, 4] and m.target_num_slicers == [1, 1]
+    # unpaired: mesh (2,) _StridedShard(0, 3) -> rank r holds pieces {r, 2 + r, 4 + r} of six
+    m = get_m2m_map([0, 1], (_StridedShard(0, split_factor=3),), [2, 3], (Shard(0),))
+    assert m.source_num_slicers == [3] and m.target_num_slicers == [3]
+    got = {(r.src.rank, r.src.cell[0]): (r.dsts[0].rank, r.dsts[0].cell[0]) for r in m.routes}
+    # global cell of source rank r, local piece i is 2 * i + r; target rank 2 + g // 3 holds it at local g % 3
+    assert got == {(r, i): (2 + (2 * i + r) // 3, (2 * i + r) % 3) for r in (0, 1) for i in range(3)}

@@ -12,7 +12,7 @@ import math
 import numpy as np
 import pytest
 import torch
-from torch.distributed.tensor.placement_types import Partial, Replicate, Shard
+from torch.distributed.tensor.placement_types import Partial, Replicate, Shard, _StridedShard
 
 from etha_amd.comm import LoopbackWire
 from etha_amd.world import ReshardJob, TensorSpec
@@ -30,7 +30,9 @@ def _random_layout(rng, ndim, allow_partial):
     placements, partial = [], False
     for _ in mesh_shape:
         kind = rng.choice(["shard", "rep", "partial"] if allow_partial else ["shard", "rep"], p=None)
-        if kind == "shard":
+        if kind == "shard" and rng.random() < 0.15:  # a strided shard, also with split factors no later Shard pairs with
+            placements.append(_StridedShard(int(rng.integers(ndim)), split_factor=int(rng.choice([2, 3]))))
+        elif kind == "shard":
             placements.append(Shard(int(rng.integers(ndim))))
         elif kind == "partial":
             placements.append(Partial("sum"))
@@ -46,10 +48,17 @@ def _random_spec(rng, idx, wire_size):
     src_mesh, src_pl, partial = _random_layout(rng, ndim, allow_partial=wire_size in (2, 4) and rng.random() < 0.25)
     tgt_mesh, tgt_pl, _ = _random_layout(rng, ndim, allow_partial=False)
     shards = []
+    def cuts(mesh, placements, d):  # how finely a layout cuts dim d
+        out = 1
+        for m, p in zip(mesh, placements):
+            if isinstance(p, _StridedShard) and p.dim == d:
+                out *= m * p.split_factor
+            elif isinstance(p, Shard) and p.dim == d:
+                out *= m
+        return out
+
     for d in range(ndim):
-        s = math.prod(m for m, p in zip(src_mesh, src_pl) if isinstance(p, Shard) and p.dim == d)
-        t = math.prod(m for m, p in zip(tgt_mesh, tgt_pl) if isinstance(p, Shard) and p.dim == d)
-        shards.append(math.lcm(s, t))
+        shards.append(math.lcm(cuts(src_mesh, src_pl, d), cuts(tgt_mesh, tgt_pl, d)))
     shape = tuple(int(l * rng.integers(1, 7)) for l in shards)
     shape = shape[:-1] + (shape[-1] * int(rng.choice([1, 1, 8, 19])),)
     # one wire item size per batch: the reference cannot mix item sizes in a bucket unless every offset
