@@ -577,11 +577,12 @@ def test_equal_width_dtypes_convert_instead_of_reinterpreting(gpu_device):
 @pytest.mark.parametrize("seed", range(60))
 def test_random_batches_gpu(gpu_device, seed):
     """Random meshes / placements / shapes / dtypes / strides / bucket sizes on the GPU, against the oracle."""
-    from test_random_layouts_cpu import _random_spec
+    from test_random_layouts_cpu import _random_spec, _uneven_spec
 
     rng = np.random.default_rng(10_000 + seed)
     wire_size = int(rng.choice([1, 2, 2, 4, 4, 8]))
-    specs = [_random_spec(rng, i, wire_size) for i in range(int(rng.integers(1, 5)))]
+    spec_fn = _uneven_spec if seed % 4 == 3 else _random_spec  # every fourth batch: uneven shards, rank up to 5
+    specs = [spec_fn(rng, i, wire_size) for i in range(int(rng.integers(1, 5)))]
     bucket_size = [None, 64, 4096, 1 << 20][int(rng.integers(4))]
     view = None
     if rng.random() < 0.35:

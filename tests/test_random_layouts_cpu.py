@@ -135,11 +135,52 @@ def _peers_of(plan):
     return np.asarray(ptrs, dtype=np.uint64) if ptrs else None
 
 
+def _uneven_spec(rng, idx, wire_size):
+    """Uneven shard sizes (torch.chunk rule, empty shards included) on tensors of rank 1-5: every sharded dim is
+    cut by a single Shard on one side only, the layout pairs for which an uneven split is defined."""
+    del wire_size
+    ndim = int(rng.integers(1, 6))
+
+    def side(free_dims, partial_ok):
+        mesh = [int(rng.choice([1, 2, 3, 4, 6])) for _ in range(int(rng.integers(1, 3)))]
+        while math.prod(mesh) > 8:
+            mesh[int(rng.integers(len(mesh)))] = 1
+        placements, used, op = [], set(), str(rng.choice(["sum", "avg", "max"]))
+        for _ in mesh:
+            free = [d for d in free_dims if d not in used]
+            if free and rng.random() < 0.7:
+                d = int(rng.choice(free))
+                used.add(d)
+                placements.append(Shard(d))
+            elif partial_ok and rng.random() < 0.3:
+                placements.append(Partial(op))
+            else:
+                placements.append(Replicate())
+        return mesh, tuple(placements)
+
+    dims = list(range(ndim))
+    rng.shuffle(dims)
+    half = int(rng.integers(0, ndim + 1))
+    src_mesh, src_pl = side(dims[:half], True)
+    tgt_mesh, tgt_pl = side(dims[half:], False)
+    shape = tuple(int(rng.integers(1, 14)) for _ in range(ndim))
+    partial = any(isinstance(p, Partial) for p in src_pl)
+    tgt_start = 0 if (not partial and rng.random() < 0.3) else math.prod(src_mesh)
+    return TensorSpec(f"t{idx}", shape, mesh_of(0, src_mesh), src_pl, mesh_of(tgt_start, tgt_mesh), tgt_pl,
+                      torch.float32, seed=2000 + idx, std=1.0)
+
+
+@pytest.mark.parametrize("seed", range(60))
+def test_random_uneven_batches(seed):
+    test_random_batches(100_000 + seed, spec_fn=_uneven_spec)
+
+
 @pytest.mark.parametrize("seed", range(150))
-def test_random_batches(seed):
+def test_random_batches(seed, spec_fn=None):
+    spec_fn = spec_fn or _random_spec
     rng = np.random.default_rng(seed)
     wire_size = int(rng.choice([1, 2, 2, 4, 4, 8]))
-    specs = [_random_spec(rng, i, wire_size) for i in range(int(rng.integers(1, 5)))]
+    specs = [spec_fn(rng, i, wire_size) for i in range(int(rng.integers(1, 5)))]
     # all tensors of a batch share rank numbering: re-home each spec's meshes on disjoint or overlapping ranks as drawn
     bucket_size = [None, 64, 4096, 1 << 20][int(rng.integers(4))]
     view = None
