@@ -193,9 +193,11 @@ def test_random_batches(seed, spec_fn=None):
             wide = torch.zeros(shape, dtype=t.dtype)
             return wide[..., 1 : 1 + t.shape[-1]]
     merged = bool(rng.integers(2))
-    direct = rng.random() < 0.3  # no bucket buffers: the target side copies straight from the source shards
+    # wire options must not change results: plain buckets, lent single-chunk buckets, or no buckets at all
+    mode = ["buckets", "buckets", "zero_copy", "direct"][int(rng.integers(4))]
     job = ReshardJob(specs, device="cpu", bucket_size=bucket_size, keep_globals=True, fill=cpu_fill, local_view=view,
-                     wire=LoopbackWire("cpu", segment_bytes=1 << 22, host_inspection=True), direct=direct)
+                     wire=LoopbackWire("cpu", segment_bytes=1 << 22, host_inspection=True), direct=mode == "direct",
+                     zero_copy=mode == "zero_copy")
     ref = ReshardJob(specs, device="cpu", bucket_size=bucket_size, keep_globals=True, fill=cpu_fill, local_view=view)
     for a, b in zip(job.source_locals, ref.source_locals):  # Partial sources are drawn per job: make them equal
         for r in a:
