@@ -47,10 +47,6 @@ class TransferPlan:
         self.steps: list[tuple[str, int, int, object]] = []
         self.lent: set[int] = set()  # ids of source buckets that are consumed straight from their tensor
         self.direct_read_bytes = 0  # bytes the direct steps read from producers' tensors (source dtype)
-        send_index: dict[tuple, int] = {}
-        recv_index: dict[tuple, int] = {}
-        from .loopback import wire_key
-
         for bucket in buckets:
             if not bucket.chunks:
                 continue
@@ -85,11 +81,8 @@ class TransferPlan:
                         local.add_chunk(c)
                     self.steps.append((_SELF, first, len(bucket.chunks), None))
                 continue
-            key = wire_key(bucket)
             if bucket.is_source:
-                idx = send_index.get(key, 0)
-                send_index[key] = idx + 1
-                slot = wire.slot_for_send(bucket, idx, device)
+                slot = wire.slot_for_send(bucket, device)
                 if slot.borrowed:  # zero-copy: the consumer reads the tensor itself; nothing to launch
                     self.steps.append((_LEND, 0, 0, slot))
                     self.lent.add(id(bucket))
@@ -100,9 +93,7 @@ class TransferPlan:
                     send.add_chunk(c, c.tensor, c.src_slice, slot, off, reduce=reduce)
                 self.steps.append((_REDUCE if reduce else _PACK, first, len(bucket.chunks), slot))
             elif bucket.is_target:
-                idx = recv_index.get(key, 0)
-                recv_index[key] = idx + 1
-                slot = wire.slot_for_recv(bucket, idx)
+                slot = wire.slot_for_recv(bucket)
                 if slot.sources is not None:  # direct wire: copy from the producer's regions, no bucket
                     first = len(local)
                     reduce = slot.sources[0][3] is not None  # buckets never mix Partial and plain chunks

@@ -8,8 +8,10 @@ assigned when a bucket list is first planned and reused by every later transfer,
 consumer's tile program can hold absolute addresses.
 
 Matching follows the point-to-point rule of the reference's transports: the k-th bucket a rank
-sends on a wire key ``(src_rank, dst_ranks, transport)`` is the k-th bucket its peers receive on
-that key.
+sends on a wire key ``(src_rank, dst_ranks, transport)`` is the k-th bucket each of its peers
+receives on that key.  Because slots are assigned when bucket lists are *planned*, "k-th" counts
+over everything ever planned on the key: several registered batches between the same ranks get
+consecutive sequence numbers, provided both ends plan their lists in the same order.
 """
 
 from __future__ import annotations
@@ -95,7 +97,10 @@ class LoopbackWire:
         # a "sent" tensor must be left alone until the consumer has run.  Only within one process.
         self.direct_same_device = False
         self.pool: BucketPool | None = None
-        self._sent: dict[tuple, list[tuple[Slot, tuple[int, ...]]]] = defaultdict(list)
+        # per wire key: sequence number -> (slot, chunk sizes) of every planned send bucket still alive
+        self._sent: dict[tuple, dict[int, tuple[Slot, tuple[int, ...]]]] = defaultdict(dict)
+        self._send_seq: dict[tuple, int] = defaultdict(int)  # next number to hand to a send bucket, per key
+        self._recv_seq: dict[tuple, int] = defaultdict(int)  # next number a receiver expects, per (key, rank)
         self._plans: dict[tuple, object] = {}
         self._side_streams: list[torch.cuda.Stream] = []
 
@@ -108,17 +113,10 @@ class LoopbackWire:
         return self.pool
 
     # -- plan-time rendezvous -------------------------------------------------------------------
-    def slot_for_send(self, bucket: Bucket, index: int, device: torch.device) -> Slot:
-        """Slot of the ``index``-th bucket sent on this bucket's wire key (allocated on first use)."""
-        sent = self._sent[wire_key(bucket)]
+    def slot_for_send(self, bucket: Bucket, device: torch.device) -> Slot:
+        """Assign the next sequence number on this bucket's wire key and a slot to go with it."""
+        key = wire_key(bucket)
         sizes = tuple(c.nbytes for c in bucket.chunks)
-        if index < len(sent):
-            slot, known = sent[index]
-            if known != sizes:
-                raise RuntimeError(f"{bucket}: re-planned with a different chunk layout")
-            return slot
-        if index != len(sent):
-            raise RuntimeError(f"{bucket}: send buckets must be planned in order")
         slot = None
         if self.direct_same_device:
             self._pool_for(device)
@@ -136,19 +134,26 @@ class LoopbackWire:
                 slot.keepalive = region[3]
         if slot is None:
             slot = self._pool_for(device).alloc(bucket.total_bytes)
-        sent.append((slot, sizes))
+        seq = self._send_seq[key]
+        self._send_seq[key] = seq + 1
+        self._sent[key][seq] = (slot, sizes)
         return slot
 
-    def slot_for_recv(self, bucket: Bucket, index: int) -> Slot:
-        sent = self._sent.get(wire_key(bucket), [])
-        if index >= len(sent):
+    def slot_for_recv(self, bucket: Bucket) -> Slot:
+        """Slot of the send bucket this receive bucket pairs with: the next one its rank has not yet planned."""
+        key = wire_key(bucket)
+        who = (key, bucket.rank)
+        seq = self._recv_seq[who]
+        entry = self._sent.get(key, {}).get(seq)
+        if entry is None:
             raise RuntimeError(
-                f"{bucket}: no matching send bucket #{index} has been planned on this wire "
+                f"{bucket}: no matching send bucket #{seq} has been planned on this wire "
                 "(plan/run the source side first; a real wire would deadlock here)"
             )
-        slot, sizes = sent[index]
+        slot, sizes = entry
         if sizes != tuple(c.nbytes for c in bucket.chunks):
             raise RuntimeError(f"{bucket}: chunk layout differs from the matching send bucket")
+        self._recv_seq[who] = seq + 1
         return slot
 
     # -- across processes ----------------------------------------------------------------------
@@ -170,17 +175,17 @@ class LoopbackWire:
         slots: dict = {}
         for key, entries in self._sent.items():
             out = []
-            for slot, sizes in entries:
+            for seq, (slot, sizes) in sorted(entries.items()):
                 if slot.sources is not None:
                     raise NotImplementedError("a direct wire has no bucket buffers to export; it works inside one process")
                 if slot.borrowed:  # lives in a source tensor: export that allocation, range = the slot itself
                     with torch.cuda.device(self.pool.device):
                         segments.append({"ipc": nat.ipc_export(slot.ptr), "nbytes": slot.nbytes})
-                    out.append({"segment": len(segments) - 1, "offset": 0, "nbytes": slot.nbytes, "sizes": sizes})
+                    out.append({"seq": seq, "segment": len(segments) - 1, "offset": 0, "nbytes": slot.nbytes, "sizes": sizes})
                     continue
                 idx = next(i for i, seg in enumerate(self.pool.segments)
                            if seg.data_ptr() <= slot.ptr and slot.ptr + slot.nbytes <= seg.data_ptr() + seg.numel())
-                out.append({"segment": idx, "offset": slot.ptr - self.pool.segments[idx].data_ptr(),
+                out.append({"seq": seq, "segment": idx, "offset": slot.ptr - self.pool.segments[idx].data_ptr(),
                             "nbytes": slot.nbytes, "sizes": sizes})
             slots[key] = out
         return {"device": self.pool.device.index, "segments": segments, "slots": slots}
@@ -203,14 +208,14 @@ class LoopbackWire:
             for e in entries:
                 base, nbytes = bases[e["segment"]]
                 slot = Slot(ptr=base + e["offset"], nbytes=e["nbytes"], lo=base, hi=base + nbytes)
-                wire._sent[key].append((slot, tuple(e["sizes"])))
+                wire._sent[key][e["seq"]] = (slot, tuple(e["sizes"]))
         return wire
 
     def mark_packed(self) -> None:
         """Consumer side: the producer reported that every exported slot has been packed (and its stream
         synchronised) once more."""
         for entries in self._sent.values():
-            for slot, _ in entries:
+            for slot, _ in entries.values():
                 slot.filled += 1
 
     def close_imported(self) -> None:
@@ -251,13 +256,10 @@ class LoopbackWire:
                 continue
             owned = False
             for key, entries in list(self._sent.items()):
-                kept = [(s, sizes) for s, sizes in entries if s is not slot]
-                if len(kept) != len(entries):
+                mine = [seq for seq, (s, _) in entries.items() if s is slot]
+                for seq in mine:  # sequence numbers are never reused: later plans on this key keep theirs
+                    del entries[seq]
                     owned = True
-                    if kept:
-                        self._sent[key] = kept
-                    else:
-                        del self._sent[key]
             if (owned or kind == "pack") and not slot.borrowed:
                 if not any(slot is s for s in self.pool._free.get(slot.nbytes, [])):
                     self.pool.release(slot)
@@ -265,6 +267,8 @@ class LoopbackWire:
     def reset(self) -> None:
         self._plans.clear()
         self._sent.clear()
+        self._send_seq.clear()
+        self._recv_seq.clear()
         self.pool = None
 
 

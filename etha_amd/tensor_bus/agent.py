@@ -72,6 +72,8 @@ class BatchState:
     send_count: dict = field(default_factory=dict)
     recv_count: dict = field(default_factory=dict)
     owed: dict = field(default_factory=dict)  # destination rank -> number of receives its sources have asked of it
+    send_arrived: dict = field(default_factory=dict)  # rank -> number of send commands it has issued so far
+    partial_members: dict = field(default_factory=dict)  # rank -> other ranks of its Partial reductions (cached)
     transfer_signal: bool = False
 
 
@@ -386,6 +388,19 @@ class TensorBusAgent:
             self.wire.plan(buckets)
 
     @staticmethod
+    def _partial_members(batch: BatchState, rank: int) -> set[int]:
+        """The other ranks whose tensors this rank's send reads, or whose sends read this rank's tensors."""
+        if rank not in batch.partial_members:
+            members: set[int] = set()
+            for b in batch.send_buckets.get(rank, []):
+                for c in b.chunks:
+                    for group, _ in c.source_partial_groups or ():
+                        members.update(int(r) for r in group.ranks)
+            members.discard(rank)
+            batch.partial_members[rank] = members
+        return batch.partial_members[rank]
+
+    @staticmethod
     def _peers(buckets, attr: str) -> set[int]:
         out: set[int] = set()
         for b in buckets:
@@ -411,28 +426,43 @@ class TensorBusAgent:
                 )
             return True, None
         if cmd.transfer_type == "send":
-            if entry.started:  # already launched; this send lends tensor memory and waits for its receivers
+            members = self._partial_members(batch, rank)
+            if not entry.started:
                 gen = batch.send_count[rank]
-                if all(batch.recv_count.get(d, gen) >= gen for d in self._peers(buckets, "dst")):
-                    return True, entry.result
-                return False, None
-            gen = batch.send_count[rank]
-            for d in self._peers(buckets, "dst"):
-                if d in batch.recv_count and batch.recv_count[d] < gen:
-                    return False, None  # the previous generation has not been consumed yet
-            batch.transfer_signal = True
-            result = {"ms": 0.0}
-            self._unsynced.append((result, time.perf_counter(), f"batch {cmd.batch_id} rank {rank} send #{gen}"))
-            bucket_comm(buckets, wire=self.wire, merge_launches=True, synchronize=False)
-            batch.send_count[rank] = gen + 1
-            for d in self._peers(buckets, "dst"):
-                batch.owed[d] = max(batch.owed.get(d, 0), gen + 1)
-            if self.wire.plan(buckets).lends_tensor_memory():
+                for d in self._peers(buckets, "dst"):
+                    if d in batch.recv_count and batch.recv_count[d] < gen:
+                        return False, None  # the previous generation has not been consumed yet
+                if batch.send_arrived.get(rank, 0) <= gen:
+                    batch.send_arrived[rank] = gen + 1
+                    self._moved = True
+                # A Partial source is a collective among its members, as the all-reduce is in the reference:
+                # the primary's reduce reads every member's tensor, so it starts only once all of them have
+                # called send for this generation ...
+                if any(batch.send_arrived.get(m, 0) <= gen for m in members):
+                    return False, None
+                batch.transfer_signal = True
+                entry.result = {"ms": 0.0}
+                self._unsynced.append((entry.result, time.perf_counter(), f"batch {cmd.batch_id} rank {rank} send #{gen}"))
+                bucket_comm(buckets, wire=self.wire, merge_launches=True, synchronize=False)
+                batch.send_count[rank] = gen + 1
+                for d in self._peers(buckets, "dst"):
+                    batch.owed[d] = max(batch.owed.get(d, 0), gen + 1)
                 entry.started = True
-                entry.result = result
-                self.stats["transfers"] += 1
                 self._moved = True
+                self.stats["transfers"] += 1
+            done_gen = batch.send_count[rank]
+            # ... and no member's send returns before every member's launch is enqueued (the sweep synchronises
+            # the device before it replies), because a member's tensor is read by another member's kernel
+            if any(batch.send_count.get(m, 0) < done_gen for m in members):
                 return False, None
+            # a send whose tensors are lent to receivers - its own buckets, or a Partial reduction that another
+            # member ships and the receiver computes - waits for those receivers to have run
+            for m in members | {rank}:
+                theirs = batch.send_buckets.get(m)
+                if theirs and self.wire.plan(theirs).lends_tensor_memory() and not all(
+                        batch.recv_count.get(d, done_gen) >= done_gen for d in self._peers(theirs, "dst")):
+                    return False, None
+            return True, entry.result
         else:
             gen = batch.recv_count[rank]
             for s in self._peers(buckets, "src"):

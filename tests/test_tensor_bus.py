@@ -3,6 +3,7 @@
 import json
 import multiprocessing as mp
 import os
+import threading
 import time
 
 import pytest
@@ -286,5 +287,83 @@ def test_agent_zero_copy_send_completes_only_after_receive(gpu_device, tmp_path)
             h.close()
         for c in clients.values():
             c.close()
+    finally:
+        agent.close()
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("mode", ["buckets", "zero_copy", "direct"])
+def test_agent_many_rounds_two_batches_all_wire_modes(gpu_device, tmp_path, mode):
+    """Two registered batches (one with a Partial source) alternate for several rounds with new values each
+    time; senders never wait for receivers between rounds except where the wire lends their tensors.  Every
+    round's result must be the closed form of that round's values, in every wire mode."""
+    agent = TensorBusAgent(6, path_naming(str(tmp_path)), device=gpu_device, heartbeat_interval=0.05,
+                           zero_copy_single_chunk=mode == "zero_copy", direct_same_device=mode == "direct")
+    agent.start_in_thread()
+    naming = path_naming(str(tmp_path))
+    rounds = 4
+
+    def values(batch, i, round_, r=None):
+        g = torch.Generator().manual_seed(1000 * round_ + 10 * i + (0 if batch == "a" else 500) + (0 if r is None else 7 * r + 1))
+        shape = {("a", 0): (64, 96), ("a", 1): (128,), ("a", 2): (32, 40), ("b", 0): (48, 64), ("b", 1): (16, 24)}[(batch, i)]
+        return torch.randn(shape, generator=g)
+
+    # batch a: Shard(0)@4 -> Shard(1)@2 / Replicate / Shard(0); batch b: tensor 0 Partial@4 -> Shard(0)@2, tensor 1 Shard(1)@4 -> Replicate
+    src_a = {r: [values("a", 0, 0)[16 * r:16 * r + 16].clone().to(gpu_device), values("a", 1, 0)[32 * r:32 * r + 32].clone().to(gpu_device),
+                 values("a", 2, 0)[8 * r:8 * r + 8].clone().to(gpu_device)] for r in range(4)}
+    tgt_a = {4 + j: [torch.zeros(64, 48, device=gpu_device), torch.zeros(128, device=gpu_device), torch.zeros(16, 40, device=gpu_device)]
+             for j in range(2)}
+    src_b = {r: [values("b", 0, 0, r).to(gpu_device), values("b", 1, 0)[:, 6 * r:6 * r + 6].clone().to(gpu_device)] for r in range(4)}
+    tgt_b = {4 + j: [torch.zeros(24, 64, device=gpu_device), torch.zeros(16, 24, device=gpu_device)] for j in range(2)}
+    barrier = threading.Barrier(6)
+    failures = []
+
+    def body(r):
+        c = _client(naming, r, connection_timeout=10)
+        trainer = r < 4
+        me, other, n = ("trainer", "inference", 4) if trainer else ("inference", "trainer", 2)
+        mesh = torch.arange(n)
+        pls = {"a0": ((Shard(0),), (Shard(1),)), "a1": ((Shard(0),), (Replicate(),)), "a2": ((Shard(0),), (Shard(0),)),
+               "b0": ((Partial(),), (Shard(0),)), "b1": ((Shard(1),), (Replicate(),))}
+        for name, (sp, tp) in pls.items():
+            c.init_pair(name, me, other, n, device_mesh=mesh, placements=sp if trainer else tp, timeout=60)
+        mine_a, mine_b = (src_a[r], src_b[r]) if trainer else (tgt_a[r], tgt_b[r])
+        ha = c.register_tensors("a", [(t, f"a{i}") for i, t in enumerate(mine_a)], bucket_size=4096, timeout=60)
+        hb = c.register_tensors("b", [(t, f"b{i}") for i, t in enumerate(mine_b)], bucket_size=1 << 20, timeout=60)
+        for round_ in range(rounds):
+            for batch, h in (("a", ha), ("b", hb)):
+                if trainer:
+                    if round_ > 0:  # new values in the registered tensors
+                        if batch == "a":
+                            src_a[r][0].copy_(values("a", 0, round_)[16 * r:16 * r + 16])
+                            src_a[r][1].copy_(values("a", 1, round_)[32 * r:32 * r + 32])
+                            src_a[r][2].copy_(values("a", 2, round_)[8 * r:8 * r + 8])
+                        else:
+                            src_b[r][0].copy_(values("b", 0, round_, r))
+                            src_b[r][1].copy_(values("b", 1, round_)[:, 6 * r:6 * r + 6])
+                        torch.cuda.synchronize()
+                    h.transfer("send", blocking=True, timeout=60)
+                else:
+                    h.transfer("recv", blocking=True, timeout=60)
+                    j = r - 4
+                    if batch == "a":
+                        want = [values("a", 0, round_)[:, 48 * j:48 * j + 48], values("a", 1, round_), values("a", 2, round_)[16 * j:16 * j + 16]]
+                        got = tgt_a[r]
+                    else:
+                        acc = values("b", 0, round_, 0)
+                        for m in (1, 2, 3):
+                            acc = acc + values("b", 0, round_, m)
+                        want = [acc[24 * j:24 * j + 24], values("b", 1, round_)]
+                        got = tgt_b[r]
+                    for i, (g_, w_) in enumerate(zip(got, want)):
+                        if not torch.equal(g_.cpu(), w_):
+                            failures.append((mode, round_, batch, i, r))
+            barrier.wait(60)  # a new round only overwrites source values once every receiver has checked
+        ha.close(); hb.close(); c.close()
+
+    try:
+        run_ranks(body, range(6))
+        assert not failures, failures[:5]
+        assert agent.stats["transfers"] == 6 * 2 * rounds
     finally:
         agent.close()
