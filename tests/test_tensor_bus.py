@@ -359,11 +359,26 @@ def test_agent_many_rounds_two_batches_all_wire_modes(gpu_device, tmp_path, mode
                         if not torch.equal(g_.cpu(), w_):
                             failures.append((mode, round_, batch, i, r))
             barrier.wait(60)  # a new round only overwrites source values once every receiver has checked
+        # the same registration also carries the reverse direction: inference ranks send, trainer ranks receive
+        if not trainer:
+            j = r - 4
+            tgt_a[r][0].copy_(values("a", 0, 99)[:, 48 * j:48 * j + 48])
+            tgt_a[r][1].copy_(values("a", 1, 99))
+            tgt_a[r][2].copy_(values("a", 2, 99)[16 * j:16 * j + 16])
+            torch.cuda.synchronize()
+            ha.transfer("send", blocking=True, timeout=60)
+        else:
+            ha.transfer("recv", blocking=True, timeout=60)
+            want = [values("a", 0, 99)[16 * r:16 * r + 16], values("a", 1, 99)[32 * r:32 * r + 32], values("a", 2, 99)[8 * r:8 * r + 8]]
+            for i, (g_, w_) in enumerate(zip(src_a[r], want)):
+                if not torch.equal(g_.cpu(), w_):
+                    failures.append((mode, "reverse", "a", i, r))
+        barrier.wait(60)
         ha.close(); hb.close(); c.close()
 
     try:
         run_ranks(body, range(6))
         assert not failures, failures[:5]
-        assert agent.stats["transfers"] == 6 * 2 * rounds
+        assert agent.stats["transfers"] == 6 * 2 * rounds + 6
     finally:
         agent.close()
