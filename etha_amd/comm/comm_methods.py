@@ -38,8 +38,9 @@ _PACK, _REDUCE, _UNPACK, _SELF, _LEND, _DIRECT, _DIRECT_REDUCE = (
 class TransferPlan:
     """Compiled form of one rank's bucket list."""
 
-    def __init__(self, wire, buckets: list[Bucket]):
+    def __init__(self, wire, buckets: list[Bucket], scope=None):
         self.wire = wire
+        self.scope = scope
         self.buckets = buckets
         self.device: torch.device | None = None
         send, recv, local = DescBuilder(), DescBuilder(), SelfCopyBuilder()
@@ -82,7 +83,7 @@ class TransferPlan:
                     self.steps.append((_SELF, first, len(bucket.chunks), None))
                 continue
             if bucket.is_source:
-                slot = wire.slot_for_send(bucket, device)
+                slot = wire.slot_for_send(bucket, device, scope)
                 if slot.borrowed:  # zero-copy: the consumer reads the tensor itself; nothing to launch
                     self.steps.append((_LEND, 0, 0, slot))
                     self.lent.add(id(bucket))
@@ -93,7 +94,7 @@ class TransferPlan:
                     send.add_chunk(c, c.tensor, c.src_slice, slot, off, reduce=reduce)
                 self.steps.append((_REDUCE if reduce else _PACK, first, len(bucket.chunks), slot))
             elif bucket.is_target:
-                slot = wire.slot_for_recv(bucket)
+                slot = wire.slot_for_recv(bucket, scope)
                 if slot.sources is not None:  # direct wire: copy from the producer's regions, no bucket
                     first = len(local)
                     reduce = slot.sources[0][3] is not None  # buckets never mix Partial and plain chunks
@@ -259,6 +260,7 @@ def bucket_comm(
     merge_launches: bool = False,
     synchronize: bool = True,
     fanout: int = 1,
+    scope=None,
 ) -> None:
     """Run the bucket pipeline for one rank's buckets.
 
@@ -266,7 +268,8 @@ def bucket_comm(
     there is nothing to throttle.  The keyword-only arguments are additions: ``wire`` selects the
     loopback wire (default: the process-wide one), ``merge_launches`` fuses consecutive buckets of
     one kind into a single launch, ``synchronize=False`` leaves the stream un-synchronised, ``fanout``
-    spreads per-bucket launches over that many side streams (see :meth:`TransferPlan.run`).
+    spreads per-bucket launches over that many side streams (see :meth:`TransferPlan.run`), ``scope``
+    namespaces the pairing of send and receive buckets on the wire (see :class:`LoopbackWire`).
     """
     del max_in_flight
     if wire is None:
@@ -275,7 +278,7 @@ def bucket_comm(
         wire = default_wire()
     if not buckets:
         return
-    plan = wire.plan(buckets)
+    plan = wire.plan(buckets, scope=scope)
     plan.run(merge_launches=merge_launches, fanout=fanout)
     if synchronize and plan.device is not None:
         torch.cuda.current_stream(plan.device).synchronize()

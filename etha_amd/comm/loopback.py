@@ -11,7 +11,9 @@ Matching follows the point-to-point rule of the reference's transports: the k-th
 sends on a wire key ``(src_rank, dst_ranks, transport)`` is the k-th bucket each of its peers
 receives on that key.  Because slots are assigned when bucket lists are *planned*, "k-th" counts
 over everything ever planned on the key: several registered batches between the same ranks get
-consecutive sequence numbers, provided both ends plan their lists in the same order.
+consecutive sequence numbers, provided both ends plan their lists in the same order.  A caller that
+cannot promise that order names a ``scope`` (any hashable, e.g. a batch id) when planning: sequence
+numbers are then counted per scope.
 """
 
 from __future__ import annotations
@@ -113,9 +115,9 @@ class LoopbackWire:
         return self.pool
 
     # -- plan-time rendezvous -------------------------------------------------------------------
-    def slot_for_send(self, bucket: Bucket, device: torch.device) -> Slot:
-        """Assign the next sequence number on this bucket's wire key and a slot to go with it."""
-        key = wire_key(bucket)
+    def slot_for_send(self, bucket: Bucket, device: torch.device, scope=None) -> Slot:
+        """Assign the next sequence number on this bucket's wire key (within ``scope``) and a slot to go with it."""
+        key = (scope, *wire_key(bucket))
         sizes = tuple(c.nbytes for c in bucket.chunks)
         slot = None
         if self.direct_same_device:
@@ -139,9 +141,9 @@ class LoopbackWire:
         self._sent[key][seq] = (slot, sizes)
         return slot
 
-    def slot_for_recv(self, bucket: Bucket) -> Slot:
+    def slot_for_recv(self, bucket: Bucket, scope=None) -> Slot:
         """Slot of the send bucket this receive bucket pairs with: the next one its rank has not yet planned."""
-        key = wire_key(bucket)
+        key = (scope, *wire_key(bucket))
         who = (key, bucket.rank)
         seq = self._recv_seq[who]
         entry = self._sent.get(key, {}).get(seq)
@@ -235,13 +237,15 @@ class LoopbackWire:
         return self._side_streams[:n]
 
     # -- plan cache -----------------------------------------------------------------------------
-    def plan(self, buckets: list[Bucket]):
+    def plan(self, buckets: list[Bucket], scope=None):
+        """Compiled plan of a bucket list (cached by the identity of its buckets).  ``scope`` only matters when the
+        plan is first built: it namespaces the send/receive pairing."""
         from .comm_methods import TransferPlan
 
         key = tuple(id(b) for b in buckets)
         plan = self._plans.get(key)
         if plan is None:
-            plan = TransferPlan(self, list(buckets))
+            plan = TransferPlan(self, list(buckets), scope=scope)
             self._plans[key] = plan
         return plan
 

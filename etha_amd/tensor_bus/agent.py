@@ -66,7 +66,9 @@ class BatchState:
     pair_names: list[str]
     bucket_size: int | None
     registrations: dict = field(default_factory=dict)  # rank -> [(pair_name, tensor)]
-    planned: bool = False
+    planned_ranks: set = field(default_factory=set)  # ranks whose bucket lists exist
+    send_compiled: set = field(default_factory=set)  # ranks whose send / receive tile programs exist
+    recv_compiled: set = field(default_factory=set)
     send_buckets: dict = field(default_factory=dict)
     recv_buckets: dict = field(default_factory=dict)
     send_count: dict = field(default_factory=dict)
@@ -326,29 +328,51 @@ class TensorBusAgent:
             for p in pair_names:
                 if p not in self.pairs or not self.pairs[p].matched:
                     raise ValueError(f"RegisterTensors for unknown pair: {p}")
-            batch = self.batches.setdefault(cmd.batch_id, BatchState(cmd.batch_id, pair_names, cmd.bucket_size))
-            if batch.planned:
-                raise ValueError(f"batch {cmd.batch_id} is already registered")
+                self._side_of(self.pairs[p], entry.rank)  # raises if the rank is not part of the pair
+            batch = self.batches.setdefault(cmd.batch_id, BatchState(cmd.batch_id, [], cmd.bucket_size))
+            if entry.rank in batch.registrations:
+                raise ValueError(f"batch {cmd.batch_id} is already registered by rank {entry.rank}")
+            for p in pair_names:
+                if p not in batch.pair_names:
+                    batch.pair_names.append(p)
             index = self.device.index if self.device.type == "cuda" else None
             batch.registrations[entry.rank] = [(p, import_tensor(payload, index)) for p, payload in cmd.tensors]
             for _, t in batch.registrations[entry.rank]:
                 self.stats["ipc_tensors" if isinstance(t, IpcTensor) else "in_process_tensors"] += 1
+            self._plan_ready_ranks(batch)
         batch = self.batches[cmd.batch_id]
-        if batch.planned:
-            return True, None
-        expected = set()
-        for p in batch.pair_names:
-            for ranks in self.pairs[p].ranks.values():
-                expected.update(ranks)
-        if not expected.issubset(batch.registrations):
-            return False, None
-        self._plan_batch(batch)
-        return True, None
+        return (True, None) if entry.rank in batch.planned_ranks else (False, None)
 
-    def _plan_batch(self, batch: BatchState) -> None:
-        send_chunks: dict[int, list] = {}
-        recv_chunks: dict[int, list] = {}
-        for pair_name in batch.pair_names:
+    def _pair_complete(self, batch: BatchState, pair_name: str) -> bool:
+        """Has every rank of the pair registered tensors for it in this batch?"""
+        pair = self.pairs[pair_name]
+        return all(r in batch.registrations and any(p == pair_name for p, _ in batch.registrations[r])
+                   for ranks in pair.ranks.values() for r in ranks)
+
+    def _plan_ready_ranks(self, batch: BatchState) -> None:
+        """Plan every registered rank whose pairs have all become complete (each rank is planned once; ranks of
+        one batch may take part in different pairs, as each rank's own agent would plan only its own pairs)."""
+        for rank in sorted(batch.registrations):
+            if rank in batch.planned_ranks:
+                continue
+            mine = list(dict.fromkeys(p for p, _ in batch.registrations[rank]))
+            if all(self._pair_complete(batch, p) for p in mine):
+                self._plan_rank(batch, rank, mine)
+                batch.planned_ranks.add(rank)
+        # tile programs: a receive list pairs with send lists, so it is compiled once all its sources' lists are
+        for rank in sorted(batch.planned_ranks - batch.send_compiled):
+            self._plan_if_device(batch.send_buckets.get(rank), batch.batch_id)
+            batch.send_compiled.add(rank)
+        for rank in sorted(batch.planned_ranks - batch.recv_compiled):
+            buckets = batch.recv_buckets.get(rank)
+            if all(s in batch.send_compiled for s in self._peers(buckets or [], "src")):
+                self._plan_if_device(buckets, batch.batch_id)
+                batch.recv_compiled.add(rank)
+
+    def _plan_rank(self, batch: BatchState, rank: int, pair_names: list[str]) -> None:
+        send_chunks: list = []
+        recv_chunks: list = []
+        for pair_name in pair_names:
             pair = self.pairs[pair_name]
             per_rank = {r: [t for p, t in regs if p == pair_name] for r, regs in batch.registrations.items()}
             names = sorted(pair.sides)
@@ -363,29 +387,21 @@ class TensorBusAgent:
                     src = {r: per_rank[r][i] for r in pair.ranks[a]}
                     tgt = {r: per_rank[r][i] for r in pair.ranks[b]}
                     wire_dtype = transfer_dtype_rule(next(iter(src.values())).dtype, next(iter(tgt.values())).dtype)
-                    mesh_a = pair.meshes[a][0]
-                    for r, t in src.items():
-                        groups = create_partial_groups(mesh_a, m2m.source_partial_reductions, r, src) or None
-                        send_chunks.setdefault(r, []).extend(
-                            m2m_to_chunks(m2m, r, source_tensor=t, transfer_dtype=wire_dtype, source_partial_groups=groups))
-                    for r, t in tgt.items():
-                        recv_chunks.setdefault(r, []).extend(
-                            m2m_to_chunks(m2m, r, target_tensor=t, transfer_dtype=wire_dtype))
+                    if rank in src:
+                        groups = create_partial_groups(pair.meshes[a][0], m2m.source_partial_reductions, rank, src) or None
+                        send_chunks.extend(m2m_to_chunks(m2m, rank, source_tensor=src[rank], transfer_dtype=wire_dtype,
+                                                         source_partial_groups=groups))
+                    if rank in tgt:
+                        recv_chunks.extend(m2m_to_chunks(m2m, rank, target_tensor=tgt[rank], transfer_dtype=wire_dtype))
         size = batch.bucket_size or 1
-        batch.send_buckets = {r: chunk_to_bucket_ops(c, size) for r, c in sorted(send_chunks.items())}
-        batch.recv_buckets = {r: chunk_to_bucket_ops(c, size) for r, c in sorted(recv_chunks.items())}
-        # compile now, sources first, so that the first transfer finds every slot
-        for buckets in batch.send_buckets.values():
-            self._plan_if_device(buckets)
-        for buckets in batch.recv_buckets.values():
-            self._plan_if_device(buckets)
-        batch.send_count = {r: 0 for r in batch.send_buckets}
-        batch.recv_count = {r: 0 for r in batch.recv_buckets}
-        batch.planned = True
+        batch.send_buckets[rank] = chunk_to_bucket_ops(send_chunks, size)
+        batch.recv_buckets[rank] = chunk_to_bucket_ops(recv_chunks, size)
+        batch.send_count[rank] = 0
+        batch.recv_count[rank] = 0
 
-    def _plan_if_device(self, buckets) -> None:
+    def _plan_if_device(self, buckets, scope) -> None:
         if buckets and buckets[0].chunks[0].tensor.device.type == "cuda":
-            self.wire.plan(buckets)
+            self.wire.plan(buckets, scope=scope)
 
     @staticmethod
     def _partial_members(batch: BatchState, rank: int) -> set[int]:
@@ -412,9 +428,9 @@ class TensorBusAgent:
         batch = self.batches.get(cmd.batch_id)
         if batch is None:
             raise ValueError(f"Transfer for unknown batch: {cmd.batch_id}")
-        if not batch.planned:
-            return False, None
         rank = entry.rank
+        if rank not in batch.planned_ranks:
+            return False, None
         table = batch.send_buckets if cmd.transfer_type == "send" else batch.recv_buckets
         other = batch.recv_buckets if cmd.transfer_type == "send" else batch.send_buckets
         buckets = table.get(rank)
@@ -443,7 +459,7 @@ class TensorBusAgent:
                 batch.transfer_signal = True
                 entry.result = {"ms": 0.0}
                 self._unsynced.append((entry.result, time.perf_counter(), f"batch {cmd.batch_id} rank {rank} send #{gen}"))
-                bucket_comm(buckets, wire=self.wire, merge_launches=True, synchronize=False)
+                bucket_comm(buckets, wire=self.wire, merge_launches=True, synchronize=False, scope=batch.batch_id)
                 batch.send_count[rank] = gen + 1
                 for d in self._peers(buckets, "dst"):
                     batch.owed[d] = max(batch.owed.get(d, 0), gen + 1)
@@ -470,7 +486,7 @@ class TensorBusAgent:
                     return False, None  # wait for the source's send of this generation
             result = {"ms": 0.0}
             self._unsynced.append((result, time.perf_counter(), f"batch {cmd.batch_id} rank {rank} recv #{gen}"))
-            bucket_comm(buckets, wire=self.wire, merge_launches=True, synchronize=False)
+            bucket_comm(buckets, wire=self.wire, merge_launches=True, synchronize=False, scope=batch.batch_id)
             batch.recv_count[rank] = gen + 1
             if all(batch.recv_count.get(d, 0) >= n for d, n in batch.owed.items()):
                 batch.transfer_signal = False  # every destination of every send so far has received

@@ -70,7 +70,7 @@ def test_init_pair_register_and_errors_on_cpu(agent_factory):
     state = json.load(open(naming(0)[1]))
     assert state["pairs"]["w"] == "matched"
     batch = agent.batches["b0"]
-    assert batch.planned and len(batch.send_buckets[0]) == 1 and len(batch.recv_buckets[2]) == 2
+    assert batch.planned_ranks == {0, 1, 2} and len(batch.send_buckets[0]) == 1 and len(batch.recv_buckets[2]) == 2
     assert batch.send_buckets[1][0].chunks[0].dst_ranks == (2,)
     assert handlers[2].query_transfer_signal() is False
     with pytest.raises(ValueError, match="cannot be empty"):
@@ -382,3 +382,42 @@ def test_agent_many_rounds_two_batches_all_wire_modes(gpu_device, tmp_path, mode
         assert agent.stats["transfers"] == 6 * 2 * rounds + 6
     finally:
         agent.close()
+
+
+@pytest.mark.gpu
+def test_ranks_of_one_batch_in_different_pairs(gpu_device, agent_factory):
+    """One batch id, two pairs with different members: ranks 0-1 -> rank 4 over pair "p", ranks 2-3 -> rank 5 over
+    pair "q"; rank 4 additionally receives from pair "q"'s broadcast.  Every rank registers only its own pairs and
+    is planned as soon as those are complete."""
+    agent, naming = agent_factory(6, device=gpu_device)
+    g = torch.Generator().manual_seed(9)
+    gp, gq = torch.randn(32, 16, generator=g), torch.randn(8, 24, generator=g)
+    src_p = {r: gp[16 * r:16 * r + 16].clone().to(gpu_device) for r in (0, 1)}
+    src_q = {r: gq[:, 12 * (r - 2):12 * (r - 2) + 12].clone().to(gpu_device) for r in (2, 3)}
+    tgt_p = {4: torch.zeros(32, 16, device=gpu_device)}
+    tgt_q = {4: torch.zeros(8, 24, device=gpu_device), 5: torch.zeros(8, 24, device=gpu_device)}
+
+    def body(r):
+        c = _client(naming, r, connection_timeout=5)
+        regs = []
+        if r in (0, 1):
+            c.init_pair("p", "src", "dst", 2, device_mesh=torch.arange(2), placements=(Shard(0),), timeout=30)
+            regs.append((src_p[r], "p"))
+        if r in (2, 3):
+            c.init_pair("q", "src", "dst", 2, device_mesh=torch.arange(2), placements=(Shard(1),), timeout=30)
+            regs.append((src_q[r], "q"))
+        if r == 4:
+            c.init_pair("p", "dst", "src", 1, device_mesh=torch.arange(1), placements=(Replicate(),), timeout=30)
+            regs.append((tgt_p[4], "p"))
+        if r in (4, 5):
+            c.init_pair("q", "dst", "src", 2, device_mesh=torch.arange(2), placements=(Replicate(),), timeout=30)
+            regs.append((tgt_q[r], "q"))
+        h = c.register_tensors("mixed", regs, bucket_size=1 << 20, timeout=30)
+        h.transfer("send" if r < 4 else "recv", blocking=True, timeout=30)
+        h.close()
+        c.close()
+
+    run_ranks(body, range(6))
+    torch.cuda.synchronize()
+    assert torch.equal(tgt_p[4].cpu(), gp)
+    assert torch.equal(tgt_q[4].cpu(), gq) and torch.equal(tgt_q[5].cpu(), gq)
