@@ -9,13 +9,16 @@ agent rank of the GPU:
 * ``InitPair``: a pair matches when ``expected_world_size`` ranks of both sides have registered;
   meshes are rebuilt as ``arange`` from each side's first rank and the M2M map is planned in both
   directions, skipping a direction whose target is Partial (``agent.py:203-436``);
-* ``RegisterTensors``: tensors arrive as hipIPC handles; when every rank of the batch has
-  registered, chunks and buckets are planned per rank with the transfer-dtype rule
-  (``agent.py:543-687``) and compiled into device tile programs;
+* ``RegisterTensors``: tensors arrive as hipIPC handles; a rank is planned once every pair it named
+  is complete in the batch (all ranks of both sides have registered tensors for it): chunks and
+  buckets with the transfer-dtype rule (``agent.py:543-687``), compiled into device tile programs;
 * ``Transfer``: runs that rank's send or recv buckets through the HIP path (``agent.py:438-507``).
   The reference brackets a transfer with barriers over both sides; here a send waits until its
   previous generation has been consumed and a recv waits for its sources' sends, which gives the
-  same lock step;
+  same lock step.  The sends of the members of a Partial reduction form a collective (the primary's
+  kernel reads every member's tensor), and a send whose tensors are lent to the receivers completes
+  only after they have run.  Commands that are ready are handled in one sweep: enqueue every launch,
+  synchronise the device once, publish state once, reply;
 * ``QueryStatus`` (``transfer_signal``) and ``CleanupBatch``.
 
 A failing command is reported back to the worker as an exception of the same type; the reference
