@@ -22,7 +22,7 @@ import torch
 
 from .command_queue import BusyError, CommandQueue, Completion
 from .commands import CleanupBatch, InitPair, QueryStatus, RegisterTensors, Transfer
-from .ipc_tensor import export_tensor
+from .ipc_tensor import export_tensor, release_local
 
 logger = logging.getLogger(__name__)
 
@@ -88,7 +88,6 @@ class TensorBusClient:
         if lmdb_command_queue_path is None:
             lmdb_command_queue_path = os.environ.get("TENSOR_BUS_COMMAND_QUEUE_PATH")
         self.command_queue = CommandQueue(lmdb_command_queue_path)
-        self._payloads: dict[str, list[bytes]] = {}
 
     # ---- plumbing ---------------------------------------------------------------------------
     def _read_state(self) -> dict | None:
@@ -175,17 +174,17 @@ class TensorBusClient:
             if t.device.type == "cuda":
                 torch.cuda.current_stream(t.device).synchronize()  # the agent works on its own stream
         payloads = [(pair_name, export_tensor(tensor)) for tensor, pair_name in tensors]
-        self._payloads[batch_id] = [p for _, p in payloads]
         msg = RegisterTensors(batch_id=batch_id, tensors=payloads, bucket_size=bucket_size)
-        self._execute_command_with_semaphore(msg, "register_tensors", context_id=f"batch_{batch_id}", blocking=True, timeout=timeout)
+        try:
+            self._execute_command_with_semaphore(msg, "register_tensors", context_id=f"batch_{batch_id}", blocking=True,
+                                                 timeout=timeout)
+        finally:
+            # An agent in this process has taken the tensor objects by now; an agent in another process maps the
+            # memory and, as in the reference, the worker keeps its tensors alive for as long as the batch lives.
+            for _, p in payloads:
+                release_local(p)
         unique_pair_names = list(dict.fromkeys(pair_name for _, pair_name in tensors))
         return BatchHandler(client=self, batch_id=batch_id, pair_names=unique_pair_names)
 
     def close(self):
-        from .ipc_tensor import release_local
-
-        for payloads in self._payloads.values():
-            for p in payloads:
-                release_local(p)
-        self._payloads.clear()
         self.command_queue.close()

@@ -73,7 +73,13 @@ def trainer_process(tmpdir, device, rounds, out_q):
         for i, (_, shape, src, _, sdt, _) in enumerate(BUS_TENSORS):
             g = _global(i, 0).to(names[sdt])
             for pos, r in enumerate(SRC_RANKS):
-                shards[r].append(local_shard(g, (len(SRC_RANKS),), parse_placements(src), (pos,)).clone().to(device))
+                shard = local_shard(g, (len(SRC_RANKS),), parse_placements(src), (pos,)).clone().to(device)
+                if i == 1:  # a view at a storage offset inside a wider parent: strides and offset must travel too
+                    parent = torch.zeros(shard.shape[0], shard.shape[1] + 6, dtype=shard.dtype, device=device)
+                    view = parent[:, 3 : 3 + shard.shape[1]]
+                    view.copy_(shard)
+                    shard = view
+                shards[r].append(shard)
         barrier = threading.Barrier(len(SRC_RANKS))
 
         def rank_body(r):
