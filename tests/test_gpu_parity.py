@@ -599,11 +599,12 @@ def test_random_batches_gpu(gpu_device, seed):
                          zero_copy=mode == "zero_copy", direct=mode == "direct")
     cpu_job = ReshardJob(specs, device="cpu", bucket_size=bucket_size, keep_globals=True, fill=cpu_fill, local_view=view)
     mirror_partials(gpu_job, cpu_job)
-    gpu_job.run(merge_launches=merge)
+    fanout = 3 if seed % 5 == 4 else 1  # every fifth batch: launches spread over side streams
+    gpu_job.run(merge_launches=merge, fanout=fanout)
     run_oracle(cpu_job)
     for i, spec in enumerate(specs):
         for r, t in gpu_job.target_locals[i].items():
-            assert_bit_equal(t, cpu_job.target_locals[i][r], f"seed {seed} ({mode}) {spec.name} rank {r}")
+            assert_bit_equal(t, cpu_job.target_locals[i][r], f"seed {seed} ({mode}, fanout {fanout}) {spec.name} rank {r}")
 
 
 @pytest.mark.parametrize("dtype", [torch.int8, torch.bfloat16, torch.float32, torch.float64])
