@@ -354,3 +354,22 @@ def test_direct_table_rejects_partial_destinations_and_selfcopy_rejects_partial_
         nat.Table.create_selfcopy(bad_src.reshape(1), dst.reshape(1), upload=False)
     with pytest.raises(nat.EthaNativeError, match="outside partial_ptrs"):
         nat.Table.create_selfcopy(bad_src.reshape(1), dst.reshape(1), upload=False, partial_ptrs=ptrs[:1])
+
+
+def test_expanded_source_with_zero_stride():
+    """A source that is an expanded view (stride 0 along a dim) packs as that many copies; it can only be read."""
+    arena = HostArena(8192)
+    t = arena.alloc(64)
+    row = np.arange(8, dtype=np.float32)
+    arena.bytes_at(t, 32)[:] = row.view(np.uint8)
+    b = arena.alloc(5 * 32 + 6 * 4 * 3)
+    d = _mk_desc(t, t, t + 32, b, b, b + 5 * 32, (0, 0), (5, 8), (0, 1), nat.F32, nat.F32)
+    table = nat.Table.create(d.reshape(1), upload=False)
+    execute(table, arena, "pack")
+    assert np.array_equal(arena.bytes_at(b, 5 * 32).view(np.float32).reshape(5, 8), np.tile(row, (5, 1)))
+    # both dims expanded from one element, converting: 2 x 3 copies of one value
+    d2 = _mk_desc(t + 4, t, t + 32, b, b, b + 6 * 2, (0, 0), (2, 3), (0, 0), nat.F32, nat.BF16)
+    table2 = nat.Table.create(d2.reshape(1), upload=False)
+    execute(table2, arena, "pack")
+    want = co.cast(np.full(6, 1.0, dtype=np.float32).view(np.uint32), co.F32, co.BF16, np.uint16)
+    assert np.array_equal(arena.bytes_at(b, 12).view(np.uint16), want)
