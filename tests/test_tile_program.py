@@ -373,3 +373,68 @@ def test_expanded_source_with_zero_stride():
     execute(table2, arena, "pack")
     want = co.cast(np.full(6, 1.0, dtype=np.float32).view(np.uint32), co.F32, co.BF16, np.uint16)
     assert np.array_equal(arena.bytes_at(b, 12).view(np.uint16), want)
+
+
+@pytest.mark.parametrize("seed", range(120))
+def test_random_descriptors_against_numpy(seed):
+    """Random parent shapes (1-6 dims), storage permutations and padding, slices (also empty), dtype pairs,
+    address skews and bucket offsets: pack must equal numpy's gather (+ the oracle's cast), unpack must write the
+    region and nothing else."""
+    r = np.random.RandomState(seed)
+    nd = r.randint(1, 7)
+    pshape = [int(r.randint(1, 7)) for _ in range(nd)]
+    pshape[-1] = int(r.choice([1, 3, 8, 17, 64, 100, 257, 1024]))
+    if r.rand() < 0.3 and nd > 1:
+        pshape[int(r.randint(nd))] = int(r.choice([33, 70, 200]))
+    floats = [nat.F16, nat.BF16, nat.F32, nat.F64]
+    if r.rand() < 0.5:
+        tdt, wdt = int(r.choice(floats)), int(r.choice(floats))
+    else:
+        tdt = wdt = int(r.choice([nat.B8, nat.B16, nat.B32, nat.B64, nat.F32, nat.BF16]))
+    es, ws = ES[tdt], ES[wdt]
+    raw_of = {1: np.uint8, 2: np.uint16, 4: np.uint32, 8: np.uint64}
+    perm = list(r.permutation(nd)) if r.rand() < 0.4 else list(range(nd))
+    pad = int(r.choice([0, 0, 1, 5]))  # extra elements at the end of the innermost storage dim
+    stride, acc = [0] * nd, 1
+    for k in range(nd - 1, -1, -1):
+        stride[perm[k]] = acc
+        acc *= pshape[perm[k]] + (pad if k == nd - 1 else 0)
+    pn = acc
+    start = [int(r.randint(0, s)) for s in pshape]
+    cshape = [int(r.randint(1, s - st + 1)) for s, st in zip(pshape, start)]
+    if r.rand() < 0.1:
+        cshape[int(r.randint(nd))] = 0
+    cn = int(np.prod(cshape))
+    skew = int(r.choice([0, 0, 1, 2, 3])) * es
+    arena = HostArena(2 * pn * es + cn * ws + 65536)
+    t_addr, t2_addr = arena.alloc(pn * es, skew=skew), arena.alloc(pn * es, skew=skew)
+    if tdt in floats:
+        raw = co.cast(r.randn(pn).astype(np.float64).view(np.uint64), co.F64, tdt, raw_of[es])
+    else:
+        raw = r.randint(0, 256, pn * es).astype(np.uint8).view(raw_of[es])
+    arena.bytes_at(t_addr, pn * es)[:] = raw.view(np.uint8)
+    arena.bytes_at(t2_addr, pn * es)[:] = 0x5A
+    boff = int(r.randint(0, 9)) * ws
+    b_addr = arena.alloc(cn * ws + boff + 64)
+    region = tuple(slice(a, a + n) for a, n in zip(start, cshape))
+
+    def strided(flat, item):
+        return np.lib.stride_tricks.as_strided(flat, shape=pshape, strides=[s * item for s in stride])
+
+    d = _mk_desc(t_addr, t_addr, t_addr + pn * es, b_addr + boff, b_addr, b_addr + boff + cn * ws + 64, start, cshape,
+                 stride, tdt, wdt)
+    execute(nat.Table.create(d.reshape(1), upload=False), arena, "pack")
+    want = np.ascontiguousarray(strided(raw, es)[region]).reshape(-1)
+    if tdt != wdt:
+        want = co.cast(want, tdt, wdt, raw_of[ws])
+    assert np.array_equal(arena.bytes_at(b_addr + boff, cn * ws).view(raw_of[ws]), want), "pack"
+    d2 = _mk_desc(t2_addr, t2_addr, t2_addr + pn * es, b_addr + boff, b_addr, b_addr + boff + cn * ws + 64, start, cshape,
+                  stride, tdt, wdt)
+    execute(nat.Table.create(d2.reshape(1), upload=False), arena, "unpack")
+    back = arena.bytes_at(t2_addr, pn * es).view(raw_of[es])
+    want_back = want if tdt == wdt else co.cast(want, wdt, tdt, raw_of[es])
+    assert np.array_equal(strided(back, es)[region], want_back.reshape(cshape)), "unpack"
+    untouched = np.ones(pn, dtype=bool)
+    untouched[strided(np.arange(pn), 8)[region].reshape(-1)] = False
+    fill = np.frombuffer(bytes([0x5A]) * es, dtype=raw_of[es])[0]
+    assert np.all(back[untouched] == fill), "bytes outside the region were written"
