@@ -1,10 +1,11 @@
 """Headline benchmark: effective reshard GB/s (pack + unpack) on one MI355X.
 
 One step = one pass of the hot path over the workload: every source rank packs its buckets for the
-measured target rank's share, then that target rank unpacks them.  Inputs are resident in HBM
-before the timed region.  Prints ONE JSON line.
+measured target rank's share and that target rank unpacks them, through a bounded bucket pool (a ring
+of ``--max-in-flight`` slots per channel).  Inputs are resident in HBM before the timed region.
+Prints ONE JSON line.
 
-    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload NAME] [--per-bucket]
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload NAME] [--per-bucket] [--pool resident]
 """
 
 from __future__ import annotations
@@ -19,16 +20,7 @@ ROOT = os.path.dirname(os.path.abspath(__file__))
 sys.path.insert(0, ROOT)
 
 HBM_PEAK_GBS = 8000.0  # MI355X HBM3E, published
-
-# HBM bytes per launch of the dominant kernel, from two rocprofv3 --pmc runs (FETCH_SIZE, WRITE_SIZE), each
-# scaled by what the counter reads for a plain 1 GiB copy; the summary of those runs is
-# profiles/etha_tile_kernel_llama3_8b_fsdp8_to_tp2.txt.  Keyed by (workload, kernel, launch granularity).
-MEASURED_TRAFFIC_BYTES = {
-    ("llama3_8b_fsdp8_to_tp2", "etha_tile_kernel<false>", "run of buckets"): 2043040739,
-    ("llama3_8b_fsdp8_to_tp2", "etha_tile_kernel<true>", "run of buckets"): 16249517705,
-    # profiles/etha_reduce_kernel_partial4_to_shard2.txt
-    ("partial4_to_shard2", "etha_reduce_kernel", "run of buckets"): 5436000000,
-}
+TRAFFIC_FILE = os.path.join(ROOT, "profiles", "hbm_traffic.txt")
 
 
 def parse_args():
@@ -37,8 +29,14 @@ def parse_args():
     ap.add_argument("--steps", type=int, default=20)
     ap.add_argument("--warmup", type=int, default=3)
     ap.add_argument("--workload", default="llama3_8b_fsdp8_to_tp2")
-    ap.add_argument("--per-bucket", action="store_true", help="one launch per bucket instead of one per run of buckets")
-    ap.add_argument("--fanout", type=int, default=1, help="side streams for per-bucket launches (with --per-bucket)")
+    ap.add_argument("--pool", choices=["ring", "resident"], default="ring",
+                    help="ring: max-in-flight slots per channel (the reference's memory bound); resident: a slot per bucket")
+    ap.add_argument("--max-in-flight", type=int, default=2, help="buckets of one channel prepared or in flight (= ring slots)")
+    ap.add_argument("--per-bucket", action="store_true",
+                    help="strictly one launch per bucket (default: buckets that become ready together and are neighbours "
+                         "in their table share a launch)")
+    ap.add_argument("--in-order", action="store_true", help="issue every launch ordered after the previous one")
+    ap.add_argument("--fanout", type=int, default=1, help="side streams for per-bucket launches (resident pool only)")
     ap.add_argument("--zero-copy", action="store_true",
                     help="lend contiguous single-chunk buckets to the consumer instead of packing them")
     ap.add_argument("--direct", action="store_true",
@@ -46,10 +44,11 @@ def parse_args():
                          "not the pack+unpack path the headline is quoted on)")
     ap.add_argument("--graph", action="store_true", help="replay the step from a captured HIP graph (whole step timed)")
     ap.add_argument("--no-cpu-baseline", action="store_true")
-    ap.add_argument("--no-per-bucket-leg", action="store_true",
-                    help="skip the extra one-launch-per-bucket measurement after the timed region (use under a "
-                         "profiler, so that per-kernel statistics cover the timed configuration only)")
-    ap.add_argument("--cpu-layers", type=int, default=8, help="layers of the workload the CPU baseline sample covers")
+    ap.add_argument("--no-extra-legs", action="store_true",
+                    help="only the timed configuration (use under a profiler, so that per-kernel statistics cover one "
+                         "configuration)")
+    ap.add_argument("--cpu-layers", type=int, default=8,
+                    help="decoder layers of the sample the CPU baseline falls back to when host memory is short")
     ap.add_argument("--cpu-seconds", type=float, default=15.0, help="CPU work the baseline leg is bounded to")
     ap.add_argument("--calibration-copy", action="store_true",
                     help="after the timed region run three plain 1 GiB torch copies (known traffic, for scaling "
@@ -97,20 +96,36 @@ def gloo_baseline(workload: str, passes: int = 20):
     }
 
 
+def _host_memory_available() -> int:
+    try:
+        import psutil
+
+        return int(psutil.virtual_memory().available)
+    except Exception:
+        return 0
+
+
 def cpu_baseline(workload: str, layers: int, seconds: float):
-    """The oracle's op-for-op restatement of the reference path, timed on this host's cores."""
+    """The oracle's op-for-op restatement of the reference path, timed on this host's cores: the whole workload
+    where host memory allows (shards + target share + one pass of bucket buffers), else a sample of it."""
     import torch
 
     from etha_amd import workloads
     from etha_amd.world import ReshardJob
     from oracle import reference_path
 
-    if workload == "llama3_8b_fsdp8_to_tp2":
-        specs, targets, bucket = workloads.llama3_8b_fsdp8_to_tp2(n_layers=layers, with_embeddings=False)
-        sample = f"{layers} decoder layers of the workload (no embeddings), same layouts and 64 MiB buckets"
-    else:
-        specs, targets, bucket = workloads.WORKLOADS[workload]()
-        sample = "whole workload"
+    specs, targets, bucket = workloads.WORKLOADS[workload]()
+    sample = "whole workload"
+    if workload.startswith("llama3_8b_fsdp8_to_tp2"):
+        # the whole share: 16 GB of source shards + 8 GB of targets + 8 GB of bucket buffers alive during a pass
+        need = 48 << 30
+        have = _host_memory_available()
+        if have < need:
+            specs, targets, bucket = workloads.llama3_8b_fsdp8_to_tp2(n_layers=layers, with_embeddings=False)
+            sample = (f"{layers} decoder layers of the workload (no embeddings), same layouts and 64 MiB buckets - "
+                      f"host memory available {have >> 30} GiB < {need >> 30} GiB needed for the whole share")
+        else:
+            sample = "whole workload (embeddings included)"
 
     job = ReshardJob(specs, device="cpu", bucket_size=bucket, target_ranks=targets, fill=_cheap_fill)
     payload = job.payload_bytes()
@@ -136,10 +151,102 @@ def cpu_baseline(workload: str, layers: int, seconds: float):
         "unit": "GB/s",
         "cores": torch.get_num_threads(),
         "kind": "port",
-        "sample": f"{sample}; {payload} payload bytes per pass, median of {len(times)} passes "
+        "sample": f"{sample}; {payload} payload bytes per pass, median of {len(times)} passes after one warm-up "
                   f"({sum(times):.1f} s of CPU work)",
         "host_cpus": os.cpu_count(),
     }
+
+
+def read_traffic(workload: str, mode: str):
+    """HBM bytes per step of a workload from the committed counter summary (``profiles/hbm_traffic.txt``), with the
+    commit and command it was measured at.  Lines: ``workload | mode | fetch_bytes | write_bytes | launches | commit``."""
+    try:
+        with open(TRAFFIC_FILE) as f:
+            for line in f:
+                parts = [p.strip() for p in line.split("|")]
+                if len(parts) >= 6 and parts[0] == workload and parts[1] == mode:
+                    return {"fetch_bytes_per_step": int(parts[2]), "write_bytes_per_step": int(parts[3]),
+                            "launches_per_step": int(parts[4]), "measured_at_commit": parts[5],
+                            "source": "profiles/hbm_traffic.txt"}
+    except OSError:
+        pass
+    return None
+
+
+def _numel(shape):
+    n = 1
+    for d in shape:
+        n *= d
+    return n
+
+
+def algorithmic_bytes(job):
+    """(pack side bytes, unpack side bytes) per step: pack reads the source dtype (every member's partial for a
+    reduce-pack) and writes the wire dtype; unpack reads the wire dtype and writes the target dtype; a same-rank
+    chunk is one direct copy (read source region, write target region), counted with the pack side."""
+    send_plans = [job.wire.plan(b) for b in job.send_buckets.values()]
+    recv_plans = [job.wire.plan(b) for b in job.recv_buckets.values()]
+
+    def table_bytes(plan, which):
+        t = getattr(plan, which)
+        return t.info().payload_bytes if t is not None else 0
+
+    wire_bytes = sum(table_bytes(p, "send_table") for p in send_plans)
+    pack_read = self_bytes = 0
+    for p in send_plans:
+        for b in p.buckets:
+            if b.transport.value in ("p2p", "broadcast") and b.is_source and id(b) not in p.lent:
+                for c in b.chunks:
+                    peers = c.partial_peers()
+                    pack_read += _numel(c.chunk_shape) * c.tensor.element_size() * (len(peers[0]) if peers else 1)
+            elif b.transport.value == "local":
+                for c in b.chunks:
+                    src_t = c.src_tensor if c.src_tensor is not None else c.tensor
+                    self_bytes += _numel(c.chunk_shape) * (src_t.element_size() + c.tensor.element_size())
+    unpack_write = sum(_numel(c.chunk_shape) * c.tensor.element_size() for p in recv_plans for b in p.buckets for c in b.chunks)
+    unpack_read = sum(table_bytes(p, "recv_table") for p in recv_plans)
+    unpack_read += sum(p.direct_read_bytes for p in recv_plans)  # direct wire: reads the source regions themselves
+    kinds = {s[0] for p in send_plans + recv_plans for s in p.steps}
+    return pack_read + wire_bytes + self_bytes, unpack_read + unpack_write, self_bytes, kinds, pack_read == wire_bytes
+
+
+def time_steps(job, steps, run):
+    """Per-step device time (HIP events on the stream the launches go to) and wall time per step."""
+    import torch
+
+    stream = torch.cuda.current_stream(job.device)
+    ev = [torch.cuda.Event(enable_timing=True) for _ in range(steps + 1)]
+    # an untimed burst first: the first time steps queue up behind each other without a host synchronisation the
+    # HIP runtime grows its internal pools once (a host stall of tens of milliseconds)
+    for _ in range(min(steps, 5)):
+        run()
+    torch.cuda.synchronize()
+    import gc
+
+    gc.collect()
+    gc.disable()  # a full collection in the middle of the region stalls the host for tens of milliseconds
+    try:
+        wall0 = time.perf_counter()
+        ev[0].record(stream)
+        for k in range(steps):
+            run()
+            ev[k + 1].record(stream)
+        torch.cuda.synchronize()
+        wall = time.perf_counter() - wall0
+    finally:
+        gc.enable()
+    dev = [ev[k].elapsed_time(ev[k + 1]) for k in range(steps)]
+    return sum(dev) / steps, wall * 1e3 / steps
+
+
+def launches_per_step(job, run):
+    import torch
+
+    log = job.wire.launch_log = []
+    run()
+    torch.cuda.synchronize()
+    job.wire.launch_log = None
+    return len(log), sum(1 for entry in log if entry[3] & 1)
 
 
 def main():
@@ -162,113 +269,53 @@ def main():
     dev = torch.device("cuda:0")
     torch.cuda.set_device(dev)
     specs, targets, bucket = workloads.WORKLOADS[args.workload]()
-    t0 = time.time()
-    job = ReshardJob(specs, device=dev, bucket_size=bucket, target_ranks=targets, zero_copy=args.zero_copy,
-                     direct=args.direct)
     merge = not args.per_bucket
-    # plan (compiles the tile programs) + warm-up
-    for _ in range(max(args.warmup, 1)):
+    if args.fanout > 1 and args.pool != "resident":
+        print("--fanout needs --pool resident (side streams run a bucket list in list order)", file=sys.stderr)
+        sys.exit(2)
+
+    def make_job(pool, depth):
+        return ReshardJob(specs, device=dev, bucket_size=bucket, target_ranks=targets, zero_copy=args.zero_copy,
+                          direct=args.direct, pool=pool, max_in_flight=depth)
+
+    t0 = time.time()
+    job = make_job(args.pool, args.max_in_flight)
+    job.wire.unordered_launches = not args.in_order
+    for _ in range(max(args.warmup, 1)):  # plans (compiles the tile programs) + warm-up
         job.run(merge_launches=merge, fanout=args.fanout)
     setup_s = time.time() - t0
 
     S = job.payload_bytes()
-    send_plans = [job.wire.plan(b) for b in job.send_buckets.values()]
-    recv_plans = [job.wire.plan(b) for b in job.recv_buckets.values()]
-    steps_of = (lambda p: p.merged_steps) if merge else (lambda p: p.steps)
-    n_pack = sum(1 for p in send_plans for s in steps_of(p) if s[0] in ("pack", "reduce_pack"))
-    n_self = sum(1 for p in send_plans + recv_plans for s in steps_of(p) if s[0] == "selfcopy")
-    n_unpack = sum(1 for p in send_plans + recv_plans for s in steps_of(p) if s[0] in ("unpack", "direct", "direct_reduce"))
-
-    # algorithmic bytes: pack reads the source dtype and writes the wire dtype; unpack reads the wire
-    # dtype and writes the target dtype; a reduce-pack reads every member's partial
-    def table_bytes(plan, which):
-        t = getattr(plan, which)
-        return t.info().payload_bytes if t is not None else 0
-
-    wire_bytes = sum(table_bytes(p, "send_table") for p in send_plans)
-    pack_read = 0
-    for p in send_plans:
-        for b in p.buckets:
-            if b.transport.value in ("p2p", "broadcast") and b.is_source and id(b) not in p.lent:
-                for c in b.chunks:
-                    peers = c.partial_peers()
-                    n = 1
-                    for d in c.chunk_shape:
-                        n *= d
-                    pack_read += n * c.tensor.element_size() * (len(peers[0]) if peers else 1)
-    unpack_write = 0
-    for p in recv_plans:
-        for b in p.buckets:
-            for c in b.chunks:
-                n = 1
-                for d in c.chunk_shape:
-                    n *= d
-                unpack_write += n * c.tensor.element_size()
-    unpack_read = sum(table_bytes(p, "recv_table") for p in recv_plans)
-    unpack_read += sum(p.direct_read_bytes for p in recv_plans)  # direct wire: reads the source regions themselves
-    # LOCAL chunks run inside the send phase as direct copies: read the source region, write the target
-    self_bytes = 0
-    for p in send_plans:
-        for b in p.buckets:
-            if b.transport.value == "local":
-                for c in b.chunks:
-                    n = 1
-                    for d in c.chunk_shape:
-                        n *= d
-                    src_t = c.src_tensor if c.src_tensor is not None else c.tensor
-                    self_bytes += n * (src_t.element_size() + c.tensor.element_size())
-    pack_bytes = pack_read + wire_bytes + self_bytes
-    unpack_bytes = unpack_read + unpack_write
-
-    stream = torch.cuda.current_stream(dev)
-    ev = [[torch.cuda.Event(enable_timing=True) for _ in range(3)] for _ in range(args.steps)]
+    pack_bytes, unpack_bytes, self_bytes, kinds, byte_move = algorithmic_bytes(job)
+    total_bytes = pack_bytes + unpack_bytes
     graph = None
     if args.graph:
         graph = job.capture(merge_launches=merge)
         graph.replay()
-    torch.cuda.synchronize()
-    wall0 = time.perf_counter()
-    for k in range(args.steps):
-        ev[k][0].record(stream)
-        if graph is not None:
-            graph.replay()
-            ev[k][1].record(stream)
-        else:
-            job.run_send(merge, args.fanout)
-            ev[k][1].record(stream)
-            job.run_recv(merge, args.fanout)
-        ev[k][2].record(stream)
-    torch.cuda.synchronize()
-    wall = time.perf_counter() - wall0
-    pack_ms = [ev[k][0].elapsed_time(ev[k][1]) for k in range(args.steps)]
-    unpack_ms = [ev[k][1].elapsed_time(ev[k][2]) for k in range(args.steps)]
-    if graph is not None:  # a replayed graph is one unit: split the step time by algorithmic bytes
-        whole = [p + u for p, u in zip(pack_ms, unpack_ms)]
-        share = pack_bytes / max(pack_bytes + unpack_bytes, 1)
-        pack_ms = [w * share for w in whole]
-        unpack_ms = [w * (1 - share) for w in whole]
-    step_ms = wall * 1e3 / args.steps
-    pack_avg, unpack_avg = sum(pack_ms) / len(pack_ms), sum(unpack_ms) / len(unpack_ms)
-    dev_ms = pack_avg + unpack_avg
+    step = graph.replay if graph is not None else (lambda: job.run(merge_launches=merge, fanout=args.fanout, synchronize=False))
+    dev_ms, step_ms = time_steps(job, args.steps, step)
+    if args.pool == "ring":
+        n_launch, n_unordered = launches_per_step(job, lambda: job.run(merge_launches=merge, synchronize=False))
+    else:
+        plans = [job.wire.plan(b) for bs in (job.send_buckets, job.recv_buckets) for b in bs.values()]
+        n_launch = sum(1 for p in plans for s in (p.merged_steps if merge else p.steps) if s[0] != "lend")
+        n_unordered = 0
 
-    value = S / (step_ms * 1e-3) / 1e9
-    pack_gbs = pack_bytes / (pack_avg * 1e-3) / 1e9 if pack_avg > 0 else 0.0
-    unpack_gbs = unpack_bytes / (unpack_avg * 1e-3) / 1e9 if unpack_avg > 0 else 0.0
-    dominant = "pack" if pack_avg >= unpack_avg else "unpack"
-    dom_bytes, dom_ms, dom_launches = (
-        (pack_bytes, pack_avg, max(n_pack, 1)) if dominant == "pack" else (unpack_bytes, unpack_avg, max(n_unpack, 1))
-    )
-    kernel_name = {"pack": "etha_tile_kernel<false>", "unpack": "etha_tile_kernel<true>"}[dominant]
-    if dominant == "pack" and any(s[0] == "reduce_pack" for p in send_plans for s in steps_of(p)):
-        kernel_name = "etha_reduce_kernel"
-    if dominant == "unpack" and args.direct:
-        kernel_name = "etha_tile_kernel<false>"  # the direct copy runs source region -> target region
-        if any(s[0] == "direct_reduce" for p in recv_plans for s in steps_of(p)):
-            kernel_name = "etha_reduce_kernel"
-    achieved = dom_bytes / (dom_ms * 1e-3) / 1e9
+    kernels = []
+    if kinds & {"pack", "unpack", "selfcopy", "direct"}:
+        kernels.append("etha_tile_kernel")
+    if kinds & {"reduce_pack", "direct_reduce"}:
+        kernels.insert(0, "etha_reduce_kernel")
+    granularity = ("bucket" if not merge else
+                   "buckets ready together" if args.pool == "ring" else "run of buckets")
+    mode = f"{args.pool}/{'bucket' if not merge else 'runs'}"
+    element = str(specs[0].source_dtype).replace("torch.", "")
+    achieved = total_bytes / (dev_ms * 1e-3) / 1e9
+    traffic = None if (args.zero_copy or args.direct or args.graph or args.fanout > 1 or args.in_order
+                       or args.max_in_flight != 2) else read_traffic(args.workload, mode)
     out = {
         "metric": "effective reshard GB/s (pack+unpack, 1 GPU) and % of HBM peak",
-        "value": round(value, 2),
+        "value": round(S / (step_ms * 1e-3) / 1e9, 2),
         "unit": "GB/s",
         "n_gpus": 1,
         "steps": args.steps,
@@ -277,13 +324,17 @@ def main():
         "higher_is_better": True,
         "scaling": "weak",
         "vs_baseline": None,
-        "dtype": "u8" if pack_read == wire_bytes else "f32",
+        "dtype": f"{element} (byte move)" if byte_move else f"{element} -> wire dtype (f32 arithmetic)",
         "data": "synthetic",
         "config": {
             "workload": args.workload,
             "payload_bytes": S,
             "bucket_bytes": bucket,
-            "launch_granularity": "run of buckets" if merge else "bucket",
+            "pool": args.pool,
+            "max_in_flight": args.max_in_flight,
+            "pool_reserved_bytes": job.wire.pool.reserved_bytes if job.wire.pool is not None else 0,
+            "launch_granularity": granularity,
+            "unordered_launches": bool(job.wire.unordered_launches and args.pool == "ring"),
             "fanout_streams": args.fanout,
             "hip_graph": bool(args.graph),
             "zero_copy_single_chunk": bool(args.zero_copy),
@@ -291,45 +342,88 @@ def main():
             **job.counts(),
         },
         "device_ms_per_step": round(dev_ms, 4),
-        "pct_of_hbm_peak": round(100.0 * (pack_bytes + unpack_bytes) / (dev_ms * 1e-3) / 1e9 / HBM_PEAK_GBS, 2),
-        "pack": {"GB/s": round(pack_gbs, 1), "ms": round(pack_avg, 4), "bytes": pack_bytes, "launches": n_pack},
-        "unpack": {"GB/s": round(unpack_gbs, 1), "ms": round(unpack_avg, 4), "bytes": unpack_bytes, "launches": n_unpack},
-        "selfcopy": {"launches": n_self, "bytes": self_bytes, "note": "timed inside the pack phase"},
+        "pct_of_hbm_peak": round(100.0 * achieved / HBM_PEAK_GBS, 2),
+        "algorithmic_bytes_per_step": {"pack": pack_bytes, "unpack": unpack_bytes, "of_which_self_copy": self_bytes},
+        "launches_per_step": n_launch,
+        "unordered_launches_per_step": n_unordered,
         "roofline": {
             "bound": "hbm",
-            "kernel": kernel_name,
+            "kernel": " + ".join(kernels),
             "achieved": round(achieved, 1),
             "peak": HBM_PEAK_GBS,
             "unit": "GB/s",
             "frac": round(achieved / HBM_PEAK_GBS, 4),
-            # measured for the default configuration only
-            "traffic": None if (args.zero_copy or args.direct or args.graph or args.fanout > 1) else
-            MEASURED_TRAFFIC_BYTES.get((args.workload, kernel_name, "run of buckets" if merge else "bucket")),
-            "bytes_per_launch": dom_bytes // dom_launches,
-            "avg_launch_ms": round(dom_ms / dom_launches, 5),
-            "launches_per_step": dom_launches,
+            # HBM bytes per launch from the committed rocprofv3 counter summary (null when this configuration has none)
+            "traffic": None if traffic is None else
+            (traffic["fetch_bytes_per_step"] + traffic["write_bytes_per_step"]) // max(traffic["launches_per_step"], 1),
+            "traffic_detail": traffic,
+            "bytes_per_launch": total_bytes // max(n_launch, 1),
+            # launches overlap their neighbours: the average is the timed region over the launches in it
+            "avg_launch_ms": round(dev_ms / max(n_launch, 1), 5),
+            "launches_per_step": n_launch,
         },
         "setup_s": round(setup_s, 1),
     }
-    if merge and graph is None and args.fanout == 1 and not args.no_per_bucket_leg:
-        # the strict form of the same step, one launch per bucket, for comparison (not the headline)
-        n_strict = sum(1 for p in send_plans + recv_plans for s in p.steps if s[0] != "lend")
+
+    def leg(j, reps=None, **kw):
+        reps = reps or max(3, min(args.steps, 10))
         for _ in range(2):
-            job.run(merge_launches=False)
-        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+            j.run(**kw)
+        ms, _ = time_steps(j, reps, lambda: j.run(synchronize=False, **kw))
+        return ms
+
+    def describe(ms, launches=None, pool_bytes=None):
+        d = {"device_ms_per_step": round(ms, 4),
+             "pct_of_hbm_peak": round(100.0 * total_bytes / (ms * 1e-3) / 1e9 / HBM_PEAK_GBS, 2),
+             "effective_GB/s": round(S / (ms * 1e-3) / 1e9, 1)}
+        if launches is not None:
+            d["launches_per_step"] = launches
+        if pool_bytes is not None:
+            d["pool_reserved_bytes"] = pool_bytes
+        return d
+
+    plain = not (args.no_extra_legs or args.graph or args.fanout > 1 or args.zero_copy or args.direct or args.in_order)
+    if plain and args.pool == "ring":
+        # the same step in its other forms, for comparison (none of them is `value`)
+        pool_bytes = job.wire.pool.reserved_bytes if job.wire.pool is not None else 0
+        other = not merge
+        ms = leg(job, merge_launches=other)
+        n, _ = launches_per_step(job, lambda: job.run(merge_launches=other, synchronize=False))
+        out["one_launch_per_bucket" if merge else "buckets_ready_together"] = describe(ms, n, pool_bytes)
+        job.wire.unordered_launches = False
+        out["every_launch_in_order"] = describe(leg(job, merge_launches=merge), n_launch, pool_bytes)
+        job.wire.unordered_launches = True
+        del job
+        torch.cuda.empty_cache()
+        deeper = make_job("ring", 2 * args.max_in_flight)
+        ms = leg(deeper, merge_launches=merge)
+        n, _ = launches_per_step(deeper, lambda: deeper.run(merge_launches=merge, synchronize=False))
+        out[f"ring_of_{2 * args.max_in_flight}_slots"] = describe(ms, n, deeper.wire.pool.reserved_bytes if deeper.wire.pool else 0)
+        del deeper
+        torch.cuda.empty_cache()
+        # a slot per bucket: all packs, then all unpacks, each side in as few launches as the lists allow
+        res = make_job("resident", args.max_in_flight)
+        for _ in range(2):
+            res.run(merge_launches=True)
+        stream = torch.cuda.current_stream(dev)
         reps = max(3, min(args.steps, 10))
-        e0.record(stream)
-        for _ in range(reps):
-            job.run(merge_launches=False, synchronize=False)
-        e1.record(stream)
+        ev = [[torch.cuda.Event(enable_timing=True) for _ in range(3)] for _ in range(reps)]
+        for k in range(reps):
+            ev[k][0].record(stream)
+            res.run_send(True)
+            ev[k][1].record(stream)
+            res.run_recv(True)
+            ev[k][2].record(stream)
         torch.cuda.synchronize()
-        strict_ms = e0.elapsed_time(e1) / reps
-        out["one_launch_per_bucket"] = {
-            "device_ms_per_step": round(strict_ms, 4),
-            "pct_of_hbm_peak": round(100.0 * (pack_bytes + unpack_bytes) / (strict_ms * 1e-3) / 1e9 / HBM_PEAK_GBS, 2),
-            "launches_per_step": n_strict,
-            "effective_GB/s": round(S / (strict_ms * 1e-3) / 1e9, 1),
-        }
+        p_ms = sum(e[0].elapsed_time(e[1]) for e in ev) / reps
+        u_ms = sum(e[1].elapsed_time(e[2]) for e in ev) / reps
+        plans = [res.wire.plan(b) for bs in (res.send_buckets, res.recv_buckets) for b in bs.values()]
+        d = describe(p_ms + u_ms, sum(1 for p in plans for s in p.merged_steps if s[0] != "lend"), res.wire.pool.reserved_bytes)
+        d["pack"] = {"GB/s": round(pack_bytes / (p_ms * 1e-3) / 1e9, 1), "ms": round(p_ms, 4)}
+        d["unpack"] = {"GB/s": round(unpack_bytes / (u_ms * 1e-3) / 1e9, 1), "ms": round(u_ms, 4)}
+        out["resident_pool_run_of_buckets"] = d
+        del res
+        torch.cuda.empty_cache()
     if args.calibration_copy:
         a = torch.empty(1 << 30, dtype=torch.uint8, device=dev).fill_(1)
         b = torch.empty(1 << 30, dtype=torch.uint8, device=dev)

@@ -14,7 +14,8 @@ import numpy as np
 from .build import LIB_PATH
 
 ETHA_MAX_NDIM = 8
-ABI_VERSION = 3
+ABI_VERSION = 4
+LAUNCH_UNORDERED = 1  # ETHA_LAUNCH_UNORDERED
 
 # element type codes (include/etha_reshard.h)
 F16, BF16, F32, F64, B8, B16, B32, B64 = range(8)
@@ -106,10 +107,10 @@ _SIGNATURES = {
     "etha_table_read_trans_ranges": (c_int, [c_void_p, c_void_p]),
     "etha_table_optimize_range": (c_int, [c_void_p, c_uint32, c_uint32]),
     "etha_table_read_ordered": (c_int, [c_void_p, c_uint32, c_uint32, c_int, c_void_p, c_uint64, POINTER(c_uint64)]),
-    "etha_pack_bucket": (c_int, [c_void_p, c_uint32, c_uint32, c_void_p]),
-    "etha_unpack_bucket": (c_int, [c_void_p, c_uint32, c_uint32, c_void_p]),
-    "etha_reduce_pack_bucket": (c_int, [c_void_p, c_uint32, c_uint32, c_void_p]),
-    "etha_selfcopy_bucket": (c_int, [c_void_p, c_uint32, c_uint32, c_void_p]),
+    "etha_pack_bucket": (c_int, [c_void_p, c_uint32, c_uint32, c_void_p, c_uint32]),
+    "etha_unpack_bucket": (c_int, [c_void_p, c_uint32, c_uint32, c_void_p, c_uint32]),
+    "etha_reduce_pack_bucket": (c_int, [c_void_p, c_uint32, c_uint32, c_void_p, c_uint32]),
+    "etha_selfcopy_bucket": (c_int, [c_void_p, c_uint32, c_uint32, c_void_p, c_uint32]),
     "etha_arena_create": (c_int, [c_uint64, POINTER(c_void_p)]),
     "etha_arena_destroy": (c_int, [c_void_p]),
     "etha_ipc_export": (c_int, [c_void_p, POINTER(IpcHandle)]),
@@ -249,17 +250,17 @@ class Table:
             res.append(arr)
         return res[0], res[1]
 
-    def pack(self, first: int, count: int, stream: int = 0) -> None:
-        _check("etha_pack_bucket", lib().etha_pack_bucket(self._h, first, count, c_void_p(stream)))
+    def pack(self, first: int, count: int, stream: int = 0, flags: int = 0) -> None:
+        _check("etha_pack_bucket", lib().etha_pack_bucket(self._h, first, count, c_void_p(stream), flags))
 
-    def unpack(self, first: int, count: int, stream: int = 0) -> None:
-        _check("etha_unpack_bucket", lib().etha_unpack_bucket(self._h, first, count, c_void_p(stream)))
+    def unpack(self, first: int, count: int, stream: int = 0, flags: int = 0) -> None:
+        _check("etha_unpack_bucket", lib().etha_unpack_bucket(self._h, first, count, c_void_p(stream), flags))
 
-    def reduce_pack(self, first: int, count: int, stream: int = 0) -> None:
-        _check("etha_reduce_pack_bucket", lib().etha_reduce_pack_bucket(self._h, first, count, c_void_p(stream)))
+    def reduce_pack(self, first: int, count: int, stream: int = 0, flags: int = 0) -> None:
+        _check("etha_reduce_pack_bucket", lib().etha_reduce_pack_bucket(self._h, first, count, c_void_p(stream), flags))
 
-    def selfcopy(self, first: int, count: int, stream: int = 0) -> None:
-        _check("etha_selfcopy_bucket", lib().etha_selfcopy_bucket(self._h, first, count, c_void_p(stream)))
+    def selfcopy(self, first: int, count: int, stream: int = 0, flags: int = 0) -> None:
+        _check("etha_selfcopy_bucket", lib().etha_selfcopy_bucket(self._h, first, count, c_void_p(stream), flags))
 
     def close(self) -> None:
         if self._h:

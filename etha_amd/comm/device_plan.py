@@ -83,9 +83,9 @@ def fill_region(row, tensor: torch.Tensor, slices: tuple, chunk_shape: tuple) ->
     row["tensor_dtype"] = dtype_code(tensor.dtype)
 
 
-@dataclass
+@dataclass(eq=False)
 class Slot:
-    """A bucket buffer inside the pool."""
+    """A bucket buffer inside the pool.  In a ring pool one slot serves every ``depth``-th bucket of its channel."""
 
     ptr: int
     nbytes: int
@@ -98,6 +98,9 @@ class Slot:
     # direct wire: per chunk of the send bucket ``(source tensor, src_slice, wire dtype, Partial peers or None)``;
     # the consumer copies from these regions straight into its own tensors and no bucket buffer exists (ptr is 0)
     sources: list | None = None
+    # the send bucket (a wire entry) whose bytes are in the slot and have not been read by all of its
+    # consumers yet; None = free.  A ring slot is packed again only when it is free.
+    holder: object = None
 
 
 def _rows_to_array(rows: list[np.ndarray]) -> np.ndarray:

@@ -250,7 +250,24 @@ class Bucket:
         (``Bucket.launch``, ``ir.py:266-284``)."""
         return True
 
-    def is_complete(self) -> bool:
+    def is_complete(self, wire=None) -> bool:
+        """Source bucket on a ring pool: every destination has unpacked it (its slot is free again).  Target
+        bucket on a ring pool: its send bucket has been packed.  Otherwise always True
+        (``Bucket.is_complete``, ``ir.py:286-298``)."""
+        from .comm_methods import recv_may_start
+
+        plan = self._plan(wire)
+        if plan.wire.pool_mode != "ring":
+            return True
+        for i in plan.steps_of.get(id(self), ()):
+            entry, kind = plan.info[i].entry, plan.steps[i][0]
+            if entry is None:
+                continue
+            if kind in ("unpack", "direct", "direct_reduce"):
+                if not recv_may_start(entry, self.rank):
+                    return False
+            elif entry.left:
+                return False
         return True
 
     def finalize(self, wire=None) -> None:

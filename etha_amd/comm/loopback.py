@@ -7,6 +7,18 @@ of a persistent bucket pool, the consumer unpacks from the very same slot (zero 
 assigned when a bucket list is first planned and reused by every later transfer, so the
 consumer's tile program can hold absolute addresses.
 
+Pool.  By default the pool is a **ring**: every wire key (channel) of a planned send list owns
+``max_in_flight`` slots, each as large as the channel's largest bucket, and the channel's k-th bucket
+uses slot ``k mod max_in_flight``.  That is the reference's memory bound - at most ``max_in_flight``
+buckets per channel are prepared or in flight, and a bucket's buffer is dropped at ``finalize``
+(``comm_methods.py:53-119``, ``ir.py:246,310``).  A slot is packed again only after every consumer of
+its previous bucket has unpacked, so senders and receivers advance together: the wire keeps the bucket
+pipelines (:class:`etha_amd.comm.comm_methods.Program`) of every rank that has called ``bucket_comm``
+and steps them in turn, the single-process form of the ranks' concurrent ``bucket_comm`` loops.
+``pool="resident"`` gives every bucket a slot of its own for the life of its plan (pool = payload);
+that form allows one launch over many buckets, side streams, graph capture and exporting the pool to
+another process.
+
 Matching follows the point-to-point rule of the reference's transports: the k-th bucket a rank
 sends on a wire key ``(src_rank, dst_ranks, transport)`` is the k-th bucket each of its peers
 receives on that key.  Because slots are assigned when bucket lists are *planned*, "k-th" counts
@@ -19,6 +31,7 @@ numbers are then counted per scope.
 from __future__ import annotations
 
 from collections import defaultdict
+from dataclasses import dataclass, field
 
 import torch
 
@@ -37,13 +50,14 @@ class BucketPool:
 
     def __init__(self, device: torch.device, segment_bytes: int = 1 << 30):
         self.device = device
-        self.segment_bytes = segment_bytes
+        self.segment_bytes = segment_bytes  # 0: every slot is an allocation of its own, exactly as large as asked
         self.segments: list[torch.Tensor] = []
         self._cursor = 0  # offset inside the last segment
         self._free: dict[int, list[Slot]] = {}  # released slots, reused for requests of exactly their size
 
     def release(self, slot: Slot) -> None:
         slot.filled = slot.drained = 0
+        slot.holder = None
         self._free.setdefault(slot.nbytes, []).append(slot)
 
     def alloc(self, nbytes: int) -> Slot:
@@ -51,6 +65,10 @@ class BucketPool:
         if free:
             return free.pop()
         need = max(nbytes, 1)
+        if self.segment_bytes == 0:
+            seg = torch.empty(-(-need // _SLOT_ALIGN) * _SLOT_ALIGN, dtype=torch.uint8, device=self.device)
+            self.segments.append(seg)
+            return Slot(ptr=seg.data_ptr(), nbytes=nbytes, lo=seg.data_ptr(), hi=seg.data_ptr() + seg.numel())
         if need > self.segment_bytes or not self.segments or self._cursor + need > self.segments[-1].numel():
             size = max(self.segment_bytes, need)
             self.segments.append(torch.empty(size, dtype=torch.uint8, device=self.device))
@@ -73,6 +91,29 @@ class BucketPool:
         return sum(s.numel() for s in self.segments)
 
 
+@dataclass(eq=False)
+class WireEntry:
+    """One planned send bucket on a wire key: where its bytes travel and who still has to read them."""
+
+    key: tuple
+    seq: int
+    slot: Slot
+    sizes: tuple
+    dst_ranks: tuple
+    submitted: int = 0  # transfers the sender has been asked for
+    packed: int = 0  # transfers packed into the slot so far
+    arrived: dict = field(default_factory=dict)  # destination rank -> transfers it has asked for
+    left: set = field(default_factory=set)  # consumers of the bytes now in the slot that have not unpacked yet
+
+
+class _no_context:
+    def __enter__(self):
+        return None
+
+    def __exit__(self, *exc):
+        return False
+
+
 def wire_key(bucket: Bucket) -> tuple:
     return (bucket.src_rank, tuple(bucket.dst_ranks), bucket.transport.value)
 
@@ -81,9 +122,29 @@ class LoopbackWire:
     """Process-wide stand-in for the process groups of the reference's executor."""
 
     def __init__(self, device: torch.device | str | None = None, segment_bytes: int = 1 << 30,
-                 host_inspection: bool = False):
+                 host_inspection: bool = False, pool: str = "ring", max_in_flight: int = 2):
+        if pool not in ("ring", "resident"):
+            raise ValueError(f"pool must be 'ring' or 'resident', got {pool!r}")
         self.device = torch.device(device) if device is not None else None
         self.segment_bytes = segment_bytes
+        self.pool_mode = pool
+        # slots per channel of a ring pool; a plan's rings are sized when it is first compiled
+        self.max_in_flight = max(1, int(max_in_flight))
+        # destination ranks that buckets name but that do not exist on this wire (a job that only stages some
+        # target ranks): nobody will unpack for them, so a slot does not wait for them
+        self.absent_ranks: set[int] = set()
+        # launches that do not depend on each other are issued without ordering between them
+        # (ETHA_LAUNCH_UNORDERED), which hides the gap between one bucket's kernel and the next one's
+        self.unordered_launches = True
+        # host inspection: called as ``on_launch(plan, kind, first, count, flags)`` instead of launching
+        self.on_launch = None
+        self.launch_log: list | None = None  # when a list: (kind, first, count, flags) of every launch
+        self._programs: list = []  # bucket pipelines that still have work, in arrival order
+        self._epoch_reads: set[int] = set()  # allocations read / written by launches since the last ordered one
+        self._epoch_writes: set[int] = set()
+        self._ordered_next = True
+        self._stream = None
+        self._carried = False  # pipelines were left pending by an earlier drive (their launches sit on _stream)
         # True: bucket lists on host tensors may be *planned* (tile programs compiled against host
         # addresses, for checking them on the CPU); they still cannot be run
         self.host_inspection = host_inspection
@@ -109,14 +170,34 @@ class LoopbackWire:
     def _pool_for(self, device: torch.device) -> BucketPool:
         if self.pool is None:
             self.device = self.device or device
-            self.pool = BucketPool(self.device, self.segment_bytes)
+            self.pool = BucketPool(self.device, 0 if self.pool_mode == "ring" else self.segment_bytes)
         if device != self.pool.device:
             raise RuntimeError(f"loopback wire is bound to {self.pool.device}, got a bucket on {device}")
         return self.pool
 
     # -- plan-time rendezvous -------------------------------------------------------------------
-    def slot_for_send(self, bucket: Bucket, device: torch.device, scope=None) -> Slot:
-        """Assign the next sequence number on this bucket's wire key (within ``scope``) and a slot to go with it."""
+    def open_rings(self, buckets: list[Bucket], device: torch.device, depth: int) -> dict:
+        """Ring pool: the slots of one send list, ``{wire key: [slot, ...]}``.  A channel gets ``depth`` slots
+        (fewer if it has fewer buckets) of its largest bucket's size."""
+        need: dict[tuple, list[int]] = {}
+        for b in buckets:
+            if not b.chunks or not b.is_source or b.transport.value not in ("p2p", "broadcast"):
+                continue
+            if self.direct_same_device:
+                continue
+            if self.zero_copy_single_chunk:
+                from .device_plan import zero_copy_region
+
+                if zero_copy_region(b) is not None:
+                    continue
+            need.setdefault(wire_key(b), []).append(b.total_bytes)
+        pool = self._pool_for(device) if need else None
+        return {key: [pool.alloc(max(sizes)) for _ in range(min(depth, len(sizes)))] for key, sizes in need.items()}
+
+    def entry_for_send(self, bucket: Bucket, device: torch.device, scope=None, ring: list | None = None,
+                       ordinal: int = 0) -> WireEntry:
+        """Assign the next sequence number on this bucket's wire key (within ``scope``) and a slot to go with it:
+        slot ``ordinal mod depth`` of ``ring`` in a ring pool, else a slot of the bucket's own."""
         key = (scope, *wire_key(bucket))
         sizes = tuple(c.nbytes for c in bucket.chunks)
         slot = None
@@ -134,15 +215,18 @@ class LoopbackWire:
                 self._pool_for(device)
                 slot = Slot(ptr=region[0], nbytes=bucket.total_bytes, lo=region[1], hi=region[2], borrowed=True)
                 slot.keepalive = region[3]
+        if slot is None and ring:
+            slot = ring[ordinal % len(ring)]
         if slot is None:
             slot = self._pool_for(device).alloc(bucket.total_bytes)
         seq = self._send_seq[key]
         self._send_seq[key] = seq + 1
-        self._sent[key][seq] = (slot, sizes)
-        return slot
+        entry = WireEntry(key=key, seq=seq, slot=slot, sizes=sizes, dst_ranks=tuple(bucket.dst_ranks))
+        self._sent[key][seq] = entry
+        return entry
 
-    def slot_for_recv(self, bucket: Bucket, scope=None) -> Slot:
-        """Slot of the send bucket this receive bucket pairs with: the next one its rank has not yet planned."""
+    def entry_for_recv(self, bucket: Bucket, scope=None) -> WireEntry:
+        """The send bucket this receive bucket pairs with: the next one on its key that its rank has not yet planned."""
         key = (scope, *wire_key(bucket))
         who = (key, bucket.rank)
         seq = self._recv_seq[who]
@@ -152,11 +236,13 @@ class LoopbackWire:
                 f"{bucket}: no matching send bucket #{seq} has been planned on this wire "
                 "(plan/run the source side first; a real wire would deadlock here)"
             )
-        slot, sizes = entry
-        if sizes != tuple(c.nbytes for c in bucket.chunks):
+        if entry.sizes != tuple(c.nbytes for c in bucket.chunks):
             raise RuntimeError(f"{bucket}: chunk layout differs from the matching send bucket")
         self._recv_seq[who] = seq + 1
-        return slot
+        return entry
+
+    def consumers(self, entry: WireEntry) -> set:
+        return {r for r in entry.dst_ranks if r not in self.absent_ranks}
 
     # -- across processes ----------------------------------------------------------------------
     def export_manifest(self) -> dict:
@@ -168,6 +254,10 @@ class LoopbackWire:
         """
         from .. import _native as nat
 
+        if self.pool_mode != "resident":
+            raise NotImplementedError(
+                "a ring pool is recycled under a hand-shake that only exists inside one process; "
+                "export needs LoopbackWire(pool='resident')")
         if self.pool is None:
             return {"device": None, "segments": [], "slots": {}}
         segments = []
@@ -177,7 +267,8 @@ class LoopbackWire:
         slots: dict = {}
         for key, entries in self._sent.items():
             out = []
-            for seq, (slot, sizes) in sorted(entries.items()):
+            for seq, entry in sorted(entries.items()):
+                slot, sizes = entry.slot, entry.sizes
                 if slot.sources is not None:
                     raise NotImplementedError("a direct wire has no bucket buffers to export; it works inside one process")
                 if slot.borrowed:  # lives in a source tensor: export that allocation, range = the slot itself
@@ -198,7 +289,7 @@ class LoopbackWire:
         from .. import _native as nat
 
         dev = torch.device(device) if device is not None else torch.device("cuda", manifest["device"] or 0)
-        wire = cls(dev)
+        wire = cls(dev, pool="resident")
         wire._imported = []
         bases = []
         with torch.cuda.device(dev):
@@ -210,15 +301,16 @@ class LoopbackWire:
             for e in entries:
                 base, nbytes = bases[e["segment"]]
                 slot = Slot(ptr=base + e["offset"], nbytes=e["nbytes"], lo=base, hi=base + nbytes)
-                wire._sent[key][e["seq"]] = (slot, tuple(e["sizes"]))
+                wire._sent[key][e["seq"]] = WireEntry(key=key, seq=e["seq"], slot=slot, sizes=tuple(e["sizes"]),
+                                                      dst_ranks=tuple(key[2]))
         return wire
 
     def mark_packed(self) -> None:
         """Consumer side: the producer reported that every exported slot has been packed (and its stream
         synchronised) once more."""
         for entries in self._sent.values():
-            for slot, _ in entries.values():
-                slot.filled += 1
+            for entry in entries.values():
+                entry.slot.filled += 1
 
     def close_imported(self) -> None:
         from .. import _native as nat
@@ -237,35 +329,31 @@ class LoopbackWire:
         return self._side_streams[:n]
 
     # -- plan cache -----------------------------------------------------------------------------
-    def plan(self, buckets: list[Bucket], scope=None):
-        """Compiled plan of a bucket list (cached by the identity of its buckets).  ``scope`` only matters when the
-        plan is first built: it namespaces the send/receive pairing."""
+    def plan(self, buckets: list[Bucket], scope=None, max_in_flight: int | None = None):
+        """Compiled plan of a bucket list (cached by the identity of its buckets).  ``scope`` and ``max_in_flight``
+        only matter when the plan is first built: the scope namespaces the send/receive pairing, and a ring pool
+        gives every channel of the list ``max_in_flight`` slots (default: the wire's)."""
         from .comm_methods import TransferPlan
 
         key = tuple(id(b) for b in buckets)
         plan = self._plans.get(key)
         if plan is None:
-            plan = TransferPlan(self, list(buckets), scope=scope)
+            plan = TransferPlan(self, list(buckets), scope=scope, max_in_flight=max_in_flight or self.max_in_flight)
             self._plans[key] = plan
         return plan
 
     def release(self, buckets: list[Bucket]) -> None:
-        """Forget a bucket list: drop its compiled plan and hand its send slots back to the pool.
+        """Forget a bucket list: drop its compiled plan and hand its slots back to the pool.
         The caller guarantees that no transfer of these buckets, on either end, is still in flight."""
         plan = self._plans.pop(tuple(id(b) for b in buckets), None)
         if plan is None:
             return
-        for kind, _, _, slot in plan.steps:
-            if slot is None or self.pool is None:
-                continue
-            owned = False
-            for key, entries in list(self._sent.items()):
-                mine = [seq for seq, (s, _) in entries.items() if s is slot]
-                for seq in mine:  # sequence numbers are never reused: later plans on this key keep theirs
-                    del entries[seq]
-                    owned = True
-            if (owned or kind == "pack") and not slot.borrowed:
-                if not any(slot is s for s in self.pool._free.get(slot.nbytes, [])):
+        self._programs = [p for p in self._programs if p.plan is not plan]
+        for entry in plan.owned_entries:  # sequence numbers are never reused: later plans on this key keep theirs
+            self._sent.get(entry.key, {}).pop(entry.seq, None)
+        if self.pool is not None:
+            for slot in plan.owned_slots:
+                if not slot.borrowed and not any(slot is s for s in self.pool._free.get(slot.nbytes, [])):
                     self.pool.release(slot)
 
     def reset(self) -> None:
@@ -273,7 +361,114 @@ class LoopbackWire:
         self._sent.clear()
         self._send_seq.clear()
         self._recv_seq.clear()
+        self._programs.clear()
         self.pool = None
+
+    # -- the bucket pipelines of every rank on this wire ---------------------------------------
+    def submit(self, plan, max_in_flight: int, merge_launches: bool = False):
+        """Start one transfer of a planned bucket list: its pipeline joins the ones :meth:`drive` steps."""
+        from .comm_methods import Program
+
+        if any(p.plan is plan for p in self._programs):
+            raise RuntimeError(
+                "the previous transfer of these buckets has not completed: its receivers have not unpacked yet "
+                "(a real wire would block here)")
+        program = Program(plan, max_in_flight, merge_launches)
+        self._programs.append(program)
+        return program
+
+    def drive(self) -> None:
+        """Step every pending pipeline, in arrival order, until none can move.  Launches go to the current stream
+        of the wire's device.  A sender's pipeline that is waiting for its receivers stays pending and is picked
+        up by the call that brings them."""
+        if not self._programs:
+            return
+        cuda = self.device is not None and self.device.type == "cuda" and self.on_launch is None
+        if cuda:
+            stream = torch.cuda.current_stream(self.device)
+            if self._carried and self._stream is not None and self._stream != stream:
+                # work enqueued earlier for pipelines that are still pending sits on another stream
+                done = torch.cuda.Event()
+                done.record(self._stream)
+                stream.wait_event(done)
+            self._stream = stream
+        # whatever is on the stream already (the caller's own kernels) must be finished before the first launch
+        self._ordered_next = True
+        self._epoch_reads, self._epoch_writes = set(), set()
+        with torch.cuda.device(self.device) if cuda else _no_context():
+            moved = True
+            while moved:
+                moved = False
+                for program in list(self._programs):
+                    if program.sweep(self):
+                        moved = True
+                    if program.finished:
+                        self._programs.remove(program)
+        self._carried = bool(self._programs)
+
+    def idle(self) -> bool:
+        """True when no pipeline is waiting for a peer."""
+        return not self._programs
+
+    def in_progress(self, buckets: list[Bucket]) -> bool:
+        """True while a transfer of this bucket list is still waiting for a peer (a send whose receivers have
+        not all unpacked, a receive whose senders have not packed everything yet)."""
+        plan = self._plans.get(tuple(id(b) for b in buckets))
+        return plan is not None and any(p.plan is plan for p in self._programs)
+
+    def pending(self) -> list[str]:
+        return [repr(p) for p in self._programs]
+
+    def emit(self, plan, indices: list[int], merge: bool = False) -> None:
+        """Issue steps ``indices`` of ``plan``.  They became ready in the same phase of one pipeline sweep, so they
+        are independent of each other; with ``merge`` those that are neighbours in their table share a launch.
+        Each launch is ordered against earlier launches only where their bytes meet."""
+        todo = []
+        for i in indices:
+            kind, first, count, _ = plan.steps[i]
+            info = plan.info[i]
+            if info.tiles:  # else nothing to move (empty shards): no launch, so nothing that could order later launches
+                todo.append([kind, first, count, info.reads, info.writes, info.excl])
+        if merge and len(todo) > 1:
+            todo.sort(key=lambda t: (t[0], t[1]))
+            runs = [todo[0]]
+            for t in todo[1:]:
+                last = runs[-1]
+                if t[0] == last[0] and last[1] + last[2] == t[1]:
+                    last[2] += t[2]
+                    last[3], last[4], last[5] = last[3] | t[3], last[4] | t[4], last[5] | t[5]
+                    last.append(True)  # covers several buckets
+                else:
+                    runs.append(t)
+            todo = runs
+            for t in todo:
+                if len(t) > 6:
+                    plan.order_by_written_address(t[0], t[1], t[2])
+        for kind, first, count, reads, writes, excl, *_ in todo:
+            self._issue(plan, kind, first, count, reads, writes, excl)
+
+    def _issue(self, plan, kind, first, count, reads, writes, excl) -> None:
+        ordered = (self._ordered_next or not self.unordered_launches or not self._epoch_writes.isdisjoint(reads)
+                   or not self._epoch_reads.isdisjoint(writes) or not self._epoch_writes.isdisjoint(excl))
+        if not ordered and self.on_launch is None and torch.cuda.is_current_stream_capturing():
+            ordered = True  # a captured stream records its launches as a chain anyway
+        if ordered:
+            self._epoch_reads, self._epoch_writes = set(reads), set(writes)
+        else:
+            self._epoch_reads |= reads
+            self._epoch_writes |= writes
+        self._ordered_next = False
+        from .. import _native as nat
+
+        flags = 0 if ordered else nat.LAUNCH_UNORDERED
+        if self.launch_log is not None:
+            self.launch_log.append((kind, first, count, flags))
+        if self.on_launch is not None:
+            self.on_launch(plan, kind, first, count, flags)
+            return
+        if plan.device is None or plan.device.type != "cuda":
+            raise RuntimeError("this plan was compiled for host inspection; the executor only runs on a GPU (there is no CPU path)")
+        plan.launch_step(kind, first, count, self._stream.cuda_stream, flags)
 
 
 _default_wire: LoopbackWire | None = None

@@ -13,6 +13,7 @@
 // Bucket.prepare / Chunk.finalize / Bucket.finalize (src/etha/comm/ir.py:101-141, 229-264,
 // 300-310) - slice, contiguous(), all_reduce, to(dtype), narrow/view/copy_.
 #include <hip/hip_runtime.h>
+#include <hip/hip_ext.h>
 
 #include <cstdarg>
 #include <cstdio>
@@ -985,30 +986,59 @@ int check_range(const EthaTable* t, uint32_t first, uint32_t count, int kind) {
   return ETHA_OK;
 }
 
+// Launch with or without ordering against the launches already on the stream.  An ordinary launch waits
+// for every earlier packet of its queue (that is how a stream stays in order).  ETHA_LAUNCH_UNORDERED
+// clears that wait for this one dispatch: the kernel may start while earlier launches are still running,
+// which removes the drain/ramp bubble between launches that do not depend on each other.  The next
+// ordinary launch on the stream again waits for everything before it, unordered launches included.
+template <typename... Args, typename F>
+void launch_kernel(F kernel, dim3 grid, dim3 block, size_t lds, void* stream, uint32_t flags, Args... args) {
+  if (flags & ETHA_LAUNCH_UNORDERED)
+    hipExtLaunchKernelGGL(kernel, grid, block, (uint32_t)lds, (hipStream_t)stream, nullptr, nullptr, hipExtAnyOrderLaunch,
+                          args...);
+  else
+    hipLaunchKernelGGL(kernel, grid, block, lds, (hipStream_t)stream, args...);
+}
+
 template <bool REV>
-int launch_tiles(const EthaTable* t, uint32_t first, uint32_t count, void* stream) {
+int launch_tiles(const EthaTable* t, uint32_t first, uint32_t count, void* stream, uint32_t flags) {
   const uint32_t r0 = t->run_begin[first], r1 = t->run_begin[first + count];
   const uint32_t w0 = t->row_begin[first], w1 = t->row_begin[first + count];
   const uint32_t n_run = r1 - r0, n_row = w1 - w0;
   const uint32_t x0 = t->trans_begin[first], n_trans = t->trans_begin[first + count] - x0;
   if (n_trans) {  // transposing chunks run in their own kernel (it needs LDS)
     const size_t lds = (size_t)kTransDim * (kTransDim + 1) * t->trans_es_max;
-    hipLaunchKernelGGL(etha_transpose_kernel<REV>, dim3(n_trans), dim3(64), lds, (hipStream_t)stream, t->d_trans + x0);
+    launch_kernel(etha_transpose_kernel<REV>, dim3(n_trans), dim3(64), lds, stream, flags, (const TransTile*)(t->d_trans + x0));
     HIP_TRY(hipGetLastError());
+    flags |= ETHA_LAUNCH_UNORDERED;  // the two kernels of one call touch different chunks
   }
   if (n_run + n_row == 0) return ETHA_OK;
+  const RunTile* d_run = t->d_run + r0;
+  const RowTile* d_row = t->d_row + w0;
   if (REV == (t->kind == 0)) {  // the direction that writes the a side (unpack) / b side (self-copy) of an ordered range
     auto it = t->ordered.find(std::make_pair(first, count));
     if (it != t->ordered.end()) {
-      hipLaunchKernelGGL(etha_tile_kernel<REV>, dim3((n_run + n_row) * kBlocksPerTile), dim3(kBlockThreads), 0,
-                         (hipStream_t)stream, it->second.d_run, n_run, it->second.d_row);
-      HIP_TRY(hipGetLastError());
-      return ETHA_OK;
+      d_run = it->second.d_run;
+      d_row = it->second.d_row;
     }
   }
-  hipLaunchKernelGGL(etha_tile_kernel<REV>, dim3((n_run + n_row) * kBlocksPerTile), dim3(kBlockThreads), 0,
-                     (hipStream_t)stream, t->d_run + r0, n_run, t->d_row + w0);
+  launch_kernel(etha_tile_kernel<REV>, dim3((n_run + n_row) * kBlocksPerTile), dim3(kBlockThreads), 0, stream, flags, d_run,
+                n_run, d_row);
   HIP_TRY(hipGetLastError());
+  return ETHA_OK;
+}
+
+int launch_reduce(const EthaTable* t, uint32_t first, uint32_t count, void* stream, uint32_t flags) {
+  const uint32_t w0 = t->row_begin[first], w1 = t->row_begin[first + count];
+  if (w1 == w0) return ETHA_OK;
+  launch_kernel(etha_reduce_kernel, dim3((w1 - w0) * kBlocksPerTile), dim3(kBlockThreads), 0, stream, flags,
+                (const RowTile*)(t->d_row + w0), (const uint64_t*)t->d_peers);
+  HIP_TRY(hipGetLastError());
+  return ETHA_OK;
+}
+
+int check_flags(uint32_t flags) {
+  if (flags & ~(uint32_t)ETHA_LAUNCH_UNORDERED) return fail(ETHA_ERR_INVALID, "unknown launch flags 0x%x", flags);
   return ETHA_OK;
 }
 
@@ -1267,47 +1297,41 @@ int etha_table_read_ordered(const EthaTable* t, uint32_t first, uint32_t count, 
   return ETHA_OK;
 }
 
-int etha_pack_bucket(const EthaTable* t, uint32_t first, uint32_t count, void* stream) {
-  const int rc = check_range(t, first, count, 0);
+int etha_pack_bucket(const EthaTable* t, uint32_t first, uint32_t count, void* stream, uint32_t flags) {
+  int rc = check_range(t, first, count, 0);
+  if (rc == ETHA_OK) rc = check_flags(flags);
   if (rc != ETHA_OK) return rc;
   if (t->reduce_prefix[first + count] != t->reduce_prefix[first])
     return fail(ETHA_ERR_INVALID, "range holds Partial chunks; use etha_reduce_pack_bucket");
-  return launch_tiles<false>(t, first, count, stream);
+  return launch_tiles<false>(t, first, count, stream, flags);
 }
 
-int etha_unpack_bucket(const EthaTable* t, uint32_t first, uint32_t count, void* stream) {
-  const int rc = check_range(t, first, count, 0);
+int etha_unpack_bucket(const EthaTable* t, uint32_t first, uint32_t count, void* stream, uint32_t flags) {
+  int rc = check_range(t, first, count, 0);
+  if (rc == ETHA_OK) rc = check_flags(flags);
   if (rc != ETHA_OK) return rc;
   if (t->reduce_prefix[first + count] != t->reduce_prefix[first])
     return fail(ETHA_ERR_INVALID, "range holds Partial chunks; a Partial placement cannot be a target");
-  return launch_tiles<true>(t, first, count, stream);
+  return launch_tiles<true>(t, first, count, stream, flags);
 }
 
-int etha_reduce_pack_bucket(const EthaTable* t, uint32_t first, uint32_t count, void* stream) {
-  const int rc = check_range(t, first, count, 0);
+int etha_reduce_pack_bucket(const EthaTable* t, uint32_t first, uint32_t count, void* stream, uint32_t flags) {
+  int rc = check_range(t, first, count, 0);
+  if (rc == ETHA_OK) rc = check_flags(flags);
   if (rc != ETHA_OK) return rc;
   if (t->reduce_prefix[first + count] - t->reduce_prefix[first] != count)
     return fail(ETHA_ERR_INVALID, "range holds chunks that are not Partial chunks");
-  const uint32_t w0 = t->row_begin[first], w1 = t->row_begin[first + count];
-  if (w1 == w0) return ETHA_OK;
-  hipLaunchKernelGGL(etha_reduce_kernel, dim3((w1 - w0) * kBlocksPerTile), dim3(kBlockThreads), 0, (hipStream_t)stream, t->d_row + w0,
-                     t->d_peers);
-  HIP_TRY(hipGetLastError());
-  return ETHA_OK;
+  return launch_reduce(t, first, count, stream, flags);
 }
 
-int etha_selfcopy_bucket(const EthaTable* t, uint32_t first, uint32_t count, void* stream) {
-  const int rc = check_range(t, first, count, 1);
+int etha_selfcopy_bucket(const EthaTable* t, uint32_t first, uint32_t count, void* stream, uint32_t flags) {
+  int rc = check_range(t, first, count, 1);
+  if (rc == ETHA_OK) rc = check_flags(flags);
   if (rc != ETHA_OK) return rc;
   const uint32_t n_reduce = t->reduce_prefix[first + count] - t->reduce_prefix[first];
-  if (n_reduce == 0) return launch_tiles<false>(t, first, count, stream);
+  if (n_reduce == 0) return launch_tiles<false>(t, first, count, stream, flags);
   if (n_reduce != count) return fail(ETHA_ERR_INVALID, "range mixes Partial and plain chunks; launch them separately");
-  const uint32_t w0 = t->row_begin[first], w1 = t->row_begin[first + count];
-  if (w1 == w0) return ETHA_OK;
-  hipLaunchKernelGGL(etha_reduce_kernel, dim3((w1 - w0) * kBlocksPerTile), dim3(kBlockThreads), 0, (hipStream_t)stream,
-                     t->d_row + w0, t->d_peers);
-  HIP_TRY(hipGetLastError());
-  return ETHA_OK;
+  return launch_reduce(t, first, count, stream, flags);
 }
 
 int etha_arena_create(uint64_t nbytes, void** out_ptr) {

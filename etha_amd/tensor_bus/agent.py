@@ -96,12 +96,14 @@ class TensorBusAgent:
 
     def __init__(self, world_size: int, path_naming_fn=None, device: str | torch.device = "cuda:0",
                  heartbeat_interval: float = 0.2, zero_copy_single_chunk: bool = False,
-                 direct_same_device: bool = False):
+                 direct_same_device: bool = False, pool: str = "ring", max_in_flight: int = 2):
         self.world_size = world_size
         self.device = torch.device(device)
         self.path_naming_fn = path_naming_fn or default_path_naming
         self.heartbeat_interval = heartbeat_interval
-        self.wire = LoopbackWire(self.device if self.device.type == "cuda" else None)
+        # bucket buffers: a ring of max_in_flight slots per channel (the reference's bound, comm_methods.py:53-119),
+        # or pool="resident" for a slot per bucket
+        self.wire = LoopbackWire(self.device if self.device.type == "cuda" else None, pool=pool, max_in_flight=max_in_flight)
         # lent buckets are read from the worker's tensor at receive time, so a send that lends memory only
         # completes once its receivers have unpacked (the reference's transfers end with a barrier as well)
         self.wire.zero_copy_single_chunk = zero_copy_single_chunk
@@ -269,7 +271,9 @@ class TensorBusAgent:
         if isinstance(cmd, CleanupBatch):
             batch = self.batches.get(cmd.batch_id)
             if batch is not None:
-                batch.registrations.pop(entry.rank, None)
+                # this rank is done with the batch (its transfers have returned, so the device has been
+                # synchronised since): drop its plans, then the mappings of its tensors
+                self._release_rank(batch, entry.rank)
                 if not batch.registrations:
                     self._release_batch(batch)
                     del self.batches[cmd.batch_id]
@@ -474,6 +478,10 @@ class TensorBusAgent:
             # the device before it replies), because a member's tensor is read by another member's kernel
             if any(batch.send_count.get(m, 0) < done_gen for m in members):
                 return False, None
+            # with a ring pool a send has only packed as far as its slots reach; the rest follows as its receivers
+            # unpack, so it completes with them - as a sender's bucket_comm does in the reference
+            if self.wire.in_progress(buckets):
+                return False, None
             # a send whose tensors are lent to receivers - its own buckets, or a Partial reduction that another
             # member ships and the receiver computes - waits for those receivers to have run
             for m in members | {rank}:
@@ -495,6 +503,21 @@ class TensorBusAgent:
                 batch.transfer_signal = False  # every destination of every send so far has received
         self.stats["transfers"] += 1
         return True, result
+
+    def _release_rank(self, batch: BatchState, rank: int) -> None:
+        """Forget one rank of a batch: its compiled bucket lists (receive side first: it only references slots
+        that send lists own) and the hipIPC mappings of the tensors it registered."""
+        for table in (batch.recv_buckets, batch.send_buckets):
+            buckets = table.pop(rank, None)
+            if buckets:
+                self.wire.release(buckets)
+        for _, t in batch.registrations.pop(rank, ()):
+            if isinstance(t, IpcTensor):
+                try:
+                    t.close()
+                except Exception:
+                    logger.exception("closing an IPC mapping failed")
+        batch.planned_ranks.discard(rank)
 
     def _release_batch(self, batch: BatchState) -> None:
         # receivers first: their plans only reference slots, the senders' plans own them

@@ -107,6 +107,8 @@ class ReshardJob:
     local_view: object = None  # optional ``(kind, tensor) -> view``: re-home a local shard inside another parent
     zero_copy: bool = False  # lend contiguous single-chunk buckets instead of packing them (see LoopbackWire)
     direct: bool = False  # no bucket buffers for plain buckets: targets copy straight from the sources (see LoopbackWire)
+    pool: str = "ring"  # "ring": max_in_flight slots per channel; "resident": one slot per bucket (see LoopbackWire)
+    max_in_flight: int = 2
     source_locals: list[dict[int, torch.Tensor]] = field(default_factory=list, init=False)
     target_locals: list[dict[int, torch.Tensor]] = field(default_factory=list, init=False)
     globals_: list[torch.Tensor | None] = field(default_factory=list, init=False)
@@ -116,7 +118,8 @@ class ReshardJob:
     def __post_init__(self) -> None:
         self.device = torch.device(self.device)
         if self.wire is None:
-            self.wire = LoopbackWire(self.device)
+            self.wire = LoopbackWire(self.device, pool=self.pool, max_in_flight=self.max_in_flight)
+        self.pool = self.wire.pool_mode
         if self.zero_copy:
             self.wire.zero_copy_single_chunk = True
         if self.direct:
@@ -125,6 +128,9 @@ class ReshardJob:
         recv_chunks: dict[int, list] = {}
         m2m_cache: dict[tuple, object] = {}
         wanted = set(self.target_ranks) if self.target_ranks is not None else None
+        if wanted is not None:  # target ranks that are not staged never unpack: the wire must not wait for them
+            named = {r for spec in self.specs for r in _flat_ranks(spec.target_mesh)}
+            self.wire.absent_ranks |= named - wanted
         for spec in self.specs:
             src_mesh, tgt_mesh = np.asarray(spec.source_mesh), np.asarray(spec.target_mesh)
             src_ranks, tgt_ranks = _flat_ranks(src_mesh), _flat_ranks(tgt_mesh)
@@ -204,19 +210,30 @@ class ReshardJob:
         return False
 
     # ------------------------------------------------------------------------------------------
-    def run_send(self, merge_launches: bool = False, fanout: int = 1) -> None:
+    def run_send(self, merge_launches: bool = False, fanout: int = 1, drive: bool = True) -> None:
         for buckets in self.send_buckets.values():
-            bucket_comm(buckets, wire=self.wire, merge_launches=merge_launches, synchronize=False, fanout=fanout)
+            bucket_comm(buckets, self.max_in_flight, wire=self.wire, merge_launches=merge_launches, synchronize=False,
+                        fanout=fanout, drive=drive)
 
-    def run_recv(self, merge_launches: bool = False, fanout: int = 1) -> None:
+    def run_recv(self, merge_launches: bool = False, fanout: int = 1, drive: bool = True) -> None:
         for buckets in self.recv_buckets.values():
-            bucket_comm(buckets, wire=self.wire, merge_launches=merge_launches, synchronize=False, fanout=fanout)
+            bucket_comm(buckets, self.max_in_flight, wire=self.wire, merge_launches=merge_launches, synchronize=False,
+                        fanout=fanout, drive=drive)
 
     def run(self, merge_launches: bool = False, synchronize: bool = True, fanout: int = 1) -> None:
-        """One transfer: every source rank packs (and self-copies), then every target rank unpacks."""
-        self.run_send(merge_launches, fanout)
-        self.run_recv(merge_launches, fanout)
-        if synchronize:
+        """One transfer: every source rank calls ``bucket_comm`` on its send list, then every target rank on its
+        receive list.  With a ring pool the senders fill their slots and wait on the wire; the receivers' calls
+        then move both sides along until every bucket has been unpacked."""
+        if self.wire.pool_mode == "ring":  # this process plays every rank: queue all pipelines, step them together
+            self.run_send(merge_launches, fanout, drive=False)
+            self.run_recv(merge_launches, fanout, drive=False)
+            self.wire.drive()
+        else:
+            self.run_send(merge_launches, fanout)
+            self.run_recv(merge_launches, fanout)
+        if not self.wire.idle():
+            raise RuntimeError(f"transfer did not complete; still waiting for a peer: {self.wire.pending()}")
+        if synchronize and self.device.type == "cuda":
             torch.cuda.current_stream(self.device).synchronize()
 
     def capture(self, merge_launches: bool = True):

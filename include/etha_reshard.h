@@ -31,7 +31,7 @@
 extern "C" {
 #endif
 
-#define ETHA_ABI_VERSION 3
+#define ETHA_ABI_VERSION 4
 #define ETHA_MAX_NDIM 8
 
 /* status codes */
@@ -53,6 +53,18 @@ enum {
   ETHA_B32 = 6,  /* opaque 4-byte element (int32/...) */
   ETHA_B64 = 7   /* opaque 8-byte element (int64/complex32/...) */
 };
+
+/*
+ * Launch flags.  By default a launch is ordered after everything enqueued on its stream before it, like any
+ * kernel.  ETHA_LAUNCH_UNORDERED declares that this launch depends on none of the launches enqueued on the
+ * stream since the last launch without the flag: it may start while they are still running, which hides the
+ * drain/ramp gap between kernels.  The next launch without the flag (of this library or any other kernel on
+ * the stream) waits for all of them.  The caller owns the dependency analysis: two launches that touch the
+ * same bucket buffer, or a launch that reads bytes another one writes, must be separated by an ordered
+ * launch.  The reference needs no such notion because each of its buckets is many small ATen launches on one
+ * stream (ir.py:246-259); here a bucket is one launch and the gap between launches is what is left to hide.
+ */
+#define ETHA_LAUNCH_UNORDERED 1u
 
 /* reduce ops of a Partial source (ir.py:51-57) */
 enum { ETHA_SUM = 0, ETHA_AVG = 1, ETHA_MAX = 2, ETHA_MIN = 3, ETHA_PRODUCT = 4 };
@@ -166,14 +178,14 @@ int etha_table_read_ordered(const EthaTable* table, uint32_t first, uint32_t cou
  * Replaces Bucket.prepare() for a source bucket (ir.py:229-264; Chunk.prepare ir.py:112-126).
  * The range must not contain reduce chunks.
  */
-int etha_pack_bucket(const EthaTable* table, uint32_t first, uint32_t count, void* stream);
+int etha_pack_bucket(const EthaTable* table, uint32_t first, uint32_t count, void* stream, uint32_t flags);
 
 /*
  * Scatter chunks [first, first+count) from their bucket positions into their tensors,
  * converting wire_dtype -> tensor_dtype.  One kernel launch.
  * Replaces Bucket.finalize() for a target bucket (ir.py:300-310; Chunk.finalize ir.py:134-141).
  */
-int etha_unpack_bucket(const EthaTable* table, uint32_t first, uint32_t count, void* stream);
+int etha_unpack_bucket(const EthaTable* table, uint32_t first, uint32_t count, void* stream, uint32_t flags);
 
 /*
  * Partial-source buckets: for every chunk combine the n_partials peer regions element-wise
@@ -182,10 +194,10 @@ int etha_unpack_bucket(const EthaTable* table, uint32_t first, uint32_t count, v
  * Replaces the clone + all_reduce + cast of Chunk.prepare (ir.py:116-126).
  * Every chunk of the range must be a reduce chunk.
  */
-int etha_reduce_pack_bucket(const EthaTable* table, uint32_t first, uint32_t count, void* stream);
+int etha_reduce_pack_bucket(const EthaTable* table, uint32_t first, uint32_t count, void* stream, uint32_t flags);
 
 /* Run chunks [first, first+count) of a self-copy or direct table.  One kernel launch. */
-int etha_selfcopy_bucket(const EthaTable* table, uint32_t first, uint32_t count, void* stream);
+int etha_selfcopy_bucket(const EthaTable* table, uint32_t first, uint32_t count, void* stream, uint32_t flags);
 
 /*
  * Bucket-pool memory that can cross a process boundary on the same GPU (the worker <-> agent

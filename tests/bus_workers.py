@@ -184,7 +184,9 @@ def producer_process(device, conn, rounds, zero_copy=False):
         from helpers import cpu_fill
 
         setup_ptrace()
-        job = ReshardJob(_pool_specs(), device=device, bucket_size=32 * 1024, fill=cpu_fill, zero_copy=zero_copy)
+        # a pool that another process reads is resident: a ring is recycled under a hand-shake inside one process
+        job = ReshardJob(_pool_specs(), device=device, bucket_size=32 * 1024, fill=cpu_fill, zero_copy=zero_copy,
+                         pool="resident")
         lent = 0
         for buckets in job.send_buckets.values():
             lent += len(job.wire.plan(buckets).lent)  # planning assigns the slots

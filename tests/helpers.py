@@ -76,10 +76,11 @@ def clone_specs(specs):
     return [copy.copy(s) for s in specs]
 
 
-def gpu_vs_oracle(specs, device, bucket_size, target_ranks=None, merge_launches=False, check_closed_form=True):
+def gpu_vs_oracle(specs, device, bucket_size, target_ranks=None, merge_launches=False, check_closed_form=True,
+                  pool="ring", max_in_flight=2):
     """Run the same job on the GPU (HIP path) and on the CPU (oracle); compare every target shard."""
     gpu_job = ReshardJob(clone_specs(specs), device=device, bucket_size=bucket_size, target_ranks=target_ranks,
-                         keep_globals=True, fill=cpu_fill)
+                         keep_globals=True, fill=cpu_fill, pool=pool, max_in_flight=max_in_flight)
     cpu_job = ReshardJob(clone_specs(specs), device="cpu", bucket_size=bucket_size, target_ranks=target_ranks,
                          keep_globals=True, fill=cpu_fill)
     mirror_partials(gpu_job, cpu_job)

@@ -281,11 +281,42 @@ def test_recv_before_send_is_an_error(gpu_device):
 
 # ---- scaled-down versions of the headline configs, against the oracle ---------------------------------
 
+@pytest.mark.parametrize("pool", ["ring", "resident"])
 @pytest.mark.parametrize("merge", [False, True])
-def test_llama_like_fsdp_to_tp_small(gpu_device, merge):
+def test_llama_like_fsdp_to_tp_small(gpu_device, merge, pool):
     specs, targets, _ = workloads.llama3_8b_fsdp8_to_tp2(n_layers=2, hidden=256, inter=896, kv=64, vocab=2056)
-    gpu_vs_oracle(specs, gpu_device, 64 * 1024, target_ranks=targets, merge_launches=merge)
-    gpu_vs_oracle(specs, gpu_device, 64 * 1024, target_ranks=None, merge_launches=merge)
+    gpu_vs_oracle(specs, gpu_device, 64 * 1024, target_ranks=targets, merge_launches=merge, pool=pool)
+    gpu_vs_oracle(specs, gpu_device, 64 * 1024, target_ranks=None, merge_launches=merge, pool=pool)
+
+
+@pytest.mark.parametrize("depth", [1, 2, 4])
+def test_ring_depths_and_unordered_launches(gpu_device, depth):
+    """Many buckets per channel through rings of 1, 2 and 4 slots: same bytes as the oracle, the pool stays
+    within channels x depth x bucket, most launches are issued without ordering, and switching that off
+    changes nothing but the flags."""
+    specs, targets, _ = workloads.llama3_8b_fsdp8_to_tp2(n_layers=6, hidden=256, inter=896, kv=64, vocab=520)
+    job, _ = gpu_vs_oracle(specs, gpu_device, 32 * 1024, target_ranks=targets, max_in_flight=depth)
+    channels = sum(len({(b.src_rank, b.dst_ranks, b.transport) for b in bs}) for bs in job.send_buckets.values())
+    largest = max(b.total_bytes for bs in job.send_buckets.values() for b in bs)
+    assert job.wire.pool.reserved_bytes <= channels * depth * (largest + 256)
+    assert job.wire.pool.reserved_bytes < job.payload_bytes() // 2
+    log = job.wire.launch_log = []
+    for d in job.target_locals:
+        for t in d.values():
+            t.zero_()
+    job.run()
+    assert sum(1 for _, _, _, flags in log if flags & 1) > len(log) // 2
+    want = [{r: t.clone() for r, t in d.items()} for d in job.target_locals]
+    job.wire.unordered_launches = False
+    log.clear()
+    for d in job.target_locals:
+        for t in d.values():
+            t.zero_()
+    job.run()
+    assert not any(flags & 1 for _, _, _, flags in log)
+    for d, w in zip(job.target_locals, want):
+        for r, t in d.items():
+            assert torch.equal(t.view(torch.uint8), w[r].view(torch.uint8))
 
 
 def test_many_small_2d_to_replicate_small(gpu_device):
@@ -335,7 +366,12 @@ def test_llama3_8b_full_size_properties(gpu_device, bucket_size):
         assert job.counts()["recv_buckets"] == 1672
     src_sums = [{r: t.view(torch.int16).sum(dtype=torch.int64).item() for r, t in d.items()} for d in job.source_locals]
     job.run(merge_launches=True)
-    from etha_amd.layout import local_shard
+    if bucket_size == 64 << 20:
+        # the pool is a ring: 2 slots per channel, each as large as the channel's largest bucket (here the
+        # 125.25 MiB single-chunk embedding buckets), instead of the 8.03 GB a slot per bucket would take
+        embed = 128256 // 8 * 4096 * 2
+        assert job.wire.pool.reserved_bytes <= 8 * 2 * embed + 8 * 2 * 65536
+    from oracle.dtensor_layout import local_shard  # the pinned convention, not the product's planner
 
     def check():
         for i, spec in enumerate(specs):
@@ -424,9 +460,12 @@ def test_moe_experts_and_uneven_vocab_full_size_properties(gpu_device):
 def test_per_bucket_launches_on_side_streams(gpu_device):
     """Fan-out over side streams (fork/join with events) gives the same bytes as one stream."""
     specs, targets, _ = workloads.llama3_8b_fsdp8_to_tp2(n_layers=3, hidden=256, inter=896, kv=64, vocab=2056)
-    gpu_job = ReshardJob(specs, device=gpu_device, bucket_size=32 * 1024, target_ranks=targets, keep_globals=True, fill=cpu_fill)
+    gpu_job = ReshardJob(specs, device=gpu_device, bucket_size=32 * 1024, target_ranks=targets, keep_globals=True, fill=cpu_fill,
+                         pool="resident")  # side streams run a list in list order: every bucket needs its own slot
     cpu_job = ReshardJob(specs, device="cpu", bucket_size=32 * 1024, target_ranks=targets, keep_globals=True, fill=cpu_fill)
     run_oracle(cpu_job)
+    with pytest.raises(ValueError, match="resident pool"):
+        ReshardJob(specs, device=gpu_device, bucket_size=32 * 1024, target_ranks=targets).run(fanout=2)
     for fanout in (3, 1, 4):
         for d in gpu_job.target_locals:
             for t in d.values():
@@ -509,22 +548,31 @@ def test_bucket_protocol_methods(gpu_device):
     for buckets in send.values():
         for b in buckets:
             b.prepare(wire)
-            assert b.launch() and b.is_complete()
-            b.finalize(wire)  # nothing to write on the source side
+            assert b.launch()
+            assert not b.is_complete(wire)  # packed into its ring slot, not yet unpacked by its destination
     for buckets in recv.values():
         for b in buckets:
             b.prepare(wire)
-            assert b.launch() and b.is_complete()
+            assert b.launch() and b.is_complete(wire)
             b.finalize(wire)
+            assert not b.is_complete(wire)  # consumed: the next transfer's bytes have not arrived
+            with pytest.raises(RuntimeError, match="before its send bucket was packed"):
+                b.finalize(wire)
+    for buckets in send.values():
+        for b in buckets:
+            assert b.is_complete(wire)
+            b.finalize(wire)  # nothing to write on the source side
     torch.cuda.synchronize()
     for j in range(2):
         assert torch.equal(tgt[2 + j].cpu(), g[:, 16 * j : 16 * (j + 1)])
 
 
-def test_hip_graph_replay_matches_eager(gpu_device):
-    """A captured transfer replays correctly, several times, with new source values each time."""
+@pytest.mark.parametrize("pool", ["ring", "resident"])
+def test_hip_graph_replay_matches_eager(gpu_device, pool):
+    """A captured transfer replays correctly, several times, with new source values each time.  (Under capture
+    the wire issues every launch in order: a captured stream is a chain anyway.)"""
     specs, targets, _ = workloads.llama3_8b_fsdp8_to_tp2(n_layers=2, hidden=256, inter=896, kv=64, vocab=2056)
-    job = ReshardJob(specs, device=gpu_device, bucket_size=64 * 1024, target_ranks=targets)
+    job = ReshardJob(specs, device=gpu_device, bucket_size=64 * 1024, target_ranks=targets, pool=pool)
     job.run(merge_launches=True)  # plans, uploads
     graph = job.capture(merge_launches=True)
     from etha_amd.layout import local_shard
@@ -595,16 +643,18 @@ def test_random_batches_gpu(gpu_device, seed):
             return wide[..., 1 : 1 + t.shape[-1]]
     merge = bool(rng.integers(2))
     mode = ["buckets", "buckets", "zero_copy", "direct"][int(rng.integers(4))]  # wire options must not change results
+    fanout = 3 if seed % 5 == 4 else 1  # every fifth batch: launches spread over side streams (needs a slot per bucket)
+    pool = "resident" if fanout > 1 or seed % 5 == 3 else "ring"
+    depth = int(rng.integers(1, 4))
     gpu_job = ReshardJob(specs, device=gpu_device, bucket_size=bucket_size, keep_globals=True, fill=cpu_fill, local_view=view,
-                         zero_copy=mode == "zero_copy", direct=mode == "direct")
+                         zero_copy=mode == "zero_copy", direct=mode == "direct", pool=pool, max_in_flight=depth)
     cpu_job = ReshardJob(specs, device="cpu", bucket_size=bucket_size, keep_globals=True, fill=cpu_fill, local_view=view)
     mirror_partials(gpu_job, cpu_job)
-    fanout = 3 if seed % 5 == 4 else 1  # every fifth batch: launches spread over side streams
     gpu_job.run(merge_launches=merge, fanout=fanout)
     run_oracle(cpu_job)
     for i, spec in enumerate(specs):
         for r, t in gpu_job.target_locals[i].items():
-            assert_bit_equal(t, cpu_job.target_locals[i][r], f"seed {seed} ({mode}, fanout {fanout}) {spec.name} rank {r}")
+            assert_bit_equal(t, cpu_job.target_locals[i][r], f"seed {seed} ({mode}, {pool} pool, fanout {fanout}) {spec.name} rank {r}")
 
 
 @pytest.mark.parametrize("dtype", [torch.int8, torch.bfloat16, torch.float32, torch.float64])

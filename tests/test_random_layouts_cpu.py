@@ -84,8 +84,47 @@ def _random_spec(rng, idx, wire_size):
                       seed=1000 + idx, std=1.0, dist="normal" if sdt in FLOATS else "bits")
 
 
+def _run_step(mem, p, kind, first, count, ordered=False, touched=None):
+    if kind in ("pack", "reduce_pack"):
+        execute(p.send_table, mem, "pack", first, count, peers=_peers_of(p), touched=touched)
+    elif kind == "unpack":
+        execute(p.recv_table, mem, "unpack", first, count, ordered=ordered, touched=touched)
+    elif kind in ("selfcopy", "direct"):
+        execute(p.local_table, mem, "selfcopy", first, count, ordered=ordered, touched=touched)
+    elif kind == "direct_reduce":
+        execute(p.local_table, mem, "selfcopy", first, count, peers=_direct_peers_of(p), touched=touched)
+    else:
+        assert kind == "lend"  # nothing runs for a lent bucket
+
+
+class _HazardCheck:
+    """Byte-level check of the wire's launch ordering, independent of how the wire decides it: launches
+    issued without ordering since the last ordered one may run at the same time on the GPU, so none of them
+    may read a byte another one writes, and no two may write the same byte."""
+
+    def __init__(self):
+        self.reads = np.zeros(0, np.int64)
+        self.writes = np.zeros(0, np.int64)
+        self.unordered = 0
+
+    def launch(self, touched: dict, flags: int) -> None:
+        r = np.unique(np.concatenate(touched["r"])) if touched.get("r") else np.zeros(0, np.int64)
+        w = np.unique(np.concatenate(touched["w"])) if touched.get("w") else np.zeros(0, np.int64)
+        if flags & 1:
+            self.unordered += 1
+            assert not len(np.intersect1d(r, self.writes)), "unordered launch reads bytes written since the last ordered launch"
+            assert not len(np.intersect1d(w, self.reads)), "unordered launch writes bytes read since the last ordered launch"
+            assert not len(np.intersect1d(w, self.writes)), "two unordered launches write the same bytes"
+            self.reads = np.union1d(self.reads, r)
+            self.writes = np.union1d(self.writes, w)
+        else:
+            self.reads, self.writes = r, w
+
+
 def _interpret(job, merged: bool):
-    """What ReshardJob.run would enqueue, executed on the host by the tile interpreter."""
+    """What ReshardJob.run would enqueue, executed on the host by the tile interpreter.  With a ring pool the
+    wire's own bucket pipelines decide the order (slots are reused, so list order would be wrong); the wire
+    hands every launch to the interpreter instead of the GPU."""
     plans = [job.wire.plan(b) for b in job.send_buckets.values()] + [job.wire.plan(b) for b in job.recv_buckets.values()]
     # the span of everything that may legitimately be touched: every shard's storage and the bucket pool
     ranges = []
@@ -101,19 +140,25 @@ def _interpret(job, merged: bool):
         return
     lo, hi = min(r[0] for r in ranges), max(r[1] for r in ranges)
     mem = AbsoluteMemory(lo, hi)
+    if job.wire.pool_mode == "ring":
+        check = _HazardCheck()
+
+        def on_launch(p, kind, first, count, flags):
+            touched = {}
+            # a recurring multi-bucket scatter runs from its written-address-ordered copy, as on the GPU
+            _run_step(mem, p, kind, first, count, ordered=(kind, first, count) in p._ordered_ranges, touched=touched)
+            check.launch(touched, flags)
+
+        job.wire.on_launch = on_launch
+        try:
+            job.run(merge_launches=merged)
+        finally:
+            job.wire.on_launch = None
+        return check
     for p in plans:
         steps = p.merged_steps if merged else [(k, f, c, (s,)) for k, f, c, s in p.steps]
         for kind, first, count, slots in steps:
-            if kind in ("pack", "reduce_pack"):
-                execute(p.send_table, mem, "pack", first, count, peers=_peers_of(p))
-            elif kind == "unpack":
-                execute(p.recv_table, mem, "unpack", first, count, ordered=merged and len(slots) > 1)
-            elif kind in ("selfcopy", "direct"):
-                execute(p.local_table, mem, "selfcopy", first, count, ordered=merged and len(slots) > 1)
-            elif kind == "direct_reduce":
-                execute(p.local_table, mem, "selfcopy", first, count, peers=_direct_peers_of(p))
-            else:
-                assert kind == "lend"  # nothing runs for a lent bucket
+            _run_step(mem, p, kind, first, count, ordered=merged and len(slots) > 1)
 
 
 def _direct_peers_of(plan):
@@ -195,9 +240,12 @@ def test_random_batches(seed, spec_fn=None):
     merged = bool(rng.integers(2))
     # wire options must not change results: plain buckets, lent single-chunk buckets, or no buckets at all
     mode = ["buckets", "buckets", "zero_copy", "direct"][int(rng.integers(4))]
+    # the pool: a ring of 1-3 slots per channel (the default form), or a slot per bucket
+    pool = ["ring", "ring", "resident"][int(rng.integers(3))]
+    depth = int(rng.integers(1, 4))
     job = ReshardJob(specs, device="cpu", bucket_size=bucket_size, keep_globals=True, fill=cpu_fill, local_view=view,
-                     wire=LoopbackWire("cpu", segment_bytes=1 << 22, host_inspection=True), direct=mode == "direct",
-                     zero_copy=mode == "zero_copy")
+                     wire=LoopbackWire("cpu", segment_bytes=1 << 22, host_inspection=True, pool=pool, max_in_flight=depth),
+                     direct=mode == "direct", zero_copy=mode == "zero_copy", max_in_flight=depth)
     ref = ReshardJob(specs, device="cpu", bucket_size=bucket_size, keep_globals=True, fill=cpu_fill, local_view=view)
     for a, b in zip(job.source_locals, ref.source_locals):  # Partial sources are drawn per job: make them equal
         for r in a:

@@ -113,6 +113,35 @@ def test_partial_target_direction_is_rejected(agent_factory):
         c.close()
 
 
+def test_cleanup_unmaps_each_ranks_ipc_tensors(agent_factory, monkeypatch):
+    """CleanupBatch from a rank closes the hipIPC mappings of the tensors that rank registered - every one, once -
+    and the batch disappears with its last rank."""
+    from etha_amd import _native
+    from etha_amd.tensor_bus.agent import BatchState, _Entry
+    from etha_amd.tensor_bus.commands import CleanupBatch
+    from etha_amd.tensor_bus.ipc_tensor import IpcTensor
+
+    agent, _ = agent_factory(2)
+    agent._stop.set()  # drive the commands by hand
+    closed = []
+    monkeypatch.setattr(_native, "ipc_close", lambda ptr: closed.append(ptr))
+    dev = torch.device("cpu")
+    batch = BatchState("b", ["p"], None)
+    batch.registrations = {
+        0: [("p", IpcTensor(0x1000, (4,), (1,), torch.float32, dev, 0x1000, 16)),
+            ("p", IpcTensor(0x2000, (4,), (1,), torch.float32, dev, 0x2000, 16))],
+        1: [("p", IpcTensor(0x3000, (4,), (1,), torch.float32, dev, 0x3000, 16)), ("p", torch.zeros(4))],
+    }
+    batch.planned_ranks = {0, 1}
+    agent.batches["b"] = batch
+    assert agent._advance(_Entry(rank=0, conn=None, command=CleanupBatch(batch_id="b"))) == (True, None)
+    assert sorted(closed) == [0x1000, 0x2000] and "b" in agent.batches and 0 not in batch.registrations
+    assert agent._advance(_Entry(rank=1, conn=None, command=CleanupBatch(batch_id="b"))) == (True, None)
+    assert sorted(closed) == [0x1000, 0x2000, 0x3000] and "b" not in agent.batches
+    assert agent._advance(_Entry(rank=1, conn=None, command=CleanupBatch(batch_id="b"))) == (True, None)  # idempotent
+    assert len(closed) == 3
+
+
 def test_bootstrap_client_resolves_rank_and_paths(agent_factory, monkeypatch):
     agent, naming = agent_factory(3)
     monkeypatch.setenv("RANK", "1")

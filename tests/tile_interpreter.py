@@ -95,10 +95,31 @@ def _unit_positions(run_tiles, row_tiles):
     return out
 
 
+_TOUCHED: dict | None = None  # while execute(..., touched=d) runs: d["r"] / d["w"] collect byte offsets
+
+
+def _note(kind: str, offsets: np.ndarray) -> None:
+    if _TOUCHED is not None:
+        _TOUCHED[kind].append(np.unique(offsets.reshape(-1)))
+
+
 def execute(table, arena, direction: str, first: int = 0, count: int | None = None,
-            peers: np.ndarray | None = None, ordered: bool = False) -> None:
+            peers: np.ndarray | None = None, ordered: bool = False, touched: dict | None = None) -> None:
     """Run chunks [first, first+count) of a table on the host. direction: 'pack' | 'unpack' | 'selfcopy'.
-    ``ordered``: use the write-ordered copy of the range (it must have been optimized)."""
+    ``ordered``: use the write-ordered copy of the range (it must have been optimized).
+    ``touched``: a dict whose lists ``"r"`` and ``"w"`` receive the arena byte offsets this launch reads / writes."""
+    global _TOUCHED
+    _TOUCHED = touched
+    if touched is not None:
+        touched.setdefault("r", [])
+        touched.setdefault("w", [])
+    try:
+        _execute(table, arena, direction, first, count, peers, ordered)
+    finally:
+        _TOUCHED = None
+
+
+def _execute(table, arena, direction, first, count, peers, ordered) -> None:
     global THREADS
     THREADS = int(table.info().tile_threads)
     run_begin, row_begin = table.ranges()
@@ -148,6 +169,8 @@ def execute(table, arena, direction: str, first: int = 0, count: int | None = No
                 assert us == ud
             if arena.writes is not None:
                 np.add.at(arena.writes, do.reshape(-1), 1)
+            _note("r", so)
+            _note("w", do)
             mem[do] = data
 
 
@@ -166,6 +189,8 @@ def _transpose_blocks(arena, trans, rev: bool) -> None:
         do = arena.offsets(dst.reshape(-1), es)[:, None] + np.arange(es)
         if arena.writes is not None:
             np.add.at(arena.writes, do.reshape(-1), 1)
+        _note("r", so)
+        _note("w", do)
         mem[do] = mem[so]
 
 
@@ -189,6 +214,7 @@ def _reduce_units(arena, mem, row_tiles, row_idx, a_off, b, ua, ub, dta, dtb, pe
             assert skew_a or np.all((base + offs) % ua == 0), "misaligned vector access on a peer"
             assert np.all((base + offs) % es == 0), "misaligned element on a peer"
             so = arena.offsets(base + offs, ua)[:, None] + np.arange(ua)
+            _note("r", so)
             staged.append(np.ascontiguousarray(mem[so]).reshape(-1).copy())
         ch = co.make_chunk(0, (0,), (n_units * n_el,), (1,), dta, out_dt, peers=[s.ctypes.data for s in staged], op=op)
         assert co.lib().oracle_reduce(ch, out.ctypes.data, scratch.ctypes.data) == 0
@@ -197,4 +223,5 @@ def _reduce_units(arena, mem, row_tiles, row_idx, a_off, b, ua, ub, dta, dtb, pe
         do = arena.offsets(b[sel], ub)[:, None] + np.arange(ub)
         if arena.writes is not None:
             np.add.at(arena.writes, do.reshape(-1), 1)
+        _note("w", do)
         mem[do] = out.view(np.uint8).reshape(n_units, ub)
