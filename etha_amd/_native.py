@@ -111,6 +111,8 @@ _SIGNATURES = {
     "etha_unpack_bucket": (c_int, [c_void_p, c_uint32, c_uint32, c_void_p, c_uint32]),
     "etha_reduce_pack_bucket": (c_int, [c_void_p, c_uint32, c_uint32, c_void_p, c_uint32]),
     "etha_selfcopy_bucket": (c_int, [c_void_p, c_uint32, c_uint32, c_void_p, c_uint32]),
+    "etha_noalloc_setup": (c_int, []),
+    "etha_copy_regions_noalloc": (c_int, [c_void_p, c_void_p, c_uint32, c_void_p]),
     "etha_arena_create": (c_int, [c_uint64, POINTER(c_void_p)]),
     "etha_arena_destroy": (c_int, [c_void_p]),
     "etha_ipc_export": (c_int, [c_void_p, POINTER(IpcHandle)]),
@@ -272,6 +274,25 @@ class Table:
             self.close()
         except Exception:
             pass
+
+
+NOALLOC_SCRATCH_BYTES = 4 << 20  # ETHA_NOALLOC_SCRATCH_BYTES
+
+
+def noalloc_setup() -> None:
+    """Once per device, with that device current: prepare ``copy_regions_noalloc``."""
+    _check("etha_noalloc_setup", lib().etha_noalloc_setup())
+
+
+def copy_regions_noalloc(src: np.ndarray, dst: np.ndarray, stream: int = 0) -> None:
+    """Copy src region i into dst region i (descriptor arrays as for ``Table.create_selfcopy``) without any device
+    allocation; at most ``NOALLOC_SCRATCH_BYTES`` of tile program per call."""
+    src = np.ascontiguousarray(src, dtype=CHUNK_DESC)
+    dst = np.ascontiguousarray(dst, dtype=CHUNK_DESC)
+    if len(src) != len(dst):
+        raise ValueError("src and dst descriptor arrays differ in length")
+    _check("etha_copy_regions_noalloc",
+           lib().etha_copy_regions_noalloc(src.ctypes.data, dst.ctypes.data, len(src), c_void_p(stream)))
 
 
 def arena_create(nbytes: int) -> int:

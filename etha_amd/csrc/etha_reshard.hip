@@ -1334,6 +1334,114 @@ int etha_selfcopy_bucket(const EthaTable* t, uint32_t first, uint32_t count, voi
   return launch_reduce(t, first, count, stream, flags);
 }
 
+// ---- region copies for callers that cannot allocate --------------------------------------------
+// The tile program of etha_copy_regions_noalloc lives in this array instead of in memory from hipMalloc.
+// Each GPU the library runs on holds its own copy until the process ends.  In host code the name is only
+// a stand-in for the symbol: its device address comes from hipGetSymbolAddress, once per device.
+static __device__ __align__(256) unsigned char scratch[ETHA_NOALLOC_SCRATCH_BYTES];
+
+namespace {
+constexpr int kMaxDevices = 64;
+struct NoAllocState {
+  void* scratch_ptr = nullptr;  // device address of `scratch` on this device
+  void* staging = nullptr;      // pinned host buffer the tile program is assembled in
+  hipEvent_t copied = nullptr;  // the last call's upload has left the staging buffer
+  bool copy_pending = false;
+};
+NoAllocState g_noalloc[kMaxDevices];
+std::mutex g_noalloc_mutex;
+
+int copy_regions_compile(const EthaChunkDesc* src, const EthaChunkDesc* dst, uint32_t n_chunks, Builder& bld) {
+  bld.run.clear();
+  bld.row.clear();
+  bld.trans.clear();
+  bld.payload_bytes = 0;
+  const ReduceSpec none;
+  static const std::vector<uint64_t> no_peers;
+  for (uint32_t i = 0; i < n_chunks; i++) {
+    if (src[i].n_partials || dst[i].n_partials) return fail(ETHA_ERR_UNSUPPORTED, "chunk %u: a region copy has no Partial side", i);
+    Region A, B;
+    int rc = tensor_region(src[i], i, src[i].tensor_ptr, false, &A);
+    if (rc == ETHA_OK) rc = tensor_region(dst[i], i, dst[i].tensor_ptr, false, &B);
+    if (rc == ETHA_OK) rc = compile_pair(bld, i, A, B, src[i].tensor_dtype, dst[i].tensor_dtype, none, no_peers);
+    if (rc != ETHA_OK) return rc;
+  }
+  return ETHA_OK;
+}
+}  // namespace
+
+int etha_noalloc_setup(void) {
+  int dev = 0;
+  HIP_TRY(hipGetDevice(&dev));
+  if (dev < 0 || dev >= kMaxDevices) return fail(ETHA_ERR_UNSUPPORTED, "device index %d is beyond %d", dev, kMaxDevices);
+  std::lock_guard<std::mutex> lock(g_noalloc_mutex);
+  NoAllocState& st = g_noalloc[dev];
+  if (st.scratch_ptr) return ETHA_OK;
+  void* ptr = nullptr;
+  HIP_TRY(hipGetSymbolAddress(&ptr, HIP_SYMBOL(scratch)));
+  if (!ptr) return fail(ETHA_ERR_HIP, "hipGetSymbolAddress returned a null address");
+  void* staging = nullptr;
+  HIP_TRY(hipHostMalloc(&staging, ETHA_NOALLOC_SCRATCH_BYTES, hipHostMallocDefault));
+  hipEvent_t ev = nullptr;
+  hipError_t e = hipEventCreateWithFlags(&ev, hipEventDisableTiming);
+  if (e != hipSuccess) {
+    (void)hipHostFree(staging);
+    return fail(ETHA_ERR_HIP, "hipEventCreateWithFlags: %s", hipGetErrorString(e));
+  }
+  st.staging = staging;
+  st.copied = ev;
+  st.scratch_ptr = ptr;
+  return ETHA_OK;
+}
+
+int etha_copy_regions_noalloc(const EthaChunkDesc* src, const EthaChunkDesc* dst, uint32_t n_chunks, void* stream) {
+  if (n_chunks && (!src || !dst)) return fail(ETHA_ERR_INVALID, "null descriptor array");
+  int dev = 0;
+  HIP_TRY(hipGetDevice(&dev));
+  if (dev < 0 || dev >= kMaxDevices || !g_noalloc[dev].scratch_ptr)
+    return fail(ETHA_ERR_INVALID, "call etha_noalloc_setup() with this device current first");
+  NoAllocState& st = g_noalloc[dev];
+  // host-side compilation reuses this thread's vectors: no heap growth once they have reached their size
+  thread_local Builder bld;
+  const int rc = copy_regions_compile(src, dst, n_chunks, bld);
+  if (rc != ETHA_OK) return rc;
+  const size_t run_bytes = bld.run.size() * sizeof(RunTile);
+  const size_t row_off = (run_bytes + 63) & ~(size_t)63, row_bytes = bld.row.size() * sizeof(RowTile);
+  const size_t trans_off = (row_off + row_bytes + 63) & ~(size_t)63, trans_bytes = bld.trans.size() * sizeof(TransTile);
+  const size_t total = trans_off + trans_bytes;
+  if (total > (size_t)ETHA_NOALLOC_SCRATCH_BYTES)
+    return fail(ETHA_ERR_UNSUPPORTED,
+                "these regions need a tile program of %llu bytes; etha_copy_regions_noalloc holds at most %llu "
+                "(use etha_selfcopy_table_create for larger copies)",
+                (unsigned long long)total, (unsigned long long)ETHA_NOALLOC_SCRATCH_BYTES);
+  if (run_bytes + row_bytes + trans_bytes == 0) return ETHA_OK;
+  if (st.copy_pending) HIP_TRY(hipEventSynchronize(st.copied));  // the previous call's upload still reads the staging buffer
+  uint8_t* stage = static_cast<uint8_t*>(st.staging);
+  if (run_bytes) memcpy(stage, bld.run.data(), run_bytes);
+  if (row_bytes) memcpy(stage + row_off, bld.row.data(), row_bytes);
+  if (trans_bytes) memcpy(stage + trans_off, bld.trans.data(), trans_bytes);
+  uint8_t* base = static_cast<uint8_t*>(st.scratch_ptr);  // the array's memory on this device: never the symbol's name
+  HIP_TRY(hipMemcpyAsync(base, stage, total, hipMemcpyHostToDevice, (hipStream_t)stream));
+  HIP_TRY(hipEventRecord(st.copied, (hipStream_t)stream));
+  st.copy_pending = true;
+  uint32_t es_max = 1;
+  for (const TransTile& tt : bld.trans)
+    if ((1u << tt.es_log2) > es_max) es_max = 1u << tt.es_log2;
+  if (!bld.trans.empty()) {
+    const size_t lds = (size_t)kTransDim * (kTransDim + 1) * es_max;
+    launch_kernel(etha_transpose_kernel<false>, dim3((uint32_t)bld.trans.size()), dim3(64), lds, stream, 0,
+                  (const TransTile*)(base + trans_off));
+    HIP_TRY(hipGetLastError());
+  }
+  const uint32_t n_run = (uint32_t)bld.run.size(), n_row = (uint32_t)bld.row.size();
+  if (n_run + n_row) {
+    launch_kernel(etha_tile_kernel<false>, dim3((n_run + n_row) * kBlocksPerTile), dim3(kBlockThreads), 0, stream, 0,
+                  (const RunTile*)base, n_run, (const RowTile*)(base + row_off));
+    HIP_TRY(hipGetLastError());
+  }
+  return ETHA_OK;
+}
+
 int etha_arena_create(uint64_t nbytes, void** out_ptr) {
   if (!out_ptr || nbytes == 0) return fail(ETHA_ERR_INVALID, "bad arena request");
   *out_ptr = nullptr;

@@ -200,6 +200,24 @@ int etha_reduce_pack_bucket(const EthaTable* table, uint32_t first, uint32_t cou
 int etha_selfcopy_bucket(const EthaTable* table, uint32_t first, uint32_t count, void* stream, uint32_t flags);
 
 /*
+ * Region copies for callers that cannot allocate device memory (code under HIP graph capture, tight serving
+ * loops, harnesses that forbid hipMalloc).  No counterpart in the reference.
+ * etha_copy_regions_noalloc does what etha_selfcopy_table_create + etha_selfcopy_bucket + etha_table_destroy
+ * do - copy src region i into dst region i, converting between their dtypes; no Partial sources - but keeps
+ * the compiled tile program in a fixed array inside the library instead of in memory from hipMalloc, and calls
+ * no hipMalloc / hipFree.  The program of one call may take at most ETHA_NOALLOC_SCRATCH_BYTES (24 bytes per
+ * 16 KiB of contiguous payload, 64 bytes per 16 KiB of short-row payload: roughly 1-2.8 GB per call); larger
+ * requests are refused with ETHA_ERR_UNSUPPORTED.  Every call on a GPU shares that GPU's array and upload
+ * buffer: calls must be issued on one stream, or otherwise ordered so that one call's launches have finished
+ * before the next call is made - calls that overlap on one GPU race.
+ * etha_noalloc_setup must have been called once with the device current (it looks up the array's device
+ * address and allocates the pinned upload buffer; it is the only part that allocates).
+ */
+#define ETHA_NOALLOC_SCRATCH_BYTES (4u << 20)
+int etha_noalloc_setup(void);
+int etha_copy_regions_noalloc(const EthaChunkDesc* src, const EthaChunkDesc* dst, uint32_t n_chunks, void* stream);
+
+/*
  * Bucket-pool memory that can cross a process boundary on the same GPU (the worker <-> agent
  * hand-off the reference does with CUDA-IPC pickling, tensor_bus/client.py:314,
  * tensor_bus/agent.py:608, tensor_bus/utils.py:14-69).  etha_arena_create is a plain
