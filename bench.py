@@ -302,7 +302,12 @@ def main():
         n_unordered = 0
 
     kernels = []
-    if kinds & {"pack", "unpack", "selfcopy", "direct"}:
+    tables = [t for p in (job.wire.plan(b) for bs in (job.send_buckets, job.recv_buckets) for b in bs.values())
+              for t in (p.send_table, p.recv_table, p.local_table) if t is not None]
+    infos = [t.info() for t in tables]
+    if any(i.n_trans_tiles for i in infos):
+        kernels.append("etha_transpose_kernel")
+    if any(i.n_run_tiles + i.n_row_tiles for i in infos) and kinds & {"pack", "unpack", "selfcopy", "direct"}:
         kernels.append("etha_tile_kernel")
     if kinds & {"reduce_pack", "direct_reduce"}:
         kernels.insert(0, "etha_reduce_kernel")

@@ -92,12 +92,38 @@ struct TransTile {   // a 2-D block whose contiguous dim differs between the two
   uint64_t b;        // address of element (j0, k0) on the b side, contiguous along k
   int64_t a_pitch;   // bytes between consecutive k on the a side
   int64_t b_pitch;   // bytes between consecutive j on the b side
-  uint32_t nj, nk;   // extent of the block (<= kTransDim each)
+  uint32_t nj, nk;   // extent of the block (<= trans_dim(element size) each)
   uint32_t es_log2;  // log2 of the element size in bytes
   uint32_t pad;
 };
 static_assert(sizeof(TransTile) == 48, "TransTile layout");
-constexpr uint32_t kTransDim = 64;  // elements per side of a transposing block; one wavefront per block
+// A transposing block is D x D elements, handled by one workgroup of kTransThreads work-items.  D is chosen
+// per element size so that a row of the block is at least 128 bytes on both sides and a full block is a
+// few 16-byte vectors per work-item.  LDS rows are padded to an odd number of 32-bit words.
+#ifndef ETHA_TRANS_THREADS
+#define ETHA_TRANS_THREADS 1024
+#endif
+#ifndef ETHA_TRANS_DIM_A
+#define ETHA_TRANS_DIM_A 128
+#endif
+#ifndef ETHA_TRANS_DIM_B
+#define ETHA_TRANS_DIM_B 128
+#endif
+#ifndef ETHA_TRANS_SUPER
+#define ETHA_TRANS_SUPER 4
+#endif
+constexpr uint32_t kTransThreads = ETHA_TRANS_THREADS;
+// block extent in elements along j (the a side's contiguous dim) and along k (the b side's); half of it for
+// 8-byte elements, which keeps the LDS footprint of a block at 16-66 KB
+__host__ __device__ constexpr uint32_t trans_dim_a(uint32_t es) { return es == 8 ? ETHA_TRANS_DIM_A / 2u : (uint32_t)ETHA_TRANS_DIM_A; }
+__host__ __device__ constexpr uint32_t trans_dim_b(uint32_t es) { return es == 8 ? ETHA_TRANS_DIM_B / 2u : (uint32_t)ETHA_TRANS_DIM_B; }
+__host__ __device__ constexpr uint32_t trans_pitch(uint32_t dim, uint32_t es) {  // LDS row pitch in elements: an odd number of words
+  return dim + (es >= 4 ? 1u : 4u / es);
+}
+__host__ __device__ constexpr uint32_t trans_lds_bytes(uint32_t es) {  // either direction: rows of one side, one row per element of the other
+  const uint32_t fwd = trans_dim_b(es) * trans_pitch(trans_dim_a(es), es) * es, rev = trans_dim_a(es) * trans_pitch(trans_dim_b(es), es) * es;
+  return fwd > rev ? fwd : rev;
+}
 
 // meta bits
 constexpr uint32_t kMetaUaShift = 0;    // 4 bits: log2 bytes per unit, a side
@@ -278,51 +304,114 @@ __global__ __launch_bounds__(ETHA_BLOCK_THREADS) void etha_tile_kernel(const Run
 }
 
 // ---- transposing chunks: staged through LDS -----------------------------------------------------
-// The a side is contiguous along j, the b side along k.  A block of up to 64 x 64 elements is read with
-// the wavefront's 64 work-items along the source's contiguous dim (one full run per instruction), parked
-// in LDS with a padded pitch, and written with the work-items along the destination's contiguous dim.
-// Both global sides therefore move whole cache-line runs; without the staging one side would touch a
-// different line per work-item.
-template <typename E, bool REV>
-__device__ __forceinline__ void transpose_block(const TransTile& t, E* __restrict__ lds) {
-  constexpr uint32_t kPitch = kTransDim + 1;  // padded: conflict-free column reads
+// The a side is contiguous along j, the b side along k.  A full block of D x D elements is read with 16-byte
+// vectors along the source's contiguous dim (consecutive work-items cover one row, then the next row),
+// parked in LDS row by row, and written with 16-byte vectors along the destination's contiguous dim, each
+// vector gathered element by element from LDS.  Both global sides therefore move whole 16-byte vectors in
+// runs of at least 128 bytes; without the staging one side would touch a different line per element.
+// Blocks at the edge of a chunk (fewer than D elements on a side) take the element-wise path.
+template <typename E, uint32_t DX, uint32_t DY>
+__device__ __forceinline__ void transpose_full(uint64_t src, int64_t src_pitch, uint64_t dst, int64_t dst_pitch,
+                                               uint8_t* __restrict__ lds) {
+  // src: DY rows (index y) of DX elements contiguous along x.  dst: DX rows (index x) of DY elements along y.
+  constexpr uint32_t kEs = sizeof(E), kV = 16 / kEs, kVecPerRow = DX / kV, kOutPerRow = DY / kV;
+  constexpr uint32_t kPitchBytes = trans_pitch(DX, kEs) * kEs;  // a multiple of 4
+  constexpr uint32_t kVecs = DY * kVecPerRow, kPerThread = (kVecs + kTransThreads - 1) / kTransThreads;
+  constexpr bool kExact = kVecs % kTransThreads == 0;
   const uint32_t tid = threadIdx.x;
-  if (!REV) {  // a -> b
-    if (tid < t.nj) {
-#pragma unroll 8
-      for (uint32_t k = 0; k < t.nk; k++)
-        lds[k * kPitch + tid] = ld_stream<E>(t.a + (uint64_t)tid * sizeof(E) + (uint64_t)((int64_t)k * t.a_pitch));
+  u32x4 v[kPerThread];
+#pragma unroll
+  for (uint32_t i = 0; i < kPerThread; i++) {
+    const uint32_t q = tid + i * kTransThreads, y = q / kVecPerRow, xv = q % kVecPerRow;
+    if (kExact || q < kVecs) v[i] = ld_stream<u32x4_any>(src + (uint64_t)((int64_t)y * src_pitch) + xv * 16u);
+  }
+#pragma unroll
+  for (uint32_t i = 0; i < kPerThread; i++) {
+    const uint32_t q = tid + i * kTransThreads, y = q / kVecPerRow, xv = q % kVecPerRow;
+    if (!kExact && q >= kVecs) break;
+    uint32_t* row = reinterpret_cast<uint32_t*>(lds + y * kPitchBytes + xv * 16u);
+    row[0] = v[i][0];
+    row[1] = v[i][1];
+    row[2] = v[i][2];
+    row[3] = v[i][3];
+  }
+  __syncthreads();
+  if constexpr (kEs == 2) {
+    // two destination rows at a time: the 32-bit words of 8 source rows hold the elements of columns x and x + 1
+    constexpr uint32_t kPairs = kVecs / 2, kPairsPerThread = (kPairs + kTransThreads - 1) / kTransThreads;
+#pragma unroll
+    for (uint32_t i = 0; i < kPairsPerThread; i++) {
+      const uint32_t q = tid + i * kTransThreads, xp = q / kOutPerRow, yv = q % kOutPerRow;
+      if (kPairs % kTransThreads != 0 && q >= kPairs) break;
+      uint32_t w[8];
+#pragma unroll
+      for (uint32_t e = 0; e < 8; e++) w[e] = *reinterpret_cast<const uint32_t*>(lds + (yv * 8 + e) * kPitchBytes + xp * 4u);
+      u32x4 lo, hi;
+#pragma unroll
+      for (uint32_t p = 0; p < 4; p++) {
+        lo[p] = (w[2 * p] & 0xffffu) | (w[2 * p + 1] << 16);
+        hi[p] = (w[2 * p] >> 16) | (w[2 * p + 1] & 0xffff0000u);
+      }
+      const uint64_t d0 = dst + (uint64_t)((int64_t)(2 * xp) * dst_pitch) + yv * 16u;
+      st_stream<u32x4_any>(d0, lo);
+      st_stream<u32x4_any>(d0 + (uint64_t)dst_pitch, hi);
     }
-    __syncthreads();
-    if (tid < t.nk) {
-#pragma unroll 8
-      for (uint32_t j = 0; j < t.nj; j++)
-        st_stream<E>(t.b + (uint64_t)((int64_t)j * t.b_pitch) + (uint64_t)tid * sizeof(E), lds[tid * kPitch + j]);
-    }
-  } else {  // b -> a
-    if (tid < t.nk) {
-#pragma unroll 8
-      for (uint32_t j = 0; j < t.nj; j++)
-        lds[tid * kPitch + j] = ld_stream<E>(t.b + (uint64_t)((int64_t)j * t.b_pitch) + (uint64_t)tid * sizeof(E));
-    }
-    __syncthreads();
-    if (tid < t.nj) {
-#pragma unroll 8
-      for (uint32_t k = 0; k < t.nk; k++)
-        st_stream<E>(t.a + (uint64_t)tid * sizeof(E) + (uint64_t)((int64_t)k * t.a_pitch), lds[k * kPitch + tid]);
-    }
+    return;
+  }
+#pragma unroll
+  for (uint32_t i = 0; i < kPerThread; i++) {
+    const uint32_t q = tid + i * kTransThreads, x = q / kOutPerRow, yv = q % kOutPerRow;
+    if (!kExact && q >= kVecs) break;
+    Pack<E, kV> out;
+#pragma unroll
+    for (uint32_t e = 0; e < kV; e++)
+      out.set(e, *reinterpret_cast<const E*>(lds + (yv * kV + e) * kPitchBytes + x * kEs));
+    out.store(dst + (uint64_t)((int64_t)x * dst_pitch) + yv * 16u);
   }
 }
 
+template <typename E, uint32_t DX>
+__device__ __forceinline__ void transpose_edge(uint64_t src, int64_t src_pitch, uint32_t nx, uint64_t dst,
+                                               int64_t dst_pitch, uint32_t ny, uint8_t* __restrict__ lds) {
+  // same roles as above with nx <= DX elements per source row and ny <= DY source rows; one element per access
+  constexpr uint32_t kEs = sizeof(E), kPitchBytes = trans_pitch(DX, kEs) * kEs;
+  const uint32_t n = nx * ny;
+  for (uint32_t q = threadIdx.x; q < n; q += kTransThreads) {
+    const uint32_t y = q / nx, x = q - y * nx;
+    *reinterpret_cast<E*>(lds + y * kPitchBytes + x * kEs) =
+        ld_stream<E>(src + (uint64_t)((int64_t)y * src_pitch) + (uint64_t)x * kEs);
+  }
+  __syncthreads();
+  for (uint32_t q = threadIdx.x; q < n; q += kTransThreads) {
+    const uint32_t x = q / ny, y = q - x * ny;
+    st_stream<E>(dst + (uint64_t)((int64_t)x * dst_pitch) + (uint64_t)y * kEs,
+                 *reinterpret_cast<const E*>(lds + y * kPitchBytes + x * kEs));
+  }
+}
+
+template <typename E, bool REV>
+__device__ __forceinline__ void transpose_block(const TransTile& t, uint8_t* __restrict__ lds) {
+  // pack (a -> b): source rows run along j (one row per k); unpack (b -> a): source rows run along k (one per j)
+  constexpr uint32_t kDX = REV ? trans_dim_b(sizeof(E)) : trans_dim_a(sizeof(E));
+  constexpr uint32_t kDY = REV ? trans_dim_a(sizeof(E)) : trans_dim_b(sizeof(E));
+  const uint64_t src = REV ? t.b : t.a, dst = REV ? t.a : t.b;
+  const int64_t src_pitch = REV ? t.b_pitch : t.a_pitch, dst_pitch = REV ? t.a_pitch : t.b_pitch;
+  const uint32_t nx = REV ? t.nk : t.nj, ny = REV ? t.nj : t.nk;
+  if (nx == kDX && ny == kDY)
+    transpose_full<E, kDX, kDY>(src, src_pitch, dst, dst_pitch, lds);
+  else
+    transpose_edge<E, kDX>(src, src_pitch, nx, dst, dst_pitch, ny, lds);
+}
+
 template <bool REV>
-__global__ __launch_bounds__(64) void etha_transpose_kernel(const TransTile* __restrict__ tiles) {
-  extern __shared__ __attribute__((aligned(16))) uint8_t lds_bytes[];  // kTransDim * (kTransDim + 1) elements
+__global__ __launch_bounds__(ETHA_TRANS_THREADS) void etha_transpose_kernel(const TransTile* __restrict__ tiles) {
+  extern __shared__ __attribute__((aligned(16))) uint8_t lds_bytes[];  // trans_lds_bytes(largest element size)
   const TransTile t = tiles[blockIdx.x];
   switch (t.es_log2) {
-    case 0: transpose_block<uint8_t, REV>(t, reinterpret_cast<uint8_t*>(lds_bytes)); break;
-    case 1: transpose_block<uint16_t, REV>(t, reinterpret_cast<uint16_t*>(lds_bytes)); break;
-    case 2: transpose_block<uint32_t, REV>(t, reinterpret_cast<uint32_t*>(lds_bytes)); break;
-    default: transpose_block<uint64_t, REV>(t, reinterpret_cast<uint64_t*>(lds_bytes)); break;
+    case 0: transpose_block<uint8_t, REV>(t, lds_bytes); break;
+    case 1: transpose_block<uint16_t, REV>(t, lds_bytes); break;
+    case 2: transpose_block<uint32_t, REV>(t, lds_bytes); break;
+    default: transpose_block<uint64_t, REV>(t, lds_bytes); break;
   }
 }
 
@@ -664,7 +753,7 @@ class PairCompiler {
 
   // Transposing chunk: no common contiguous dim, but the a side is contiguous along some other dim j while
   // the b side is contiguous along the innermost one.  Such chunks go through the LDS-staged transposing
-  // kernel in blocks of 64 x 64 elements; all other dims are unrolled here.
+  // kernel in blocks of trans_dim_a x trans_dim_b elements; all other dims are unrolled here.
   int try_transposing(bool* done) {
     *done = false;
     if (!(run_elems_ == 1 && plain_ && k_ >= 2 && sb_[k_ - 1] == esb_ && sa_[k_ - 1] != esa_)) return ETHA_OK;
@@ -675,17 +764,32 @@ class PairCompiler {
     if (j < 0 || n_[kk] < 8 || (A_.base % (uint64_t)esa_) != 0 || (B_.base % (uint64_t)esb_) != 0) return ETHA_OK;
     int64_t pos[ETHA_MAX_NDIM] = {0};
     uint64_t off_a = 0, off_b = 0;
+    const int64_t kDimJ = (int64_t)trans_dim_a((uint32_t)esa_), kDimK = (int64_t)trans_dim_b((uint32_t)esa_);
+    const int64_t nbj = (n_[j] + kDimJ - 1) / kDimJ, nbk = (n_[kk] + kDimK - 1) / kDimK;
     do {
-      for (int64_t j0 = 0; j0 < n_[j]; j0 += kTransDim)
-        for (int64_t k0 = 0; k0 < n_[kk]; k0 += kTransDim) {
+      // Launch order.  Blocks are grouped into super-blocks of S x S blocks that are emitted together: blocks
+      // that are neighbours along j read neighbouring pieces of the same source rows, neighbours along k write
+      // neighbouring pieces of the same destination rows, so running them at the same time keeps DRAM pages
+      // open on both sides.  Super-blocks follow diagonals of their grid: row-major order would make everything
+      // in flight read (or write) one narrow column stripe of rows that lie a power of two apart, i.e. the same
+      // few memory channels.
+      const int64_t S = ETHA_TRANS_SUPER;
+      const int64_t nsj = (nbj + S - 1) / S, nsk = (nbk + S - 1) / S;
+      for (int64_t d = 0; d < nsk; d++)
+        for (int64_t sj = 0; sj < nsj; sj++)
+          for (int64_t ij = 0; ij < S; ij++)
+            for (int64_t ik = 0; ik < S; ik++) {
+          const int64_t bj = sj * S + ij, bk = ((sj + d) % nsk) * S + ik;
+          if (bj >= nbj || bk >= nbk) continue;
+          const int64_t j0 = bj * kDimJ, k0 = bk * kDimK;
           TransTile t;
           memset(&t, 0, sizeof(t));
           t.a = A_.base + off_a + (uint64_t)(j0 * sa_[j]) + (uint64_t)(k0 * sa_[kk]);
           t.b = B_.base + off_b + (uint64_t)(j0 * sb_[j]) + (uint64_t)(k0 * sb_[kk]);
           t.a_pitch = sa_[kk];
           t.b_pitch = sb_[j];
-          t.nj = (uint32_t)(n_[j] - j0 < kTransDim ? n_[j] - j0 : kTransDim);
-          t.nk = (uint32_t)(n_[kk] - k0 < kTransDim ? n_[kk] - k0 : kTransDim);
+          t.nj = (uint32_t)(n_[j] - j0 < kDimJ ? n_[j] - j0 : kDimJ);
+          t.nk = (uint32_t)(n_[kk] - k0 < kDimK ? n_[kk] - k0 : kDimK);
           t.es_log2 = (uint32_t)log2u((uint64_t)esa_);
           bld_.trans.push_back(t);
         }
@@ -894,7 +998,7 @@ struct EthaTable {
   RunTile* d_run = nullptr;
   RowTile* d_row = nullptr;
   TransTile* d_trans = nullptr;
-  uint32_t trans_es_max = 1;  // largest element size among the transposing tiles (sizes the LDS)
+  uint32_t trans_lds = 0;  // LDS bytes the transposing tiles need (largest over their element sizes)
   uint64_t* d_peers = nullptr;
   uint32_t n_chunks = 0;
   uint64_t payload_bytes = 0;
@@ -962,7 +1066,7 @@ int finish_table(Builder& bld, EthaTable* t, int upload, EthaTable** out) {
   t->row_begin.swap(bld.row_begin);
   t->trans_begin.swap(bld.trans_begin);
   for (const TransTile& tt : t->h_trans)
-    if ((1u << tt.es_log2) > t->trans_es_max) t->trans_es_max = 1u << tt.es_log2;
+    if (trans_lds_bytes(1u << tt.es_log2) > t->trans_lds) t->trans_lds = trans_lds_bytes(1u << tt.es_log2);
   t->reduce_prefix.assign(t->n_chunks + 1, 0);
   for (uint32_t i = 0; i < t->n_chunks; i++) t->reduce_prefix[i + 1] = t->reduce_prefix[i] + bld.is_reduce[i];
   t->payload_bytes = bld.payload_bytes;
@@ -1007,8 +1111,8 @@ int launch_tiles(const EthaTable* t, uint32_t first, uint32_t count, void* strea
   const uint32_t n_run = r1 - r0, n_row = w1 - w0;
   const uint32_t x0 = t->trans_begin[first], n_trans = t->trans_begin[first + count] - x0;
   if (n_trans) {  // transposing chunks run in their own kernel (it needs LDS)
-    const size_t lds = (size_t)kTransDim * (kTransDim + 1) * t->trans_es_max;
-    launch_kernel(etha_transpose_kernel<REV>, dim3(n_trans), dim3(64), lds, stream, flags, (const TransTile*)(t->d_trans + x0));
+    launch_kernel(etha_transpose_kernel<REV>, dim3(n_trans), dim3(kTransThreads), t->trans_lds, stream, flags,
+                  (const TransTile*)(t->d_trans + x0));
     HIP_TRY(hipGetLastError());
     flags |= ETHA_LAUNCH_UNORDERED;  // the two kernels of one call touch different chunks
   }
@@ -1424,12 +1528,11 @@ int etha_copy_regions_noalloc(const EthaChunkDesc* src, const EthaChunkDesc* dst
   HIP_TRY(hipMemcpyAsync(base, stage, total, hipMemcpyHostToDevice, (hipStream_t)stream));
   HIP_TRY(hipEventRecord(st.copied, (hipStream_t)stream));
   st.copy_pending = true;
-  uint32_t es_max = 1;
+  uint32_t lds = 0;
   for (const TransTile& tt : bld.trans)
-    if ((1u << tt.es_log2) > es_max) es_max = 1u << tt.es_log2;
+    if (trans_lds_bytes(1u << tt.es_log2) > lds) lds = trans_lds_bytes(1u << tt.es_log2);
   if (!bld.trans.empty()) {
-    const size_t lds = (size_t)kTransDim * (kTransDim + 1) * es_max;
-    launch_kernel(etha_transpose_kernel<false>, dim3((uint32_t)bld.trans.size()), dim3(64), lds, stream, 0,
+    launch_kernel(etha_transpose_kernel<false>, dim3((uint32_t)bld.trans.size()), dim3(kTransThreads), lds, stream, 0,
                   (const TransTile*)(base + trans_off));
     HIP_TRY(hipGetLastError());
   }

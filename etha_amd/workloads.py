@@ -98,6 +98,32 @@ def moe_experts_and_uneven_vocab(n_experts: int = 8, hidden: int = 4096, inter: 
     return specs, [0], 64 * MIB
 
 
+def moe_experts_row_parallel_w2(n_experts: int = 8, hidden: int = 4096, inter: int = 14336, dtype=torch.bfloat16):
+    """The second reading of the expert layout: ``w2`` [E, H, I] as a true row-parallel weight, expert
+    Shard(0)@8 -> TP=4 Shard(2): every target rank takes I/4 = 3584 columns, i.e. rows of 7168 bytes at a
+    28672-byte pitch inside each source expert (w1/w3 stay column-parallel, Shard(1))."""
+    src, tgt = _mesh(0, (8,)), _mesh(0, (4,))
+    specs = [
+        TensorSpec("experts.w1", (n_experts, inter, hidden), src, (Shard(0),), tgt, (Shard(1),), dtype, seed=0),
+        TensorSpec("experts.w3", (n_experts, inter, hidden), src, (Shard(0),), tgt, (Shard(1),), dtype, seed=1),
+        TensorSpec("experts.w2", (n_experts, hidden, inter), src, (Shard(0),), tgt, (Shard(2),), dtype, seed=2),
+    ]
+    return specs, [0], 64 * MIB
+
+
+def transposed_parents(n_tensors: int = 16, n: int = 8192, dtype=torch.bfloat16, target_transposed: bool = False):
+    """16 bf16 [8192, 8192] weights whose source shards are ``.t()`` views (stored [in, out], handed over as
+    [out, in]): mesh (4,) Shard(0) -> mesh (2,) Shard(0), one target rank.  The contiguous dim differs between
+    shard and bucket, so every chunk goes through the LDS-staged transposing kernel."""
+    src, tgt = _mesh(0, (4,)), _mesh(4, (2,))
+    specs = [
+        TensorSpec(f"w{i}", (n, n), src, (Shard(0),), tgt, (Shard(0),), dtype, seed=i, source_layout="transposed",
+                   target_layout="transposed" if target_transposed else "contiguous")
+        for i in range(n_tensors)
+    ]
+    return specs, [4], 64 * MIB
+
+
 def llama3_8b_fsdp8_to_tp2_fp32_to_bf16():
     """Same layouts with fp32 source shards and bf16 target shards (trainer master weights -> serving
     weights): the wire dtype is bf16, so the pack kernel converts."""
@@ -111,4 +137,6 @@ WORKLOADS = {
     "many_small_2d_to_replicate": many_small_2d_to_replicate,
     "partial4_to_shard2": partial4_to_shard2,
     "moe_experts_and_uneven_vocab": moe_experts_and_uneven_vocab,
+    "moe_experts_row_parallel_w2": moe_experts_row_parallel_w2,
+    "transposed_parents": transposed_parents,
 }

@@ -35,6 +35,11 @@ class TensorSpec:
     seed: int = 0
     std: float = 0.02
     dist: str = "normal"  # "normal" | "uniform" (uniform(-1, 1))
+    # storage of the local shards: "contiguous", or "transposed" - a 2-D shard is the ``.t()`` view of a
+    # contiguous [cols, rows] tensor (a trainer that keeps a weight in [in, out] order hands over such views;
+    # non-contiguous parents are legal, tests/test_communication_replicate_shard.py:99-113)
+    source_layout: str = "contiguous"
+    target_layout: str = "contiguous"
 
 
 def transfer_dtype_rule(source: torch.dtype, target: torch.dtype) -> torch.dtype:
@@ -74,6 +79,15 @@ def create_partial_groups(mesh, partial_reductions, this_rank: int, tensors_by_r
 
 def _flat_ranks(mesh) -> list[int]:
     return [int(r) for r in np.asarray(mesh).reshape(-1)]
+
+
+def _as_transposed(t: torch.Tensor) -> torch.Tensor:
+    """The same values as a ``.t()`` view of a contiguous [cols, rows] tensor (2-D tensors only)."""
+    if t.dim() != 2:
+        return t
+    out = torch.empty(t.shape[1], t.shape[0], dtype=t.dtype, device=t.device).t()
+    out.copy_(t)
+    return out
 
 
 def make_global(spec: TensorSpec, device, seed: int | None = None, shape=None) -> torch.Tensor:
@@ -155,6 +169,8 @@ class ReshardJob:
                 for pos, r in enumerate(src_ranks):
                     view = local_shard(glob, src_mesh.shape, spec.source_placements, mesh_coord(src_mesh.shape, pos))
                     src_local[r] = view.clone(memory_format=torch.contiguous_format)
+            if spec.source_layout == "transposed":
+                src_local = {r: _as_transposed(t) for r, t in src_local.items()}
             if self.local_view is not None:
                 src_local = {r: self._rehome("source", t) for r, t in src_local.items()}
             tgt_local: dict[int, torch.Tensor] = {}
@@ -163,6 +179,8 @@ class ReshardJob:
                     continue
                 shape = local_shape(spec.shape, tgt_mesh.shape, spec.target_placements, mesh_coord(tgt_mesh.shape, pos))
                 tgt_local[r] = torch.zeros(shape, dtype=tgt_dtype, device=self.device)
+                if spec.target_layout == "transposed":
+                    tgt_local[r] = _as_transposed(tgt_local[r])
                 if self.local_view is not None:
                     tgt_local[r] = self._rehome("target", tgt_local[r])
             self.source_locals.append(src_local)

@@ -457,6 +457,48 @@ def test_moe_experts_and_uneven_vocab_full_size_properties(gpu_device):
     _check_targets_against_global(job, specs)
 
 
+@pytest.mark.parametrize("target_transposed", [False, True])
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float32, torch.int8, torch.float64])
+def test_transposed_parents_small(gpu_device, dtype, target_transposed):
+    """Shards that are ``.t()`` views on one or both sides: full 16-byte-vector blocks and element-wise edge
+    blocks of the transposing kernel, against the oracle."""
+    specs, targets, _ = workloads.transposed_parents(n_tensors=2, n=776, dtype=dtype, target_transposed=target_transposed)
+    for s in specs:
+        s.dist = "bits"
+    job, _ = gpu_vs_oracle(specs, gpu_device, 256 * 1024, target_ranks=targets)
+    assert not job.source_locals[0][0].is_contiguous()
+    assert all(job.wire.plan(b).send_table.info().n_trans_tiles > 0 for b in job.send_buckets.values())
+    recv = job.wire.plan(job.recv_buckets[4]).recv_table.info()
+    assert (recv.n_trans_tiles > 0) == target_transposed
+
+
+def test_transposed_parents_full_size_properties(gpu_device):
+    """16 bf16 [8192, 8192] weights handed over as ``.t()`` views: every target shard equals its slice of the
+    global tensor, the (non-contiguous) sources are unchanged."""
+    specs, targets, bucket = workloads.transposed_parents()
+    job = ReshardJob(specs, device=gpu_device, bucket_size=bucket, target_ranks=targets, keep_globals=True)
+    assert job.payload_bytes() == 16 * 8192 * 4096 * 2
+    sums = [{r: t.view(torch.int16).sum(dtype=torch.int64).item() for r, t in d.items()} for d in job.source_locals]
+    job.run(merge_launches=True)
+    _check_targets_against_global(job, specs)
+    for i, d in enumerate(job.source_locals):
+        for r, t in d.items():
+            assert t.view(torch.int16).sum(dtype=torch.int64).item() == sums[i][r], "source mutated"
+
+
+def test_moe_row_parallel_w2(gpu_device):
+    """The expert layout's second reading - w2 [E, H, I] row-parallel, Shard(0)@8 -> Shard(2)@4 (rows of I/4
+    elements at a pitch of I) - scaled down against the oracle, then at full size through the closed form."""
+    specs, _, _ = workloads.moe_experts_row_parallel_w2(n_experts=8, hidden=64, inter=224)
+    gpu_vs_oracle(specs, gpu_device, 32 * 1024, target_ranks=[0, 1, 2, 3])
+    specs, _, bucket = workloads.moe_experts_row_parallel_w2()
+    job = ReshardJob(specs, device=gpu_device, bucket_size=bucket, target_ranks=[0, 1, 2, 3], keep_globals=True)
+    job.run(merge_launches=True)
+    _check_targets_against_global(job, specs)
+    w2 = [c for b in job.recv_buckets[1] for c in b.chunks if c.tensor is job.target_locals[2][1]]
+    assert w2 and all(c.chunk_shape == (1, 4096, 3584) for c in w2)  # 7168-byte rows
+
+
 def test_per_bucket_launches_on_side_streams(gpu_device):
     """Fan-out over side streams (fork/join with events) gives the same bytes as one stream."""
     specs, targets, _ = workloads.llama3_8b_fsdp8_to_tp2(n_layers=3, hidden=256, inter=896, kv=64, vocab=2056)

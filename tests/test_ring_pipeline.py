@@ -113,6 +113,23 @@ def test_partial_and_self_copy_through_a_ring(op):
     assert check.unordered > 0
 
 
+@pytest.mark.parametrize("name,kw", [
+    ("transposed_parents", dict(n_tensors=2, n=392)),
+    ("transposed_parents", dict(n_tensors=2, n=392, target_transposed=True, dtype=torch.float32)),
+    ("transposed_parents", dict(n_tensors=1, n=264, target_transposed=True, dtype=torch.float64)),
+    ("transposed_parents", dict(n_tensors=1, n=520, dtype=torch.int8)),
+    ("moe_experts_row_parallel_w2", dict(n_experts=8, hidden=64, inter=224)),
+])
+def test_other_workloads_scaled_down(name, kw):
+    """Transposed parents (LDS-staged blocks, full and edge, every element size) and the row-parallel expert
+    layout, through the planner, the tile compiler and the interpreter."""
+    specs, targets, _ = workloads.WORKLOADS[name](**kw)
+    job, ref = _jobs(specs, 64 * 1024, 2, targets)
+    _interpret(job, False)
+    run_oracle(ref)
+    _compare(job, ref, specs, name)
+
+
 def test_missing_ordering_is_caught_by_the_byte_check(monkeypatch):
     """The byte-level check must fail when the wire forgets what earlier launches touched."""
     specs, targets, _ = workloads.llama3_8b_fsdp8_to_tp2(n_layers=2, hidden=64, inter=224, kv=16, vocab=520)

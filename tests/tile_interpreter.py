@@ -179,7 +179,7 @@ def _transpose_blocks(arena, trans, rev: bool) -> None:
     for t in trans:
         es = 1 << int(t["es_log2"])
         nj, nk = int(t["nj"]), int(t["nk"])
-        assert 0 < nj <= 64 and 0 < nk <= 64
+        assert 0 < nj <= 512 and 0 < nk <= 512  # block side: a fixed number of bytes per row
         j, k = np.meshgrid(np.arange(nj), np.arange(nk), indexing="ij")
         a = int(t["a"]) + j * es + k * int(t["a_pitch"])
         b = int(t["b"]) + j * int(t["b_pitch"]) + k * es
