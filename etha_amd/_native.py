@@ -97,6 +97,7 @@ class EthaNativeError(RuntimeError):
 _SIGNATURES = {
     "etha_abi_version": (c_int, []),
     "etha_last_error": (c_char_p, []),
+    "etha_source_hash": (c_char_p, []),
     "etha_table_create": (c_int, [c_void_p, c_uint32, c_void_p, c_uint32, c_int, POINTER(c_void_p)]),
     "etha_selfcopy_table_create": (c_int, [c_void_p, c_void_p, c_uint32, c_int, POINTER(c_void_p)]),
     "etha_direct_table_create": (c_int, [c_void_p, c_void_p, c_uint32, c_void_p, c_uint32, c_int, POINTER(c_void_p)]),

@@ -6,6 +6,8 @@
 
 from __future__ import annotations
 
+import ctypes
+import hashlib
 import os
 import shutil
 import subprocess
@@ -36,9 +38,32 @@ def hipcc_path() -> str:
     return path
 
 
+HEADER = os.path.join(INCLUDE_DIR, "etha_reshard.h")
+
+
+def source_hash() -> str:
+    """Digest of the sources the library is built from; the library carries the one it was built with."""
+    h = hashlib.sha256()
+    for path in (SOURCE, HEADER):
+        with open(path, "rb") as f:
+            h.update(f.read())
+    return h.hexdigest()[:32]
+
+
+def library_hash(path: str) -> str | None:
+    """The source digest a built library reports (None for a library that predates it or cannot be loaded)."""
+    try:
+        fn = ctypes.CDLL(path).etha_source_hash
+    except (OSError, AttributeError):
+        return None
+    fn.restype = ctypes.c_char_p
+    return fn().decode()
+
+
 def build_library(verbose: bool = False, defines: tuple[str, ...] = (), out_path: str | None = None) -> str:
     """Compile the shared library (always recompiles) and return its path."""
     out_path = out_path or LIB_PATH
+    defines = (*defines, f'ETHA_SOURCE_HASH="{source_hash()}"')
     cmd = [hipcc_path(), *HIPCC_FLAGS, *[f"-D{d}" for d in defines], f"-I{INCLUDE_DIR}", "-o", out_path + ".tmp", SOURCE]
     proc = subprocess.run(cmd, capture_output=True, text=True)
     if proc.returncode != 0:
@@ -50,9 +75,18 @@ def build_library(verbose: bool = False, defines: tuple[str, ...] = (), out_path
 
 
 def ensure_built() -> str:
-    """Build the library only if none is there (test / benchmark harnesses; the product itself never builds:
-    ``etha_amd._native.lib()`` raises when the library is missing)."""
-    return LIB_PATH if os.path.exists(LIB_PATH) else build_library()
+    """Build the library only if none is there, or if the one there was built from other sources than the
+    ones in the tree (test / benchmark harnesses; the product itself never builds: ``etha_amd._native.lib()``
+    raises when the library is missing)."""
+    if not os.path.exists(LIB_PATH):
+        return build_library()
+    if os.environ.get("ETHA_AMD_LIB"):
+        return LIB_PATH  # an explicitly selected build (kernel tuning experiments) is taken as it is
+    built_from = library_hash(LIB_PATH)
+    if built_from != source_hash():
+        sys.stderr.write(f"[etha_amd.build] {LIB_PATH} was built from other sources ({built_from}); rebuilding\n")
+        return build_library()
+    return LIB_PATH
 
 
 if __name__ == "__main__":

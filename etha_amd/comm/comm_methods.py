@@ -180,7 +180,7 @@ class TransferPlan:
                 read_from = frozenset((slot.ptr,)) if not slot.borrowed else _storages([slot.keepalive])
                 self._add(_UNPACK, first, len(bucket.chunks), slot, StepInfo(bucket, entry=entry, reads=read_from, writes=dsts))
         self._keepalive = send.keepalive + recv.keepalive + local.keepalive
-        self.merged_steps = self._merge(self.steps)
+        self.merged_steps = self._merge(self.steps, self.info)
         self.send_table = self.recv_table = self.local_table = None
         if self.device is None:
             return
@@ -237,19 +237,30 @@ class TransferPlan:
                 self.local_table.optimize_range(first, count)
 
     @staticmethod
-    def _merge(steps):
+    def _merge(steps, info=None):
+        """Fuse consecutive steps of one kind whose chunk ranges are adjacent.  A step that reads an allocation
+        an earlier step of the run writes (or the other way round) - two self-copy buckets inside one tensor -
+        starts a new launch, so that it still runs after the earlier one, as it does unmerged."""
         merged: list[list] = []
+        touched: list[tuple[set, set]] = []  # per merged launch: allocations read / written
         lends = [s[3] for s in steps if s[0] == _LEND]
         if lends:  # nothing is launched for them; keep them out of the way of merging their neighbours
             merged.append([_LEND, 0, 0, list(lends)])
-        for kind, first, count, slot in steps:
+            touched.append((set(), set()))
+        for i, (kind, first, count, slot) in enumerate(steps):
             if kind == _LEND:
                 continue
-            if merged and merged[-1][0] == kind and merged[-1][1] + merged[-1][2] == first:
+            reads = set(info[i].reads) if info is not None else set()
+            writes = set(info[i].writes) if info is not None else set()
+            if merged and merged[-1][0] == kind and merged[-1][1] + merged[-1][2] == first \
+                    and not (reads & touched[-1][1]) and not (writes & touched[-1][0]):
                 merged[-1][2] += count
                 merged[-1][3].append(slot)
+                touched[-1][0].update(reads)
+                touched[-1][1].update(writes)
             else:
                 merged.append([kind, first, count, [slot]])
+                touched.append((reads, writes))
         return [(k, f, c, tuple(s)) for k, f, c, s in merged]
 
     def order_by_written_address(self, kind: str, first: int, count: int) -> None:
@@ -341,15 +352,30 @@ class TransferPlan:
         for s in side:
             s.wait_event(fork)
         lane_of_slot: dict[int, int] = {}
+        lane_of_alloc: dict[int, int] = {}  # allocations written by a self-copy: later steps that touch them follow it
+        local = [(f, info.reads | info.writes, info.writes)
+                 for (k, f, _, _), info in zip(self.steps, self.info) if k == _SELF]
 
         def pick(i, slots):
             key = id(slots[0]) if slots and slots[0] is not None else None
+            kind, first, count = steps[i][0], steps[i][1], steps[i][2]
+            touched, written = set(), set()
+            if kind == _SELF:
+                for f, t, w in local:
+                    if first <= f < first + count:
+                        touched |= t
+                        written |= w
+            follow = [lane_of_alloc[a] for a in touched if a in lane_of_alloc]
             if key is not None and key in lane_of_slot:
                 lane = lane_of_slot[key]
+            elif follow:
+                lane = follow[0]
             else:
                 lane = i % len(side)
-                if key is not None:
-                    lane_of_slot[key] = lane
+            if key is not None:
+                lane_of_slot[key] = lane
+            for a in written:
+                lane_of_alloc[a] = lane
             return side[lane].cuda_stream
 
         with torch.cuda.device(self.device):

@@ -1150,7 +1150,11 @@ int check_flags(uint32_t flags) {
 
 extern "C" {
 
+#ifndef ETHA_SOURCE_HASH
+#define ETHA_SOURCE_HASH "unknown"
+#endif
 int etha_abi_version(void) { return ETHA_ABI_VERSION; }
+const char* etha_source_hash(void) { return ETHA_SOURCE_HASH; }
 const char* etha_last_error(void) { return g_err.c_str(); }
 
 int etha_table_create(const EthaChunkDesc* descs, uint32_t n_chunks, const uint64_t* partial_ptrs,

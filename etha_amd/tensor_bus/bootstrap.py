@@ -17,10 +17,14 @@ logger = logging.getLogger(__name__)
 
 def setup_ptrace() -> None:
     """Allow another process (the agent) to open this process's device allocations."""
-    PR_SET_PTRACER, PR_SET_PTRACER_ANY = 0x59616D61, -1
+    PR_SET_PTRACER = 0x59616D61
+    pr_set_ptracer_any = ctypes.c_ulong(-1)  # (unsigned long)-1: a plain -1 would travel as a 32-bit int
     libc = ctypes.CDLL("libc.so.6", use_errno=True)
-    if libc.prctl(PR_SET_PTRACER, PR_SET_PTRACER_ANY, 0, 0, 0) != 0:
-        logger.error("[Bootstrap] ptrace setup failed")
+    libc.prctl.argtypes = [ctypes.c_int, ctypes.c_ulong, ctypes.c_ulong, ctypes.c_ulong, ctypes.c_ulong]
+    if libc.prctl(PR_SET_PTRACER, pr_set_ptracer_any, 0, 0, 0) != 0:
+        err = ctypes.get_errno()
+        # without Yama ptrace restrictions the call is not needed and fails with EINVAL: hipIPC still works
+        logger.warning("[Bootstrap] prctl(PR_SET_PTRACER, ANY) failed: errno %d (%s)", err, os.strerror(err))
 
 
 @dataclass

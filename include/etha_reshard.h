@@ -111,6 +111,9 @@ typedef struct EthaIpcHandle {
 
 int etha_abi_version(void);
 const char* etha_last_error(void);
+/* digest of the sources (kernel file + this header) the library was built from, as the build recipe passed it;
+ * lets a harness notice a library that is older than the tree.  No counterpart in the reference. */
+const char* etha_source_hash(void);
 
 /*
  * Compile chunk descriptors into a tile program.

@@ -61,7 +61,7 @@ def trainer_process(tmpdir, device, rounds, out_q):
     try:
         import torch
 
-        from etha_amd.layout import local_shard
+        from oracle.dtensor_layout import local_shard  # the pinned convention, not the product's planner
         from etha_amd.tensor_bus import TensorBusClient
         from etha_amd.tensor_bus.bootstrap import setup_ptrace
         from helpers import parse_placements
@@ -114,7 +114,7 @@ def inference_process(tmpdir, device, rounds, out_q):
     try:
         import torch
 
-        from etha_amd.layout import local_shape, local_shard
+        from oracle.dtensor_layout import local_shard  # the pinned convention, not the product's planner
         from etha_amd.tensor_bus import TensorBusClient
         from etha_amd.tensor_bus.bootstrap import setup_ptrace
         from helpers import parse_placements
@@ -125,7 +125,7 @@ def inference_process(tmpdir, device, rounds, out_q):
         locals_ = {r: [] for r in TGT_RANKS}
         for i, (_, shape, _, tgt, _, tdt) in enumerate(BUS_TENSORS):
             for pos, r in enumerate(TGT_RANKS):
-                shp = local_shape(shape, (len(TGT_RANKS),), parse_placements(tgt), (pos,))
+                shp = tuple(local_shard(torch.empty(shape, device="meta"), (len(TGT_RANKS),), parse_placements(tgt), (pos,)).shape)
                 locals_[r].append(torch.full(shp, -1.0, dtype=names[tdt], device=device))
         mismatches = []
 

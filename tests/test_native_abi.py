@@ -137,3 +137,12 @@ def test_missing_library_fails_loudly(tmp_path):
     proc = subprocess.run([sys.executable, "-c", code], capture_output=True, text=True, env=env, timeout=120)
     assert proc.returncode != 0
     assert "is missing: the HIP extension is not built" in proc.stderr and "no CPU fallback" in proc.stderr
+
+
+def test_library_reports_the_sources_it_was_built_from():
+    """The harnesses rebuild a library that is older than the tree: the library carries a digest of its sources."""
+    from etha_amd import build
+
+    assert build.library_hash(build.LIB_PATH) == build.source_hash()
+    assert nat.lib().etha_source_hash().decode() == build.source_hash()
+    assert build.library_hash("libc.so.6") is None  # a library without the symbol counts as stale

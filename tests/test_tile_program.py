@@ -441,3 +441,38 @@ def test_random_descriptors_against_numpy(seed):
     untouched[strided(np.arange(pn), 8)[region].reshape(-1)] = False
     fill = np.frombuffer(bytes([0x5A]) * es, dtype=raw_of[es])[0]
     assert np.all(back[untouched] == fill), "bytes outside the region were written"
+
+
+def test_self_copy_buckets_that_feed_each_other_are_not_merged():
+    """Two LOCAL buckets inside one tensor, the second reading what the first writes: merged launches keep
+    them apart (a merged launch has no order inside), and the interpreter, run in the executor's order,
+    gives the stream-ordered result."""
+    import torch
+
+    from etha_amd.comm import Chunk, LoopbackWire, Transport, chunk_to_bucket_ops
+    from tile_interpreter import AbsoluteMemory
+
+    def chunk(t, src, dst, n):
+        return Chunk(chunk_shape=(n,), transport=Transport.LOCAL, is_source=True, is_target=True, src_rank=0, src_idx=(src // n,),
+                     dst_ranks=(0,), dst_idx=(dst // n,), src_slice=(slice(src, src + n),), dst_slice=(slice(dst, dst + n),),
+                     tensor=t, rank=0)
+
+    t = torch.arange(64, dtype=torch.float32)
+    want = t.clone()
+    want[16:32] = want[0:16]
+    want[32:48] = want[16:32]  # reads what the first copy wrote
+    buckets = chunk_to_bucket_ops([chunk(t, 0, 16, 16), chunk(t, 16, 32, 16)], bucket_size=1)  # one chunk per bucket
+    assert len(buckets) == 2
+    other = torch.zeros(32)
+    independent = chunk_to_bucket_ops([chunk(other, 0, 8, 8), chunk(other, 16, 24, 8)], bucket_size=1)
+    for pool in ("resident", "ring"):
+        wire = LoopbackWire("cpu", host_inspection=True, pool=pool)
+        plan = wire.plan(buckets)
+        assert [s[0] for s in plan.steps] == ["selfcopy", "selfcopy"]
+        assert len(plan.merged_steps) == 2  # not fused: the second launch must run after the first
+        assert len(wire.plan(independent).merged_steps) == 2  # same tensor: kept apart as well (allocation granularity)
+    st = t.untyped_storage()
+    mem = AbsoluteMemory(st.data_ptr(), st.data_ptr() + st.nbytes())
+    for kind, first, count, _ in plan.merged_steps:
+        execute(plan.local_table, mem, "selfcopy", first, count)
+    assert torch.equal(t, want)
