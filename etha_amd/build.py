@@ -6,7 +6,6 @@
 
 from __future__ import annotations
 
-import ctypes
 import hashlib
 import os
 import shutil
@@ -51,13 +50,19 @@ def source_hash() -> str:
 
 
 def library_hash(path: str) -> str | None:
-    """The source digest a built library reports (None for a library that predates it or cannot be loaded)."""
+    """The source digest a built library carries, read from the file (the library is not loaded: it must only
+    ever be loaded after torch, so that both use one HIP runtime).  None for a library without one."""
+    marker = b"etha-source-digest:"
     try:
-        fn = ctypes.CDLL(path).etha_source_hash
-    except (OSError, AttributeError):
+        with open(path, "rb") as f:
+            blob = f.read()
+    except OSError:
         return None
-    fn.restype = ctypes.c_char_p
-    return fn().decode()
+    at = blob.find(marker)
+    if at < 0:
+        return None
+    end = blob.find(b"\0", at)
+    return blob[at + len(marker):end].decode(errors="replace")
 
 
 def build_library(verbose: bool = False, defines: tuple[str, ...] = (), out_path: str | None = None) -> str:

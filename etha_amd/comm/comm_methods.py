@@ -12,7 +12,8 @@ programs (:class:`TransferPlan`) and a transfer walks the same per-channel pipel
 * ``is_complete`` of a target bucket is "its send bucket has been packed", and its ``finalize`` is one
   unpack launch; ``is_complete`` of a source bucket is "every destination has unpacked";
 * LOCAL buckets: one direct self-copy launch, or pack + unpack through a private slot when source and
-  destination bytes may overlap;
+  destination bytes may overlap; for a Partial source the launch combines the members straight into the
+  target region;
 * NONE buckets: nothing - the primary's reduce-pack already read this member's partial;
 * with the wire's ``zero_copy_single_chunk`` option, a single-chunk source bucket whose bytes already lie
   contiguously in the tensor is lent, not packed: the consumer unpacks straight from the tensor;
@@ -41,8 +42,8 @@ from .transfer import Transport
 
 __all__ = ["bucket_comm", "TransferPlan", "Program"]
 
-_PACK, _REDUCE, _UNPACK, _SELF, _LEND, _DIRECT, _DIRECT_REDUCE = (
-    "pack", "reduce_pack", "unpack", "selfcopy", "lend", "direct", "direct_reduce")
+_PACK, _REDUCE, _UNPACK, _SELF, _LEND, _DIRECT, _DIRECT_REDUCE, _SELF_REDUCE = (
+    "pack", "reduce_pack", "unpack", "selfcopy", "lend", "direct", "direct_reduce", "selfcopy_reduce")
 
 
 @dataclass
@@ -123,9 +124,12 @@ class TransferPlan:
                     self._add(_UNPACK, f_recv, len(bucket.chunks), slot, StepInfo(bucket, reads=sid, writes=_storages(dsts)))
                 else:
                     first = len(local)
+                    reduce = bool(bucket.chunks[0].source_partial_groups)  # buckets never mix Partial and plain chunks
                     for c in bucket.chunks:
                         local.add_chunk(c)
-                    self._add(_SELF, first, len(bucket.chunks), None,
+                        if reduce:
+                            srcs.extend(c.partial_peers()[0])
+                    self._add(_SELF_REDUCE if reduce else _SELF, first, len(bucket.chunks), None,
                               StepInfo(bucket, reads=_storages(srcs), writes=_storages(dsts)))
                 continue
             if bucket.is_source:
@@ -208,7 +212,7 @@ class TransferPlan:
             return self.send_table
         if kind == _UNPACK:
             return self.recv_table
-        if kind in (_SELF, _DIRECT, _DIRECT_REDUCE):
+        if kind in (_SELF, _SELF_REDUCE, _DIRECT, _DIRECT_REDUCE):
             return self.local_table
         return None
 
@@ -281,7 +285,7 @@ class TransferPlan:
             self.send_table.reduce_pack(first, count, stream, flags)
         elif kind == _UNPACK:
             self.recv_table.unpack(first, count, stream, flags)
-        elif kind in (_SELF, _DIRECT, _DIRECT_REDUCE):
+        elif kind in (_SELF, _SELF_REDUCE, _DIRECT, _DIRECT_REDUCE):
             self.local_table.selfcopy(first, count, stream, flags)
 
     # ---- resident pool: the bucket list in list order -------------------------------------------------

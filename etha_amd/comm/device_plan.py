@@ -41,6 +41,17 @@ def check_cast(src: torch.dtype, dst: torch.dtype) -> None:
         raise NotImplementedError(f"conversion {src} -> {dst} is only implemented between floating dtypes")
 
 
+def reduce_op_word(op) -> int:
+    """``reduce_op`` of a descriptor: the op's code, or ``ETHA_REDUCE_LEVELS`` for ``((op, size), ...)`` levels."""
+    if isinstance(op, str):
+        return nat.REDUCE_OPS[op]
+    ops = [nat.REDUCE_OPS[o] for o, _ in op]
+    sizes = [n for _, n in op]
+    if len(op) == 2:  # two levels: the outer one takes what the inner one leaves
+        return ops[0] | (ops[1] << 3) | (ops[1] << 6) | (sizes[0] << 16) | (1 << 24)
+    return ops[0] | (ops[1] << 3) | (ops[2] << 6) | (sizes[0] << 16) | (sizes[1] << 24)
+
+
 def _storage_range(t) -> tuple[int, int]:
     st = t.untyped_storage()
     lo = st.data_ptr()
@@ -141,7 +152,7 @@ class DescBuilder:
                     raise NotImplementedError("Partial peers must live on the same device")
             row["n_partials"] = len(tensors)
             row["partial_first"] = len(self.partial_ptrs)
-            row["reduce_op"] = nat.REDUCE_OPS[op]
+            row["reduce_op"] = reduce_op_word(op)
             self.partial_ptrs.extend(t.data_ptr() for t in tensors)
             self.keepalive.extend(tensors)
         self.keepalive.append(tensor)
@@ -169,7 +180,9 @@ class SelfCopyBuilder:
 
     def add_chunk(self, chunk: Chunk) -> None:
         src_t = chunk.src_tensor if chunk.src_tensor is not None else chunk.tensor
-        self.add_pair(src_t, chunk.src_slice, chunk.tensor, chunk.dst_slice, chunk.chunk_shape)
+        # a same-rank chunk of a Partial source: the members are combined straight into the target region
+        self.add_pair(src_t, chunk.src_slice, chunk.tensor, chunk.dst_slice, chunk.chunk_shape,
+                      peers=chunk.partial_peers(), wire_dtype=chunk.transfer_dtype)
 
     def add_pair(self, src_t, src_slice: tuple, dst_t, dst_slice: tuple, chunk_shape: tuple, peers=None,
                  wire_dtype: torch.dtype | None = None) -> None:
@@ -196,7 +209,7 @@ class SelfCopyBuilder:
             a["wire_dtype"] = dtype_code(wire)
             a["n_partials"] = len(tensors)
             a["partial_first"] = len(self.partial_ptrs)
-            a["reduce_op"] = nat.REDUCE_OPS[op]
+            a["reduce_op"] = reduce_op_word(op)
             self.partial_ptrs.extend(t.data_ptr() for t in tensors)
             self.keepalive.extend(tensors)
         self.src.append(a)
@@ -275,6 +288,8 @@ def local_bucket_needs_staging(bucket: Bucket) -> bool:
         src_t = c.src_tensor if c.src_tensor is not None else c.tensor
         srcs.append(region_hull(src_t, c.src_slice))
         dsts.append(region_hull(c.tensor, c.dst_slice))
+    if bucket.chunks[0].source_partial_groups:
+        return False  # the members' partials are separate tensors from the target
     if len(bucket.chunks) == 1:
         return False  # single-entry path of the reference copies directly (ir.py:238-244)
     for s_lo, s_hi in srcs:

@@ -82,8 +82,9 @@ def _partial_signature(m2m: M2MMap, src_rank: int) -> tuple:
     for mesh_dim, _ in m2m.source_partial_reductions:
         index[mesh_dim] = slice(None)
     ranks = tuple(sorted(int(r) for r in np.asarray(mesh[tuple(index)]).reshape(-1)))
-    ops = {op for _, op in m2m.source_partial_reductions}
-    return ((ranks, ops.pop()),) if len(ops) == 1 else ()
+    ops = [op for _, op in sorted(m2m.source_partial_reductions)]
+    # one op, or one per Partial mesh dim: either way chunks of this reduction only bundle with each other
+    return ((ranks, ops[0] if len(set(ops)) == 1 else "+".join(ops)),)
 
 
 def _shape_of(slices: tuple[slice, ...]) -> tuple[int, ...]:
@@ -151,8 +152,6 @@ def m2m_to_chunks(
                     raise ValueError(
                         f"rank {rank} is both source and destination of cell {src_idx}: pass source_tensor too"
                     )
-                if source_partial_groups:
-                    raise NotImplementedError("same-rank delivery of a Partial source is not supported")
                 chunks.append(
                     Chunk(
                         chunk_shape=_shape_of(dst_slices),
@@ -167,6 +166,8 @@ def m2m_to_chunks(
                         dst_slice=dst_slices,
                         tensor=target_tensor,
                         src_tensor=source_tensor,
+                        # a Partial source delivered to its own rank: the members are combined into the target region
+                        source_partial_groups=source_partial_groups,
                         rank=rank,
                     )
                 )

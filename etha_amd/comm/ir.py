@@ -74,17 +74,31 @@ class PartialGroup:
     ``ranks`` are in ascending order; ``tensors[i]`` is rank ``ranks[i]``'s local partial
     tensor.  Stands in for the ``ProcessGroup`` of ``Chunk.source_partial_groups`` (``ir.py:84``):
     the reduce kernel reads the peers directly instead of running a collective.
+
+    ``levels`` describes Partial mesh dims with *different* reduce ops: ``((op, size), ...)`` from the
+    first-applied mesh dim to the last, ``ranks``/``tensors`` then listed with the first-applied dim
+    varying fastest (not ascending).  The reference all-reduces once per such dim, each with its own op,
+    in mesh-dim order (``tensor_bus/agent.py:46-70``, ``ir.py:123-124``).
     """
 
     ranks: tuple[int, ...]
     tensors: tuple[torch.Tensor, ...]
+    levels: tuple = ()
 
     def __post_init__(self) -> None:
         self.ranks = tuple(self.ranks)
         self.tensors = tuple(self.tensors)
+        self.levels = tuple((str(op), int(n)) for op, n in self.levels)
         if len(self.ranks) != len(self.tensors):
             raise ValueError("PartialGroup needs one tensor per rank")
-        if list(self.ranks) != sorted(self.ranks):
+        if self.levels:
+            if not 2 <= len(self.levels) <= 3:
+                raise NotImplementedError("between two and three Partial mesh dims with different ops are supported")
+            if math.prod(n for _, n in self.levels) != len(self.ranks):
+                raise ValueError("PartialGroup levels do not multiply up to the number of members")
+            if any(op not in REDUCE_OPS for op, _ in self.levels) or any(not 1 <= n <= 255 for _, n in self.levels):
+                raise ValueError(f"bad PartialGroup levels {self.levels}")
+        elif list(self.ranks) != sorted(self.ranks):
             raise ValueError("PartialGroup ranks must be ascending (reduction order is rank order)")
 
 
@@ -128,7 +142,7 @@ class Chunk:
     def partial_signature(self) -> tuple:
         if not self.source_partial_groups:
             return tuple(self.source_partial_signature)
-        return tuple((g.ranks, op) for g, op in self.source_partial_groups)
+        return tuple((g.ranks, op, g.levels) for g, op in self.source_partial_groups)
 
     @property
     def bucket_key(self) -> tuple:
@@ -163,9 +177,12 @@ class Chunk:
             return None
         if len(self.source_partial_groups) != 1:
             raise NotImplementedError(
-                "pass one PartialGroup covering the whole Partial connected component, not one per mesh dim"
+                "pass one PartialGroup covering the whole Partial connected component (with levels when the mesh dims "
+                "reduce with different ops), not one group per mesh dim"
             )
         group, op = self.source_partial_groups[0]
+        if group.levels:
+            return group.tensors, group.levels  # one op per Partial mesh dim, innermost (first applied) first
         if op not in REDUCE_OPS:
             raise ValueError(f"unknown reduce op {op!r}")
         return group.tensors, op
@@ -243,7 +260,7 @@ class Bucket:
     def prepare(self, wire=None) -> None:
         """Source bucket: enqueue its pack (or reduce-pack / self-copy) launch.  Target bucket: nothing
         to do, its bytes arrive in the producer's pool slot (``Bucket.prepare``, ``ir.py:229-264``)."""
-        self._plan(wire).run_kinds(("pack", "reduce_pack", "selfcopy", "lend"))
+        self._plan(wire).run_kinds(("pack", "reduce_pack", "selfcopy", "selfcopy_reduce", "lend"))
 
     def launch(self) -> bool:
         """The wire step.  Always ready: the loopback hands the pool slot over in place

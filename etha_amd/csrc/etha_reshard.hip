@@ -447,11 +447,62 @@ __device__ __forceinline__ float round_via(uint32_t via, float r) {
   }
 }
 
+// Reduce-op word of a reduce tile: bits 0-2 the op of the innermost level, 3-5 and 6-8 the ops of the next
+// levels, bits 16-23 / 24-31 the member counts g0 / g1 of the two inner levels (0 = one level over all peers).
+// Peers are listed innermost level fastest.  Level l combines, in list order, the results of level l - 1;
+// an AVG level divides by its own member count.  One level is the common case (one Partial mesh dim, or
+// several with the same op, combined in rank order); several levels are Partial mesh dims with different
+// ops, applied in mesh-dim order as the reference's per-group all-reduces are (ir.py:123-124).
+__device__ __forceinline__ uint32_t level_op(uint32_t word, int level) { return (word >> (3 * level)) & 7u; }
+
+template <typename ACC, typename LOAD, int N>
+__device__ __forceinline__ void reduce_levels(const uint64_t* __restrict__ peers, uint32_t np, uint32_t word,
+                                              uint64_t a_off, ACC* acc) {
+  const uint32_t g0 = (word >> 16) & 255u, g1raw = (word >> 24) & 255u, g1 = g1raw ? g1raw : 1u;
+  const uint32_t g2 = np / (g0 * g1);
+  const uint32_t op0 = level_op(word, 0), op1 = level_op(word, 1), op2 = level_op(word, 2);
+  uint32_t p = 0;
+  ACC mid[N];
+  for (uint32_t i2 = 0; i2 < g2; i2++) {
+    for (uint32_t i1 = 0; i1 < g1; i1++) {
+      ACC inner[N];
+      LOAD::run(peers[p++] + a_off, inner);
+      for (uint32_t i0 = 1; i0 < g0; i0++) {
+        ACC v[N];
+        LOAD::run(peers[p++] + a_off, v);
+#pragma unroll
+        for (int i = 0; i < N; i++) inner[i] = combine(op0, inner[i], v[i]);
+      }
+#pragma unroll
+      for (int i = 0; i < N; i++) {
+        if (op0 == ETHA_AVG) inner[i] = inner[i] / (ACC)g0;
+        mid[i] = i1 == 0 ? inner[i] : combine(op1, mid[i], inner[i]);
+      }
+    }
+#pragma unroll
+    for (int i = 0; i < N; i++) {
+      if (op1 == ETHA_AVG) mid[i] = mid[i] / (ACC)g1;
+      acc[i] = i2 == 0 ? mid[i] : combine(op2, acc[i], mid[i]);
+    }
+  }
+#pragma unroll
+  for (int i = 0; i < N; i++)
+    if (op2 == ETHA_AVG) acc[i] = acc[i] / (ACC)g2;
+}
+
 // f16/bf16/f32 partials: fp32 accumulation, peers combined strictly in list (= rank) order.
 template <typename S, typename D, int N>
 __device__ __forceinline__ void reduce_f32(const uint64_t* __restrict__ peers, uint32_t np, uint32_t op, uint32_t via,
                                            uint64_t a_off, uint64_t dst) {
   float acc[N];
+  if (op >> 16) {  // several levels
+    reduce_levels<float, LoadF32<S, N>, N>(peers, np, op, a_off, acc);
+    Pack<typename D::bits, N> out;
+#pragma unroll
+    for (int i = 0; i < N; i++) out.set(i, from_f32(D(), round_via(via, acc[i])));
+    out.store(dst);
+    return;
+  }
   LoadF32<S, N>::run(peers[0] + a_off, acc);
   uint32_t p = 1;
   for (; p + 3 <= np; p += 3) {  // three peers' loads in flight, then combine in order
@@ -479,28 +530,38 @@ __device__ __forceinline__ void reduce_f32(const uint64_t* __restrict__ peers, u
   out.store(dst);
 }
 
+template <int N>
+struct LoadF64 {
+  __device__ static __forceinline__ void run(uint64_t addr, double* out) {
+    Pack<uint64_t, N> in;
+    in.load(addr);
+#pragma unroll
+    for (int i = 0; i < N; i++) out[i] = __builtin_bit_cast(double, in.get(i));
+  }
+};
+
 // f64 partials: f64 accumulation; result converted like a plain f64 -> D move.
 template <typename D, int N>
 __device__ __forceinline__ void reduce_f64(const uint64_t* __restrict__ peers, uint32_t np, uint32_t op, uint32_t via,
                                            uint64_t a_off, uint64_t dst) {
   double acc[N];
-  {
-    Pack<uint64_t, N> in;
-    in.load(peers[0] + a_off);
+  const bool levels = (op >> 16) != 0;
+  if (levels) {
+    reduce_levels<double, LoadF64<N>, N>(peers, np, op, a_off, acc);
+  } else {
+    LoadF64<N>::run(peers[0] + a_off, acc);
+    for (uint32_t p = 1; p < np; p++) {
+      double v[N];
+      LoadF64<N>::run(peers[p] + a_off, v);
 #pragma unroll
-    for (int i = 0; i < N; i++) acc[i] = __builtin_bit_cast(double, in.get(i));
-  }
-  for (uint32_t p = 1; p < np; p++) {
-    Pack<uint64_t, N> in;
-    in.load(peers[p] + a_off);
-#pragma unroll
-    for (int i = 0; i < N; i++) acc[i] = combine(op, acc[i], __builtin_bit_cast(double, in.get(i)));
+      for (int i = 0; i < N; i++) acc[i] = combine(op, acc[i], v[i]);
+    }
   }
   Pack<typename D::bits, N> out;
 #pragma unroll
   for (int i = 0; i < N; i++) {
     double r = acc[i];
-    if (op == ETHA_AVG) r = r / (double)np;
+    if (!levels && op == ETHA_AVG) r = r / (double)np;
     if (sizeof(typename D::bits) == 8 && via == 0)
       out.set(i, (typename D::bits)__builtin_bit_cast(uint64_t, r));
     else {
@@ -610,6 +671,22 @@ int log2u(uint64_t x) {
   int l = 0;
   while ((1ull << (l + 1)) <= x) l++;
   return l;
+}
+
+// reduce_op of a descriptor: a plain ETHA_* op, or ETHA_REDUCE_LEVELS(...) for Partial mesh dims with different ops
+int check_reduce_op(uint32_t word, uint32_t n_partials, uint32_t idx) {
+  const uint32_t g0 = (word >> 16) & 255u, g1 = (word >> 24) & 255u;
+  if (!g0 && !g1) {
+    if (word > ETHA_PRODUCT) return fail(ETHA_ERR_INVALID, "chunk %u: unknown reduce_op %u", idx, word);
+    return ETHA_OK;
+  }
+  if ((word & 0xfe00u) || !g0) return fail(ETHA_ERR_INVALID, "chunk %u: malformed reduce_op 0x%x", idx, word);
+  for (int l = 0; l < 3; l++)
+    if (((word >> (3 * l)) & 7u) > ETHA_PRODUCT) return fail(ETHA_ERR_INVALID, "chunk %u: unknown reduce_op in level %d", idx, l);
+  const uint32_t inner = g0 * (g1 ? g1 : 1u);
+  if (n_partials == 0 || n_partials % inner != 0)
+    return fail(ETHA_ERR_INVALID, "chunk %u: %u Partial members are not a whole number of groups of %u", idx, n_partials, inner);
+  return ETHA_OK;
 }
 
 struct Region {  // strided region; strides in bytes
@@ -1154,7 +1231,9 @@ extern "C" {
 #define ETHA_SOURCE_HASH "unknown"
 #endif
 int etha_abi_version(void) { return ETHA_ABI_VERSION; }
-const char* etha_source_hash(void) { return ETHA_SOURCE_HASH; }
+// the marker lets a build script find the digest in the file without loading the library
+static const char kSourceDigest[] = "etha-source-digest:" ETHA_SOURCE_HASH;
+const char* etha_source_hash(void) { return kSourceDigest + sizeof("etha-source-digest:") - 1; }
 const char* etha_last_error(void) { return g_err.c_str(); }
 
 int etha_table_create(const EthaChunkDesc* descs, uint32_t n_chunks, const uint64_t* partial_ptrs,
@@ -1177,7 +1256,7 @@ int etha_table_create(const EthaChunkDesc* descs, uint32_t n_chunks, const uint6
     std::vector<uint64_t> peer_bases;
     Region A;
     if (d.n_partials) {
-      if (d.reduce_op > ETHA_PRODUCT) return fail(ETHA_ERR_INVALID, "chunk %u: unknown reduce_op %u", i, d.reduce_op);
+      { const int rc_op = check_reduce_op(d.reduce_op, d.n_partials, i); if (rc_op != ETHA_OK) return rc_op; }
       if (!partial_ptrs || (uint64_t)d.partial_first + d.n_partials > n_partial_ptrs)
         return fail(ETHA_ERR_INVALID, "chunk %u: partial pointer range outside partial_ptrs", i);
       // every peer shares the chunk geometry; validate each peer's range with its own base
@@ -1253,7 +1332,7 @@ int etha_direct_table_create(const EthaChunkDesc* src, const EthaChunkDesc* dst,
     const EthaChunkDesc& d = src[i];
     int rc;
     if (d.n_partials) {
-      if (d.reduce_op > ETHA_PRODUCT) return fail(ETHA_ERR_INVALID, "chunk %u: unknown reduce_op %u", i, d.reduce_op);
+      { const int rc_op = check_reduce_op(d.reduce_op, d.n_partials, i); if (rc_op != ETHA_OK) return rc_op; }
       if (!partial_ptrs || (uint64_t)d.partial_first + d.n_partials > n_partial_ptrs)
         return fail(ETHA_ERR_INVALID, "chunk %u: partial pointer range outside partial_ptrs", i);
       if (dtype_size(d.wire_dtype) == 0) return fail(ETHA_ERR_INVALID, "chunk %u: unknown wire_dtype %u", i, d.wire_dtype);

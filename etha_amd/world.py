@@ -59,13 +59,11 @@ def create_partial_groups(mesh, partial_reductions, this_rank: int, tensors_by_r
     (``_create_partial_groups``, ``agent.py:46-70``) and all-reduces over them one after the other
     (``ir.py:123-124``); the net effect is one reduction over every rank that differs from this one
     only in Partial mesh coordinates.  That whole set is returned as a single group, so that the
-    reduce kernel can combine all members in one pass, in rank order.
+    reduce kernel can combine all members in one pass, in rank order.  Partial mesh dims with different ops
+    become the levels of one nested reduction.
     """
     if not partial_reductions:
         return []
-    ops = {op for _, op in partial_reductions}
-    if len(ops) != 1:
-        raise NotImplementedError(f"Partial dims with different reduce ops {sorted(ops)} are not supported")
     mesh = np.asarray(mesh)
     where = np.argwhere(mesh == this_rank)
     if len(where) != 1:
@@ -73,8 +71,18 @@ def create_partial_groups(mesh, partial_reductions, this_rank: int, tensors_by_r
     index: list = [int(c) for c in where[0]]
     for mesh_dim, _ in partial_reductions:
         index[mesh_dim] = slice(None)
-    ranks = sorted(int(r) for r in np.asarray(mesh[tuple(index)]).reshape(-1))
-    return [(PartialGroup(ranks=ranks, tensors=[tensors_by_rank[r] for r in ranks]), ops.pop())]
+    members = np.asarray(mesh[tuple(index)])  # one axis per Partial mesh dim, in mesh-dim order
+    ops = [op for _, op in sorted(partial_reductions)]
+    if len(set(ops)) == 1:
+        ranks = sorted(int(r) for r in members.reshape(-1))
+        return [(PartialGroup(ranks=ranks, tensors=[tensors_by_rank[r] for r in ranks]), ops[0])]
+    # different ops: the reference all-reduces mesh dim by mesh dim, each with its own op (agent.py:46-70,
+    # ir.py:123-124).  The members are listed with the first Partial mesh dim varying fastest and reduced level
+    # by level in that order.
+    ranks = [int(r) for r in members.transpose().reshape(-1)]
+    levels = tuple((op, int(n)) for op, n in zip(ops, members.shape))
+    group = PartialGroup(ranks=ranks, tensors=[tensors_by_rank[r] for r in ranks], levels=levels)
+    return [(group, "+".join(ops))]
 
 
 def _flat_ranks(mesh) -> list[int]:

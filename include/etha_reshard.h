@@ -68,6 +68,16 @@ enum {
 
 /* reduce ops of a Partial source (ir.py:51-57) */
 enum { ETHA_SUM = 0, ETHA_AVG = 1, ETHA_MAX = 2, ETHA_MIN = 3, ETHA_PRODUCT = 4 };
+/*
+ * Partial mesh dims with different ops.  The reference all-reduces once per Partial mesh dim, each with its own
+ * op, in mesh-dim order (tensor_bus/agent.py:46-70, ir.py:123-124).  ETHA_REDUCE_LEVELS describes that as nested
+ * levels: the peers are listed with the first-applied mesh dim varying fastest; op0 combines each run of g0
+ * peers, op1 each run of g1 such results, op2 what is left (n_partials / (g0 * g1) of them; pass g1 = 1 and
+ * op2 = op1 for two levels).  All levels accumulate in fp32 (f64 for f64 inputs) and the result is rounded
+ * once; an ETHA_AVG level divides by its own member count.
+ */
+#define ETHA_REDUCE_LEVELS(op0, g0, op1, g1, op2) \
+  ((uint32_t)(op0) | ((uint32_t)(op1) << 3) | ((uint32_t)(op2) << 6) | ((uint32_t)(g0) << 16) | ((uint32_t)(g1) << 24))
 
 /*
  * One chunk = one strided region of a local shard plus its place in a bucket.
@@ -87,7 +97,7 @@ typedef struct EthaChunkDesc {
   uint32_t wire_dtype;            /* ETHA_* element type inside the bucket (Chunk.transfer_dtype) */
   uint32_t n_partials;            /* 0 = plain chunk.  >0 = Partial source: reduce this many peers (pack only) */
   uint32_t partial_first;         /* index into partial_ptrs of the first peer's data_ptr(); peers in rank order */
-  uint32_t reduce_op;             /* ETHA_SUM.. when n_partials > 0 */
+  uint32_t reduce_op;             /* ETHA_SUM.. or ETHA_REDUCE_LEVELS(...) when n_partials > 0 */
 } EthaChunkDesc;
 
 typedef struct EthaTable EthaTable; /* compiled, device-resident tile program */

@@ -47,13 +47,27 @@ def reduce_rank_order(slices: list[torch.Tensor], op: str) -> torch.Tensor:
     return acc
 
 
+def reduce_levels(slices: list[torch.Tensor], levels) -> torch.Tensor:
+    """Partial mesh dims with different ops (``ir.py:123-124``: one all-reduce per group, each with its own op, in
+    mesh-dim order).  ``levels = ((op, size), ...)`` from the first-applied dim to the last; ``slices`` lists the
+    members with the first-applied dim varying fastest.  After the first all-reduce every member of a line holds
+    the line's result, so the whole sequence is a nested reduction: level by level, accumulators kept in fp32."""
+    values = list(slices)
+    for op, size in levels:
+        assert len(values) % size == 0
+        values = [reduce_rank_order(values[i:i + size], op) for i in range(0, len(values), size)]
+    assert len(values) == 1
+    return values[0]
+
+
 def _peers(chunk):
     groups = getattr(chunk, "source_partial_groups", None)
     if not groups:
         return None
     assert len(groups) == 1, "oracle: the Partial connected component comes as one group"
     group, op = groups[0]
-    return list(group.tensors), op
+    levels = getattr(group, "levels", ())
+    return list(group.tensors), (tuple(levels) if levels else op)
 
 
 def chunk_prepare(chunk, contiguous: bool = True) -> torch.Tensor:
@@ -66,7 +80,8 @@ def chunk_prepare(chunk, contiguous: bool = True) -> torch.Tensor:
     peers = _peers(chunk)
     if peers is not None:
         tensors, op = peers
-        red = reduce_rank_order([t[chunk.src_slice] for t in tensors], op)
+        members = [t[chunk.src_slice] for t in tensors]
+        red = reduce_levels(members, op) if isinstance(op, tuple) else reduce_rank_order(members, op)
         wire = chunk.transfer_dtype or tensor.dtype
         return red.to(wire)  # single rounding from the accumulator
     if chunk.transfer_dtype and chunk.transfer_dtype != buf.dtype:

@@ -34,8 +34,8 @@ def _random_layout(rng, ndim, allow_partial):
             placements.append(_StridedShard(int(rng.integers(ndim)), split_factor=int(rng.choice([2, 3]))))
         elif kind == "shard":
             placements.append(Shard(int(rng.integers(ndim))))
-        elif kind == "partial":
-            placements.append(Partial("sum"))
+        elif kind == "partial":  # mostly sums; sometimes another op, so that two Partial dims may differ in op
+            placements.append(Partial(str(rng.choice(["sum", "sum", "sum", "max", "avg"]))))
             partial = True
         else:
             placements.append(Replicate())
@@ -78,7 +78,7 @@ def _random_spec(rng, idx, wire_size):
     n_src = math.prod(src_mesh)
     # overlapping rank sets create LOCAL chunks; their wire dtype is the target dtype (as in the reference), so
     # they stay within the batch's wire item size only when the two dtypes agree
-    overlap = (not partial) and sdt == tdt and rng.random() < 0.4
+    overlap = sdt == tdt and rng.random() < 0.4  # with a Partial source: the primary delivers to its own rank too
     tgt_start = 0 if overlap else n_src
     return TensorSpec(f"t{idx}", shape, mesh_of(0, src_mesh), src_pl, mesh_of(tgt_start, tgt_mesh), tgt_pl, sdt, tdt,
                       seed=1000 + idx, std=1.0, dist="normal" if sdt in FLOATS else "bits")
@@ -91,7 +91,7 @@ def _run_step(mem, p, kind, first, count, ordered=False, touched=None):
         execute(p.recv_table, mem, "unpack", first, count, ordered=ordered, touched=touched)
     elif kind in ("selfcopy", "direct"):
         execute(p.local_table, mem, "selfcopy", first, count, ordered=ordered, touched=touched)
-    elif kind == "direct_reduce":
+    elif kind in ("direct_reduce", "selfcopy_reduce"):
         execute(p.local_table, mem, "selfcopy", first, count, peers=_direct_peers_of(p), touched=touched)
     else:
         assert kind == "lend"  # nothing runs for a lent bucket
@@ -164,10 +164,13 @@ def _interpret(job, merged: bool):
 def _direct_peers_of(plan):
     """Peer pointers of a plan's direct-reduce chunks, in the order the plan registered them."""
     ptrs = []
-    for kind, _, _, slot in plan.steps:
+    for (kind, _, _, slot), info in zip(plan.steps, plan.info):
         if kind == "direct_reduce":
             for _, _, _, peers in slot.sources:
                 ptrs.extend(t.data_ptr() for t in peers[0])
+        elif kind == "selfcopy_reduce":  # a Partial source delivered to its own rank
+            for c in info.bucket.chunks:
+                ptrs.extend(t.data_ptr() for t in c.partial_peers()[0])
     return np.asarray(ptrs, dtype=np.uint64) if ptrs else None
 
 

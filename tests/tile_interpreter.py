@@ -201,7 +201,7 @@ def _reduce_units(arena, mem, row_tiles, row_idx, a_off, b, ua, ub, dta, dtb, pe
         sel = row_idx == ti
         t = row_tiles[ti]
         bases = peers[int(t["peer_first"]) : int(t["peer_first"]) + int(t["n_peers"])].astype(np.int64)
-        op = {0: "sum", 1: "avg", 2: "max", 3: "min", 4: "product"}[int(t["reduce_op"])]
+        op = {0: "sum", 1: "avg", 2: "max", 3: "min", 4: "product"}[int(t["reduce_op"]) & 7]
         offs = a_off[sel]
         n_units = len(offs)
         via = int(t["via"])  # 0, or 1 + the dtype the result is rounded to before the b-side dtype
@@ -216,8 +216,29 @@ def _reduce_units(arena, mem, row_tiles, row_idx, a_off, b, ua, ub, dta, dtb, pe
             so = arena.offsets(base + offs, ua)[:, None] + np.arange(ua)
             _note("r", so)
             staged.append(np.ascontiguousarray(mem[so]).reshape(-1).copy())
-        ch = co.make_chunk(0, (0,), (n_units * n_el,), (1,), dta, out_dt, peers=[s.ctypes.data for s in staged], op=op)
-        assert co.lib().oracle_reduce(ch, out.ctypes.data, scratch.ctypes.data) == 0
+        word = int(t["reduce_op"])
+        g0, g1 = (word >> 16) & 255, (word >> 24) & 255
+        names = {0: "sum", 1: "avg", 2: "max", 3: "min", 4: "product"}
+        if g0 == 0:  # one level over all peers, in list order
+            ch = co.make_chunk(0, (0,), (n_units * n_el,), (1,), dta, out_dt, peers=[s.ctypes.data for s in staged], op=op)
+            assert co.lib().oracle_reduce(ch, out.ctypes.data, scratch.ctypes.data) == 0
+        else:  # nested levels: accumulators stay in fp32 (f64 for f64 inputs) between levels, one rounding at the end
+            g1 = g1 or 1
+            sizes = [g0, g1, len(staged) // (g0 * g1)]
+            assert sizes[0] * sizes[1] * sizes[2] == len(staged)
+            acc_dt = 3 if dta == 3 else 2
+            values, cur_dt = staged, dta
+            for level, size in enumerate(sizes):
+                last = level == 2
+                nxt = []
+                for i in range(0, len(values), size):
+                    o = out if last else np.zeros(n_units * n_el, dtype=_CODE_RAW[acc_dt])
+                    ch = co.make_chunk(0, (0,), (n_units * n_el,), (1,), cur_dt, out_dt if last else acc_dt,
+                                       peers=[v.ctypes.data for v in values[i:i + size]], op=names[(word >> (3 * level)) & 7])
+                    assert co.lib().oracle_reduce(ch, o.ctypes.data, scratch.ctypes.data) == 0
+                    nxt.append(o)
+                values, cur_dt = nxt, acc_dt
+            assert len(values) == 1
         if via:
             out = co.cast(out, out_dt, dtb, _CODE_RAW[dtb])
         do = arena.offsets(b[sel], ub)[:, None] + np.arange(ub)
