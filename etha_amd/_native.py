@@ -18,7 +18,7 @@ ABI_VERSION = 4
 LAUNCH_UNORDERED = 1  # ETHA_LAUNCH_UNORDERED
 
 # element type codes (include/etha_reshard.h)
-F16, BF16, F32, F64, B8, B16, B32, B64 = range(8)
+F16, BF16, F32, F64, B8, B16, B32, B64, I8, U8, I16, I32, I64, BOOL, F8E4M3, F8E5M2 = range(16)
 REDUCE_OPS = {"sum": 0, "avg": 1, "max": 2, "min": 3, "product": 4}
 
 ERR_INVALID, ERR_UNSUPPORTED, ERR_HIP, ERR_NOMEM = -1, -2, -3, -4

@@ -23,12 +23,25 @@ _FLOAT_CODES = {
     torch.float32: nat.F32,
     torch.float64: nat.F64,
 }
+# value types beyond the four floats: converted element by element with ``Tensor.to`` semantics
+_VALUE_CODES = {
+    torch.int8: nat.I8,
+    torch.uint8: nat.U8,
+    torch.int16: nat.I16,
+    torch.int32: nat.I32,
+    torch.int64: nat.I64,
+    torch.bool: nat.BOOL,
+    torch.float8_e4m3fn: nat.F8E4M3,
+    torch.float8_e5m2: nat.F8E5M2,
+}
 _OPAQUE_CODES = {1: nat.B8, 2: nat.B16, 4: nat.B32, 8: nat.B64}
 
 
 def dtype_code(dtype: torch.dtype) -> int:
     if dtype in _FLOAT_CODES:
         return _FLOAT_CODES[dtype]
+    if dtype in _VALUE_CODES:
+        return _VALUE_CODES[dtype]
     code = _OPAQUE_CODES.get(dtype.itemsize)
     if code is None:
         raise NotImplementedError(f"dtype {dtype} (itemsize {dtype.itemsize}) is not supported")
@@ -36,9 +49,11 @@ def dtype_code(dtype: torch.dtype) -> int:
 
 
 def check_cast(src: torch.dtype, dst: torch.dtype) -> None:
-    """Same dtype is a byte move; otherwise both must be floating (fp16/bf16/fp32/fp64)."""
-    if src != dst and not (src in _FLOAT_CODES and dst in _FLOAT_CODES):
-        raise NotImplementedError(f"conversion {src} -> {dst} is only implemented between floating dtypes")
+    """Same dtype is a byte move; otherwise both must be value types the library converts (the floats, the
+    integers, bool, the 8-bit floats).  Other types (complex, unsigned 16/32/64) can only be moved."""
+    known = (_FLOAT_CODES, _VALUE_CODES)
+    if src != dst and not (any(src in k for k in known) and any(dst in k for k in known)):
+        raise NotImplementedError(f"conversion {src} -> {dst}: only floats, integers, bool and 8-bit floats are converted")
 
 
 def reduce_op_word(op) -> int:

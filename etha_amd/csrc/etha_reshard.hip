@@ -135,6 +135,7 @@ constexpr uint32_t kMetaVec = 1u << 17; // converting move handles the full vect
 constexpr uint32_t kMetaSkew = 1u << 18;  // a-side addresses are not all multiples of the a-side unit size
 constexpr uint32_t kMetaSkewB = 1u << 19; // same for the b side (both are bookkeeping for checkers: the kernel's
                                           // accesses are legal at any element-aligned address)
+constexpr uint32_t kMetaGeneric = 1u << 20;  // converting move with an integer, bool or 8-bit float side: one element per unit
 
 // ---- typed vector access ----------------------------------------------------------------------
 typedef uint32_t u32x2 __attribute__((ext_vector_type(2)));
@@ -241,6 +242,127 @@ __device__ __forceinline__ void cvt_from(uint32_t dd, bool vec, uint64_t src, ui
   }
 }
 
+// ---- conversions with an integer, bool or 8-bit float side (Tensor.to(dtype) = static_cast, c10::convert) ----
+// 8-bit floats as the published c10 routines define them: round to nearest even on the fp32 bit pattern;
+// e4m3fn has no infinities (everything from 480 up and NaN become NaN 0x7F), e5m2 overflows to infinity.
+__device__ __forceinline__ uint8_t f32_to_e4m3(float f) {
+  uint32_t u = __builtin_bit_cast(uint32_t, f);
+  const uint32_t sign = u & 0x80000000u;
+  uint32_t mag = u ^ sign;
+  uint32_t r;
+  if (mag >= (1087u << 20)) {
+    r = 0x7f;
+  } else if (mag < (121u << 23)) {  // below 2^-6: a subnormal result, rounded by a float addition
+    const uint32_t denorm = 141u << 23;
+    float t = __builtin_bit_cast(float, mag) + __builtin_bit_cast(float, denorm);
+    r = (__builtin_bit_cast(uint32_t, t) - denorm) & 0xffu;
+  } else {
+    const uint32_t odd = (mag >> 20) & 1u;
+    mag += ((uint32_t)(7 - 127) << 23) + 0x7ffffu + odd;
+    r = (mag >> 20) & 0xffu;
+  }
+  return (uint8_t)(r | (sign >> 24));
+}
+__device__ __forceinline__ uint8_t f32_to_e5m2(float f) {
+  uint32_t u = __builtin_bit_cast(uint32_t, f);
+  const uint32_t sign = u & 0x80000000u;
+  uint32_t mag = u ^ sign;
+  uint32_t r;
+  if (mag >= (143u << 23)) {
+    r = mag > (255u << 23) ? 0x7fu : 0x7cu;
+  } else if (mag < (113u << 23)) {  // below 2^-14
+    const uint32_t denorm = 134u << 23;
+    float t = __builtin_bit_cast(float, mag) + __builtin_bit_cast(float, denorm);
+    r = (__builtin_bit_cast(uint32_t, t) - denorm) & 0xffu;
+  } else {
+    const uint32_t odd = (mag >> 21) & 1u;
+    mag += ((uint32_t)(15 - 127) << 23) + 0xfffffu + odd;
+    r = (mag >> 21) & 0xffu;
+  }
+  return (uint8_t)(r | (sign >> 24));
+}
+__device__ __forceinline__ float e4m3_to_f32(uint8_t b) {
+  const uint32_t sign = ((uint32_t)b & 0x80u) << 24, e = (b >> 3) & 0xfu, man = b & 7u;
+  if (e == 0xf && man == 7) return __builtin_bit_cast(float, sign | 0x7fc00000u);
+  if (e == 0) return __builtin_bit_cast(float, sign | __builtin_bit_cast(uint32_t, (float)man * 0.001953125f));
+  return __builtin_bit_cast(float, sign | ((e + 127 - 7) << 23) | (man << 20));
+}
+__device__ __forceinline__ float e5m2_to_f32(uint8_t b) { return to_f32(TagF16(), (uint16_t)((uint16_t)b << 8)); }
+
+// float -> integer: truncation toward zero.  Values that do not fit, and NaN, are undefined in C++; ATen's x86
+// kernels return what cvttss2si / cvttsd2si return for them (INT32_MIN, or INT64_MIN for a 64-bit result), and a
+// result narrower than 32 bits is the low bits of the 32-bit one.  A uint8 result is taken from the 64-bit
+// conversion (c10 casts through int64_t for it).  The device's own conversions saturate, hence the range checks.
+__device__ __forceinline__ int64_t trunc_i32(float f) { return (f >= -2147483648.0f && f < 2147483648.0f) ? (int64_t)(int32_t)f : (int64_t)INT32_MIN; }
+__device__ __forceinline__ int64_t trunc_i64(float f) { return (f >= -9223372036854775808.0f && f < 9223372036854775808.0f) ? (int64_t)f : INT64_MIN; }
+__device__ __forceinline__ int64_t trunc_i32(double f) { return (f > -2147483649.0 && f < 2147483648.0) ? (int64_t)(int32_t)f : (int64_t)INT32_MIN; }
+__device__ __forceinline__ int64_t trunc_i64(double f) { return (f >= -9223372036854775808.0 && f < 9223372036854775808.0) ? (int64_t)f : INT64_MIN; }
+
+__device__ __forceinline__ bool is_int_code(uint32_t dt) { return dt >= ETHA_I8 && dt <= ETHA_BOOL; }
+
+__device__ __forceinline__ int64_t load_int_elem(uint32_t dt, uint64_t addr) {
+  switch (dt) {
+    case ETHA_I8: return (int8_t)ld_stream<uint8_t>(addr);
+    case ETHA_U8: return ld_stream<uint8_t>(addr);
+    case ETHA_BOOL: return ld_stream<uint8_t>(addr) != 0;
+    case ETHA_I16: return (int16_t)ld_stream<uint16_t>(addr);
+    case ETHA_I32: return (int32_t)ld_stream<uint32_t>(addr);
+    default: return (int64_t)ld_stream<uint64_t>(addr);
+  }
+}
+__device__ __forceinline__ void store_int_elem(uint32_t dt, uint64_t addr, int64_t v) {
+  switch (dt) {
+    case ETHA_I8: case ETHA_U8: st_stream<uint8_t>(addr, (uint8_t)v); break;
+    case ETHA_BOOL: st_stream<uint8_t>(addr, v != 0 ? 1 : 0); break;
+    case ETHA_I16: st_stream<uint16_t>(addr, (uint16_t)v); break;
+    case ETHA_I32: st_stream<uint32_t>(addr, (uint32_t)v); break;
+    default: st_stream<uint64_t>(addr, (uint64_t)v); break;
+  }
+}
+__device__ __forceinline__ float load_float_elem(uint32_t dt, uint64_t addr) {  // every float type but f64 -> exact; f64 rounds
+  switch (dt) {
+    case ETHA_F16: return to_f32(TagF16(), ld_stream<uint16_t>(addr));
+    case ETHA_BF16: return to_f32(TagBF16(), ld_stream<uint16_t>(addr));
+    case ETHA_F32: return to_f32(TagF32(), ld_stream<uint32_t>(addr));
+    case ETHA_F8E4M3: return e4m3_to_f32(ld_stream<uint8_t>(addr));
+    case ETHA_F8E5M2: return e5m2_to_f32(ld_stream<uint8_t>(addr));
+    default: return to_f32(TagF64(), ld_stream<uint64_t>(addr));
+  }
+}
+__device__ __forceinline__ void store_float_elem(uint32_t dt, uint64_t addr, float f) {
+  switch (dt) {
+    case ETHA_F16: st_stream<uint16_t>(addr, from_f32(TagF16(), f)); break;
+    case ETHA_BF16: st_stream<uint16_t>(addr, from_f32(TagBF16(), f)); break;
+    case ETHA_F32: st_stream<uint32_t>(addr, from_f32(TagF32(), f)); break;
+    case ETHA_F8E4M3: st_stream<uint8_t>(addr, f32_to_e4m3(f)); break;
+    case ETHA_F8E5M2: st_stream<uint8_t>(addr, f32_to_e5m2(f)); break;
+    default: st_stream<uint64_t>(addr, from_f32(TagF64(), f)); break;
+  }
+}
+
+__device__ __forceinline__ void convert_generic(uint32_t sd, uint32_t dd, uint64_t src, uint64_t dst) {
+  if (is_int_code(sd)) {
+    const int64_t v = load_int_elem(sd, src);
+    if (is_int_code(dd))
+      store_int_elem(dd, dst, v);
+    else if (dd == ETHA_F64)
+      st_stream<uint64_t>(dst, __builtin_bit_cast(uint64_t, (double)v));
+    else
+      store_float_elem(dd, dst, (float)v);  // narrower floats are built from float(value)
+    return;
+  }
+  if (sd == ETHA_F64 && is_int_code(dd)) {
+    const double d = __builtin_bit_cast(double, ld_stream<uint64_t>(src));
+    store_int_elem(dd, dst, dd == ETHA_BOOL ? (int64_t)(d != 0.0) : (dd == ETHA_I64 || dd == ETHA_U8) ? trunc_i64(d) : trunc_i32(d));
+    return;
+  }
+  const float f = load_float_elem(sd, src);
+  if (is_int_code(dd))
+    store_int_elem(dd, dst, dd == ETHA_BOOL ? (int64_t)(f != 0.0f) : (dd == ETHA_I64 || dd == ETHA_U8) ? trunc_i64(f) : trunc_i32(f));
+  else
+    store_float_elem(dd, dst, f);
+}
+
 template <bool REV>
 __device__ __forceinline__ void move_unit(uint32_t meta, uint64_t a, uint64_t b) {
   const uint64_t src = REV ? b : a, dst = REV ? a : b;
@@ -256,6 +378,10 @@ __device__ __forceinline__ void move_unit(uint32_t meta, uint64_t a, uint64_t b)
   }
   const uint32_t dta = (meta >> kMetaDtaShift) & 15u, dtb = (meta >> kMetaDtbShift) & 15u;
   const uint32_t sd = REV ? dtb : dta, dd = REV ? dta : dtb;
+  if (meta & kMetaGeneric) {
+    convert_generic(sd, dd, src, dst);
+    return;
+  }
   const bool vec = (meta & kMetaVec) != 0;
   switch (sd) {
     case ETHA_F16: cvt_from<TagF16>(dd, vec, src, dst); break;
@@ -659,14 +785,15 @@ int fail(int code, const char* fmt, ...) {
 
 int dtype_size(uint32_t dt) {
   switch (dt) {
-    case ETHA_F16: case ETHA_BF16: case ETHA_B16: return 2;
-    case ETHA_F32: case ETHA_B32: return 4;
-    case ETHA_F64: case ETHA_B64: return 8;
-    case ETHA_B8: return 1;
+    case ETHA_F16: case ETHA_BF16: case ETHA_B16: case ETHA_I16: return 2;
+    case ETHA_F32: case ETHA_B32: case ETHA_I32: return 4;
+    case ETHA_F64: case ETHA_B64: case ETHA_I64: return 8;
+    case ETHA_B8: case ETHA_I8: case ETHA_U8: case ETHA_BOOL: case ETHA_F8E4M3: case ETHA_F8E5M2: return 1;
     default: return 0;
   }
 }
-bool is_float(uint32_t dt) { return dt <= ETHA_F64; }
+bool is_float(uint32_t dt) { return dt <= ETHA_F64; }                       // the four IEEE-style floats (vector conversions, reductions)
+bool is_typed(uint32_t dt) { return dt <= ETHA_F64 || (dt >= ETHA_I8 && dt <= ETHA_F8E5M2); }  // has a value, can be converted
 int log2u(uint64_t x) {
   int l = 0;
   while ((1ull << (l + 1)) <= x) l++;
@@ -766,11 +893,11 @@ class PairCompiler {
     if (A_.nd != B_.nd) return fail(ETHA_ERR_INVALID, "chunk %u: rank mismatch", idx_);
     for (int i = 0; i < A_.nd; i++)
       if (A_.shape[i] != B_.shape[i]) return fail(ETHA_ERR_INVALID, "chunk %u: shape mismatch in dim %d", idx_, i);
-    if (cvt_ && !(is_float(dta_) && is_float(dtb_)))
-      return fail(ETHA_ERR_UNSUPPORTED, "chunk %u: conversion %u -> %u is only implemented between floating types", idx_,
-                  dta_, dtb_);
-    if (red_.n_peers && !is_float(dta_))
-      return fail(ETHA_ERR_UNSUPPORTED, "chunk %u: Partial reduce needs a floating tensor dtype", idx_);
+    if (cvt_ && !(is_typed(dta_) && is_typed(dtb_)))
+      return fail(ETHA_ERR_UNSUPPORTED, "chunk %u: conversion %u -> %u: opaque element types can only be moved, not converted",
+                  idx_, dta_, dtb_);
+    if (red_.n_peers && !(is_float(dta_) && is_float(dtb_)))
+      return fail(ETHA_ERR_UNSUPPORTED, "chunk %u: Partial reduce needs f16/bf16/f32/f64 on both sides", idx_);
     if (region_numel(A_) == 0) return ETHA_OK;
     collapse_dims();
     bool done = false;
@@ -965,6 +1092,9 @@ class PairCompiler {
   // that; else a body of whole vectors plus a remainder of single elements; runs shorter than one vector
   // single elements.
   int compile_typed_move() {
+    if (!(is_float(dta_) && is_float(dtb_)))  // an integer, bool or 8-bit float side: element by element
+      return emit(A_.base, B_.base, run_elems_, (uint64_t)esa_, (uint64_t)esb_,
+                  dt_bits_ | kMetaCvt | kMetaGeneric | unit_bits(log2u((uint64_t)esa_), log2u((uint64_t)esb_)));
     const int epv = red_.n_peers ? 16 / (esa_ > esb_ ? esa_ : esb_) : cvt_elems_per_unit(esa_, esb_);
     const int ea = log2u((uint64_t)esa_), eb = log2u((uint64_t)esb_);
     const int va = log2u((uint64_t)(epv * esa_)), vb = log2u((uint64_t)(epv * esb_));

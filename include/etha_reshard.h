@@ -41,17 +41,29 @@ extern "C" {
 #define ETHA_ERR_HIP (-3)         /* a HIP runtime call failed */
 #define ETHA_ERR_NOMEM (-4)
 
-/* element types.  Same-type transfers are byte moves and work for every type;
- * conversions are implemented between the four floating types only. */
+/* element types.  Same-type transfers are byte moves and work for every type.  Conversions
+ * (Chunk.prepare / Chunk.finalize call buffer.to(dtype), ir.py:125-126,137-138) are implemented between all
+ * value types: vectorised between the four IEEE-style floats, element by element when an integer, bool or
+ * 8-bit float is involved.  Semantics are ATen's: round to nearest even into floats, truncation toward zero
+ * into integers (values that do not fit, and NaN, give what ATen's x86 kernels give: INT32_MIN / INT64_MIN,
+ * narrower results the low bits, uint8 through int64), != 0 into bool.  Opaque types can only be moved. */
 enum {
   ETHA_F16 = 0,
   ETHA_BF16 = 1,
   ETHA_F32 = 2,
   ETHA_F64 = 3,
-  ETHA_B8 = 4,   /* opaque 1-byte element (int8/uint8/bool/fp8) */
-  ETHA_B16 = 5,  /* opaque 2-byte element (int16/...) */
-  ETHA_B32 = 6,  /* opaque 4-byte element (int32/...) */
-  ETHA_B64 = 7   /* opaque 8-byte element (int64/complex32/...) */
+  ETHA_B8 = 4,   /* opaque 1-byte element */
+  ETHA_B16 = 5,  /* opaque 2-byte element */
+  ETHA_B32 = 6,  /* opaque 4-byte element */
+  ETHA_B64 = 7,  /* opaque 8-byte element (complex64/...) */
+  ETHA_I8 = 8,
+  ETHA_U8 = 9,
+  ETHA_I16 = 10,
+  ETHA_I32 = 11,
+  ETHA_I64 = 12,
+  ETHA_BOOL = 13,
+  ETHA_F8E4M3 = 14, /* float8_e4m3fn */
+  ETHA_F8E5M2 = 15  /* float8_e5m2 */
 };
 
 /*

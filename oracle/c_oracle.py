@@ -11,7 +11,7 @@ import numpy as np
 ORACLE_DIR = os.path.dirname(os.path.abspath(__file__))
 LIB_PATH = os.path.join(ORACLE_DIR, "liboracle.so")
 MAX_NDIM = 8
-F16, BF16, F32, F64, B8, B16, B32, B64 = range(8)
+F16, BF16, F32, F64, B8, B16, B32, B64, I8, U8, I16, I32, I64, BOOL, F8E4M3, F8E5M2 = range(16)
 OPS = {"sum": 0, "avg": 1, "max": 2, "min": 3, "product": 4}
 
 
@@ -43,8 +43,9 @@ _lib = None
 def lib() -> ctypes.CDLL:
     global _lib
     if _lib is None:
-        if not os.path.exists(LIB_PATH):
-            build()
+        source = os.path.join(ORACLE_DIR, "reshard_oracle.c")
+        if not os.path.exists(LIB_PATH) or os.path.getmtime(LIB_PATH) < os.path.getmtime(source):
+            build()  # missing, or older than its source
         h = ctypes.CDLL(LIB_PATH)
         h.oracle_f32_to_bf16.restype = ctypes.c_uint16
         h.oracle_f32_to_bf16.argtypes = [ctypes.c_uint32]

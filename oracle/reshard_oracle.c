@@ -22,7 +22,8 @@
 #include <stdint.h>
 #include <string.h>
 
-enum { OR_F16 = 0, OR_BF16 = 1, OR_F32 = 2, OR_F64 = 3, OR_B8 = 4, OR_B16 = 5, OR_B32 = 6, OR_B64 = 7 };
+enum { OR_F16 = 0, OR_BF16 = 1, OR_F32 = 2, OR_F64 = 3, OR_B8 = 4, OR_B16 = 5, OR_B32 = 6, OR_B64 = 7,
+       OR_I8 = 8, OR_U8 = 9, OR_I16 = 10, OR_I32 = 11, OR_I64 = 12, OR_BOOL = 13, OR_F8E4M3 = 14, OR_F8E5M2 = 15 };
 enum { OR_SUM = 0, OR_AVG = 1, OR_MAX = 2, OR_MIN = 3, OR_PRODUCT = 4 };
 #define OR_MAX_NDIM 8
 
@@ -43,10 +44,10 @@ typedef struct {
 
 int oracle_dtype_size(int dt) {
   switch (dt) {
-    case OR_F16: case OR_BF16: case OR_B16: return 2;
-    case OR_F32: case OR_B32: return 4;
-    case OR_F64: case OR_B64: return 8;
-    case OR_B8: return 1;
+    case OR_F16: case OR_BF16: case OR_B16: case OR_I16: return 2;
+    case OR_F32: case OR_B32: case OR_I32: return 4;
+    case OR_F64: case OR_B64: case OR_I64: return 8;
+    case OR_B8: case OR_I8: case OR_U8: case OR_BOOL: case OR_F8E4M3: case OR_F8E5M2: return 1;
     default: return 0;
   }
 }
@@ -91,7 +92,7 @@ uint16_t oracle_f32_to_f16(uint32_t u) {
 uint32_t oracle_f16_to_f32(uint16_t h) {
   uint32_t sign = ((uint32_t)h & 0x8000u) << 16;
   uint32_t e = (h >> 10) & 0x1fu, man = h & 0x3ffu;
-  if (e == 0x1f) return sign | 0x7f800000u | (man << 13);
+  if (e == 0x1f) return sign | 0x7f800000u | (man << 13) | (man ? 0x00400000u : 0u);  /* a signalling NaN comes out quiet */
   if (e == 0) {
     if (man == 0) return sign;
     int shift = 0;
@@ -119,14 +120,135 @@ static void store_from_f32(void* p, int dt, float f) {
   }
 }
 
+/* ---- 8-bit floats (OCP e4m3fn: no infinities, S.1111.111 is NaN; e5m2: IEEE-like) ----------------
+ * Restated from the published c10 conversion routines (c10/util/Float8_e4m3fn.h, Float8_e5m2.h): round to
+ * nearest even on the fp32 bit pattern; e4m3fn maps everything from 480 up (and NaN) to NaN 0x7F, e5m2 maps
+ * overflow to infinity 0x7C and NaN to 0x7F. */
+uint8_t oracle_f32_to_e4m3(uint32_t u) {
+  const uint32_t sign = u & 0x80000000u;
+  uint32_t mag = u ^ sign;
+  uint8_t r;
+  if (mag >= (1087u << 20)) {
+    r = 0x7f;
+  } else if (mag < (121u << 23)) {               /* below 2^-6: subnormal result, rounded by a float addition */
+    const uint32_t denorm = 141u << 23;
+    r = (uint8_t)(f32_to_bits(bits_to_f32(mag) + bits_to_f32(denorm)) - denorm);
+  } else {
+    const uint32_t odd = (mag >> 20) & 1u;
+    mag += ((uint32_t)(7 - 127) << 23) + 0x7ffffu + odd;
+    r = (uint8_t)(mag >> 20);
+  }
+  return (uint8_t)(r | (sign >> 24));
+}
+uint8_t oracle_f32_to_e5m2(uint32_t u) {
+  const uint32_t sign = u & 0x80000000u;
+  uint32_t mag = u ^ sign;
+  uint8_t r;
+  if (mag >= (143u << 23)) {
+    r = mag > (255u << 23) ? 0x7f : 0x7c;
+  } else if (mag < (113u << 23)) {               /* below 2^-14 */
+    const uint32_t denorm = 134u << 23;
+    r = (uint8_t)(f32_to_bits(bits_to_f32(mag) + bits_to_f32(denorm)) - denorm);
+  } else {
+    const uint32_t odd = (mag >> 21) & 1u;
+    mag += ((uint32_t)(15 - 127) << 23) + 0xfffffu + odd;
+    r = (uint8_t)(mag >> 21);
+  }
+  return (uint8_t)(r | (sign >> 24));
+}
+uint32_t oracle_e5m2_to_f32(uint8_t b) { return oracle_f16_to_f32((uint16_t)((uint16_t)b << 8)); }
+uint32_t oracle_e4m3_to_f32(uint8_t b) {
+  const uint32_t sign = ((uint32_t)b & 0x80u) << 24, e = (b >> 3) & 0xfu, man = b & 7u;
+  if (e == 0xf && man == 7) return sign | 0x7fc00000u;
+  if (e == 0) {
+    if (man == 0) return sign;
+    float v = (float)man * 0.001953125f;          /* man * 2^-9, exact */
+    return sign | f32_to_bits(v);
+  }
+  return sign | ((e + 127 - 7) << 23) | (man << 20);
+}
+
+/* ---- integers and bool: buffer.to(dtype) between any two of the types above is static_cast
+ * (c10::convert).  A float becomes an integer by truncation toward zero; for values that do not fit,
+ * and for NaN, the C++ cast is undefined and ATen's x86 CPU kernels return what cvttss2si / cvttsd2si
+ * return: INT32_MIN for a 32-bit (or narrower: the low bits of that) result, INT64_MIN for a 64-bit one.
+ * A uint8 result is taken from the 64-bit conversion (c10's static_cast_with_inter_type<uint8_t, T> casts
+ * through int64_t).  Narrow floats (f16, bf16, fp8) go through float in both directions. */
+static int is_float_dt(int dt) { return dt <= OR_F64 || dt == OR_F8E4M3 || dt == OR_F8E5M2; }
+static int is_int_dt(int dt) { return dt >= OR_I8 && dt <= OR_BOOL; }
+
+static int32_t trunc_i32_f32(float f) { return (f >= -2147483648.0f && f < 2147483648.0f) ? (int32_t)f : INT32_MIN; }
+static int64_t trunc_i64_f32(float f) { return (f >= -9223372036854775808.0f && f < 9223372036854775808.0f) ? (int64_t)f : INT64_MIN; }
+static int32_t trunc_i32_f64(double f) { return (f > -2147483649.0 && f < 2147483648.0) ? (int32_t)f : INT32_MIN; }
+static int64_t trunc_i64_f64(double f) { return (f >= -9223372036854775808.0 && f < 9223372036854775808.0) ? (int64_t)f : INT64_MIN; }
+
+static int64_t load_int(const void* p, int dt) {
+  switch (dt) {
+    case OR_I8: { int8_t v; memcpy(&v, p, 1); return v; }
+    case OR_U8: { uint8_t v; memcpy(&v, p, 1); return v; }
+    case OR_BOOL: { uint8_t v; memcpy(&v, p, 1); return v != 0; }
+    case OR_I16: { int16_t v; memcpy(&v, p, 2); return v; }
+    case OR_I32: { int32_t v; memcpy(&v, p, 4); return v; }
+    default: { int64_t v; memcpy(&v, p, 8); return v; }
+  }
+}
+static void store_int(void* p, int dt, int64_t v) {
+  switch (dt) {
+    case OR_I8: case OR_U8: { uint8_t b = (uint8_t)v; memcpy(p, &b, 1); break; }
+    case OR_BOOL: { uint8_t b = v != 0; memcpy(p, &b, 1); break; }
+    case OR_I16: { uint16_t b = (uint16_t)v; memcpy(p, &b, 2); break; }
+    case OR_I32: { uint32_t b = (uint32_t)v; memcpy(p, &b, 4); break; }
+    default: memcpy(p, &v, 8);
+  }
+}
+static float load_float_as_f32(const void* p, int dt) {
+  if (dt == OR_F8E4M3) { uint8_t b; memcpy(&b, p, 1); return bits_to_f32(oracle_e4m3_to_f32(b)); }
+  if (dt == OR_F8E5M2) { uint8_t b; memcpy(&b, p, 1); return bits_to_f32(oracle_e5m2_to_f32(b)); }
+  return load_as_f32(p, dt);
+}
+static void store_float_from_f32(void* p, int dt, float f) {
+  if (dt == OR_F8E4M3) { uint8_t b = oracle_f32_to_e4m3(f32_to_bits(f)); memcpy(p, &b, 1); return; }
+  if (dt == OR_F8E5M2) { uint8_t b = oracle_f32_to_e5m2(f32_to_bits(f)); memcpy(p, &b, 1); return; }
+  store_from_f32(p, dt, f);
+}
+
+static void cast_one(const void* src, int sdt, void* dst, int ddt) {
+  if (is_int_dt(sdt)) {
+    const int64_t v = load_int(src, sdt);
+    if (is_int_dt(ddt)) { store_int(dst, ddt, v); return; }
+    if (ddt == OR_F64) { double d = (double)v; memcpy(dst, &d, 8); return; }
+    store_float_from_f32(dst, ddt, (float)v);           /* narrower floats are built from float(value) */
+    return;
+  }
+  if (sdt == OR_F64 && is_int_dt(ddt)) {
+    double d; memcpy(&d, src, 8);
+    if (ddt == OR_BOOL) store_int(dst, ddt, d != 0.0);
+    else if (ddt == OR_I64 || ddt == OR_U8) store_int(dst, ddt, trunc_i64_f64(d));
+    else store_int(dst, ddt, trunc_i32_f64(d));
+    return;
+  }
+  const float f = load_float_as_f32(src, sdt);            /* f64 -> narrow float: two roundings, through float */
+  if (is_int_dt(ddt)) {
+    if (ddt == OR_BOOL) store_int(dst, ddt, f != 0.0f);
+    else if (ddt == OR_I64 || ddt == OR_U8) store_int(dst, ddt, trunc_i64_f32(f));
+    else store_int(dst, ddt, trunc_i32_f32(f));
+    return;
+  }
+  store_float_from_f32(dst, ddt, f);
+}
+
 /* n elements src_dt -> dst_dt.  Same dtype: byte move.  Returns 0, or -1 if unsupported. */
 int oracle_cast(const void* src, int src_dt, void* dst, int dst_dt, int64_t n) {
   int ss = oracle_dtype_size(src_dt), ds = oracle_dtype_size(dst_dt);
   if (!ss || !ds) return -1;
   if (src_dt == dst_dt) { memmove(dst, src, (size_t)(n * ss)); return 0; }
-  if (src_dt > OR_F64 || dst_dt > OR_F64) return -1;
-  for (int64_t i = 0; i < n; i++)
-    store_from_f32((char*)dst + i * ds, dst_dt, load_as_f32((const char*)src + i * ss, src_dt));
+  if (!(is_float_dt(src_dt) || is_int_dt(src_dt)) || !(is_float_dt(dst_dt) || is_int_dt(dst_dt))) return -1;
+  if (src_dt <= OR_F64 && dst_dt <= OR_F64) {
+    for (int64_t i = 0; i < n; i++)
+      store_from_f32((char*)dst + i * ds, dst_dt, load_as_f32((const char*)src + i * ss, src_dt));
+    return 0;
+  }
+  for (int64_t i = 0; i < n; i++) cast_one((const char*)src + i * ss, src_dt, (char*)dst + i * ds, dst_dt);
   return 0;
 }
 

@@ -23,6 +23,8 @@ def cpu_fill(spec: TensorSpec) -> torch.Tensor:
         return raw.view(spec.source_dtype).reshape(spec.shape)
     else:
         g = torch.randn(spec.shape, generator=gen, dtype=torch.float32) * spec.std
+    if not spec.source_dtype.is_floating_point:  # integers and bool: spread the values over a few hundred units
+        g = g * (200.0 / max(spec.std, 1e-6))
     return g.to(spec.source_dtype)
 
 

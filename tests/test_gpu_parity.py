@@ -14,7 +14,7 @@ from etha_amd import workloads
 from etha_amd.comm import Chunk, LoopbackWire, Transport, bucket_comm, chunk_to_bucket_ops
 from etha_amd.world import ReshardJob, TensorSpec
 
-from helpers import (DTYPES, assert_bit_equal, clone_specs, cpu_fill, expected_target, gpu_vs_oracle, load_cases, mesh_of,
+from helpers import (DTYPES, assert_bit_equal, bits, clone_specs, cpu_fill, expected_target, gpu_vs_oracle, load_cases, mesh_of,
                      mirror_partials, parse_placements, run_oracle)
 
 pytestmark = pytest.mark.gpu
@@ -175,6 +175,61 @@ def test_float_conversions(gpu_device, src_dt, dst_dt):
         gpu_job.run()
         run_oracle(cpu_job)
         assert_bit_equal(gpu_job.target_locals[0][1], cpu_job.target_locals[0][1], f"{src_dt}->{dst_dt} {shape}")
+
+
+_VALUE_TYPES = [torch.float16, torch.bfloat16, torch.float32, torch.float64, torch.int8, torch.uint8, torch.int16, torch.int32,
+                torch.int64, torch.bool, torch.float8_e4m3fn, torch.float8_e5m2]
+
+
+@pytest.mark.parametrize("src", _VALUE_TYPES, ids=lambda d: str(d).replace("torch.", ""))
+def test_value_type_conversions(gpu_device, src):
+    """``Tensor.to`` between every pair of value types that involves an integer, bool or 8-bit float, on random bit
+    patterns, magnitudes around the integer limits (out of range included) and the committed special values:
+    the kernel's element-wise converter against the oracle's restatement of the reference path (torch's CPU casts)."""
+    import json
+    import os
+
+    with open(os.path.join(os.path.dirname(os.path.abspath(__file__)), "golden", "cast_kats.json")) as f:
+        kats = json.load(f)
+    name = {torch.float16: "f16", torch.bfloat16: "bf16", torch.float32: "f32", torch.float64: "f64",
+            torch.float8_e4m3fn: "e4m3", torch.float8_e5m2: "e5m2"}.get(src)
+
+    def fill(spec):
+        g = torch.Generator().manual_seed(11)
+        n = spec.shape[0] * spec.shape[1]
+        raw = torch.randint(0, 256, (n * src.itemsize,), generator=g, dtype=torch.uint8)
+        x = ((raw % 2).view(src) if src == torch.bool else raw.view(src)).clone()
+        if src.is_floating_point:
+            k = n // 3
+            x[:k] = (torch.randn(k, generator=g, dtype=torch.float64) * 300).to(src)
+            x[k:2 * k] = (torch.randn(k, generator=g, dtype=torch.float64) * 3e9).to(src)
+            special = np.array([int(v, 16) for v in kats["float_to_int"][f"{name}->i32"]["in"]], dtype=np.uint64)
+            raw_np = {1: np.uint8, 2: np.uint16, 4: np.uint32, 8: np.uint64}[src.itemsize]
+            x[2 * k:2 * k + len(special)] = torch.from_numpy(special.astype(raw_np).view(np.uint8).copy()).view(src)
+        return x.reshape(spec.shape)
+
+    for dst in _VALUE_TYPES:
+        if dst == src or (src in _VALUE_TYPES[:4] and dst in _VALUE_TYPES[:4]):
+            continue  # the four IEEE-style floats among themselves: test_float_conversions
+        spec = TensorSpec("w", (33, 50), mesh_of(0, [2]), (Shard(1),), mesh_of(2, [3]), (Shard(0),), src, dst, seed=5)
+        gpu_job = ReshardJob([spec], device=gpu_device, bucket_size=512, keep_globals=True, fill=fill)
+        cpu_job = ReshardJob([spec], device="cpu", bucket_size=512, keep_globals=True, fill=fill)
+        gpu_job.run()
+        run_oracle(cpu_job)
+        for r, got in gpu_job.target_locals[0].items():
+            want = cpu_job.target_locals[0][r]
+            a, b = bits(got).view(got.shape + (-1,)), bits(want).view(want.shape + (-1,))
+            same = (a == b).all(-1)
+            if dst.is_floating_point:  # NaN payloads are not pinned
+                same |= torch.isnan(got.cpu().to(torch.float64)) & torch.isnan(want.to(torch.float64))
+            assert bool(same.all()), f"{src} -> {dst} rank {r}: {int((~same).sum())} elements differ"
+
+
+def test_opaque_types_can_only_be_moved(gpu_device):
+    spec = TensorSpec("c", (8, 8), mesh_of(0, [1]), (Replicate(),), mesh_of(1, [1]), (Replicate(),), torch.complex64, torch.float32)
+    job = ReshardJob([spec], device=gpu_device, bucket_size=1 << 20, fill=lambda s: torch.zeros(s.shape, dtype=torch.complex64))
+    with pytest.raises(NotImplementedError, match="only floats, integers, bool and 8-bit floats are converted"):
+        job.run()
 
 
 def test_nan_stays_nan(gpu_device):

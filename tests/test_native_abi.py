@@ -69,8 +69,10 @@ def test_validation_rejects_bad_descriptors():
         nat.Table.create(_desc(bucket_lo=0x900000, bucket_hi=0x900000 + 100), upload=False)
     with pytest.raises(nat.EthaNativeError, match="ndim"):
         nat.Table.create(_desc(ndim=9), upload=False)
-    with pytest.raises(nat.EthaNativeError, match="only implemented between floating"):
+    with pytest.raises(nat.EthaNativeError, match="can only be moved, not converted"):
         nat.Table.create(_desc(tensor_dtype=nat.B32, wire_dtype=nat.F32), upload=False)
+    generic = nat.Table.create(_desc(tensor_dtype=nat.I32, wire_dtype=nat.F32), upload=False)  # a value type: converted
+    assert all(int(m) & (1 << 20) for tiles in generic.tiles() for m in tiles["meta"])
     with pytest.raises(nat.EthaNativeError, match="unknown"):
         nat.Table.create(_desc(wire_dtype=99), upload=False)
     with pytest.raises(nat.EthaNativeError, match="null tensor"):

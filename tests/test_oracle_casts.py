@@ -168,3 +168,96 @@ def test_reduce_is_fp32_rank_order():
         of = np.zeros(1, dtype=np.float32)
         assert co.lib().oracle_reduce(ch, of.ctypes.data, scratch.ctypes.data) == 0
         assert of[0] == np.float32(want)
+
+
+# ---- integers, bool and the 8-bit floats ------------------------------------------------------------------
+_TORCH = {co.F16: torch.float16, co.BF16: torch.bfloat16, co.F32: torch.float32, co.F64: torch.float64, co.I8: torch.int8,
+          co.U8: torch.uint8, co.I16: torch.int16, co.I32: torch.int32, co.I64: torch.int64, co.BOOL: torch.bool,
+          co.F8E4M3: torch.float8_e4m3fn, co.F8E5M2: torch.float8_e5m2}
+_RAW = {1: np.uint8, 2: np.uint16, 4: np.uint32, 8: np.uint64}
+_NAMES = {"f16": co.F16, "bf16": co.BF16, "f32": co.F32, "f64": co.F64, "e4m3": co.F8E4M3, "e5m2": co.F8E5M2, "i8": co.I8,
+          "u8": co.U8, "i16": co.I16, "i32": co.I32, "i64": co.I64, "bool": co.BOOL}
+
+
+def _kats():
+    import json
+    import os
+
+    with open(os.path.join(os.path.dirname(os.path.abspath(__file__)), "golden", "cast_kats.json")) as f:
+        return json.load(f)
+
+
+def _from_hex(values, size):
+    return np.array([int(v, 16) for v in values], dtype=np.uint64).astype(_RAW[size])
+
+
+def _is_nan(raw, dt):
+    t = torch.from_numpy(raw.view(np.uint8).copy()).view(_TORCH[dt])
+    return torch.isnan(t.to(torch.float64) if dt != co.F64 else t).numpy()
+
+
+@pytest.mark.parametrize("group", ["float_to_int", "float_to_float8", "int_to_float"])
+def test_value_casts_known_answers(group):
+    """Committed answers of torch's CPU ``Tensor.to`` for out-of-range floats, NaN into integers (what C++ leaves
+    undefined) and the 8-bit float limits: truncation, INT_MIN for what does not fit, uint8 through int64."""
+    for pair, kat in _kats()[group].items():
+        s, d = (_NAMES[n] for n in pair.split("->"))
+        src = _from_hex(kat["in"], co.lib().oracle_dtype_size(s))
+        want = _from_hex(kat["out"], co.lib().oracle_dtype_size(d))
+        got = co.cast(src, s, d, _RAW[co.lib().oracle_dtype_size(d)])
+        differ = got != want
+        if d in (co.F16, co.BF16, co.F32, co.F64, co.F8E4M3, co.F8E5M2):
+            differ &= ~(_is_nan(got, d) & _is_nan(want, d))  # NaN payloads are not pinned
+        assert not differ.any(), (pair, [kat["in"][i] for i in np.nonzero(differ)[0][:5]])
+
+
+def test_float8_to_f32_every_pattern():
+    for name, want in _kats()["float8_to_f32"].items():
+        dt = _NAMES[name]
+        got = co.cast(np.arange(256, dtype=np.uint8), dt, co.F32, np.uint32)
+        want = _from_hex(want, 4)
+        nan = _is_nan(want, co.F32)
+        assert np.array_equal(got[~nan], want[~nan]) and _is_nan(got, co.F32)[nan].all(), name
+        # and back: every finite pattern survives the round trip
+        back = co.cast(got, co.F32, dt, np.uint8)
+        assert np.array_equal(back[~nan], np.arange(256, dtype=np.uint8)[~nan])
+
+
+def test_float8_rounding_is_to_nearest_even_and_monotone():
+    """Independent of torch: every fp32 between two neighbouring 8-bit floats goes to the nearer one, ties to the
+    even one; the mapping is monotone over the finite range."""
+    for dt in (co.F8E4M3, co.F8E5M2):
+        vals = co.cast(np.arange(128, dtype=np.uint8), dt, co.F32, np.uint32).view(np.float32).astype(np.float64)
+        finite = np.isfinite(vals)
+        codes = np.arange(128)[finite]
+        vals = vals[finite]
+        for lo, hi, c_lo, c_hi in zip(vals[:-1], vals[1:], codes[:-1], codes[1:]):
+            mid = (lo + hi) / 2
+            for x, want in ((lo + (hi - lo) * 0.49, c_lo), (lo + (hi - lo) * 0.51, c_hi), (mid, c_lo if c_lo % 2 == 0 else c_hi)):
+                got = co.cast(np.array([np.float32(x)]).view(np.uint32), co.F32, dt, np.uint8)[0]
+                assert got == want, (dt, x, got, want)
+        xs = np.sort(np.random.RandomState(3).uniform(0, float(vals.max()), size=5000).astype(np.float32))
+        out = co.cast(xs.view(np.uint32), co.F32, dt, np.uint8)
+        assert np.all(np.diff(out.astype(np.int32)) >= 0)
+
+
+def test_every_value_cast_matches_torch_cpu():
+    """All 132 pairs of the twelve value types on random bit patterns and a spread of magnitudes, against torch's CPU
+    ``Tensor.to`` (the call the reference makes, ir.py:125-126,137-138)."""
+    g = torch.Generator().manual_seed(0)
+    for s, sdt in _TORCH.items():
+        raw = torch.randint(0, 256, (4000 * sdt.itemsize,), generator=g, dtype=torch.uint8)
+        x = (raw % 2).view(sdt) if sdt == torch.bool else raw.view(sdt)
+        if sdt.is_floating_point:
+            x = torch.cat([x, (torch.randn(3000, generator=g, dtype=torch.float64) * 300).to(sdt),
+                           (torch.randn(1000, generator=g, dtype=torch.float64) * 3e9).to(sdt)])
+        src = x.view(torch.uint8).numpy().view(_RAW[sdt.itemsize])
+        for d, ddt in _TORCH.items():
+            if s == d:
+                continue
+            want = x.to(ddt).view(torch.uint8).numpy().view(_RAW[ddt.itemsize])
+            got = co.cast(src, s, d, _RAW[ddt.itemsize])
+            differ = got != want
+            if ddt.is_floating_point:
+                differ &= ~(_is_nan(got, d) & _is_nan(want, d))
+            assert not differ.any(), (sdt, ddt, int(differ.sum()))

@@ -64,16 +64,19 @@ def _random_spec(rng, idx, wire_size):
     # one wire item size per batch: the reference cannot mix item sizes in a bucket unless every offset
     # happens to be a multiple of the larger one (its view(dtype) of the bucket slice raises, ir.py:252)
     pairs = {
-        1: [(torch.int8, torch.int8), (torch.uint8, torch.uint8)],
+        1: [(torch.int8, torch.int8), (torch.uint8, torch.uint8), (torch.float32, torch.int8), (torch.int8, torch.float16),
+            (torch.bfloat16, torch.float8_e4m3fn), (torch.float8_e5m2, torch.float32), (torch.bool, torch.int32),
+            (torch.float64, torch.uint8)],
         2: [(torch.bfloat16, torch.bfloat16), (torch.float16, torch.float16), (torch.bfloat16, torch.float32),
             (torch.float32, torch.bfloat16), (torch.float16, torch.float64), (torch.float64, torch.bfloat16),
-            (torch.float16, torch.bfloat16), (torch.float32, torch.float16)],
+            (torch.float16, torch.bfloat16), (torch.float32, torch.float16), (torch.int16, torch.float32),
+            (torch.float64, torch.int16)],
         4: [(torch.float32, torch.float32), (torch.int32, torch.int32), (torch.float32, torch.float64),
-            (torch.float64, torch.float32)],
-        8: [(torch.float64, torch.float64), (torch.int64, torch.int64)],
+            (torch.float64, torch.float32), (torch.int32, torch.float64), (torch.float32, torch.int32)],
+        8: [(torch.float64, torch.float64), (torch.int64, torch.int64), (torch.int64, torch.float64)],
     }[wire_size]
-    if partial:
-        pairs = [p for p in pairs if p[0] in FLOATS[:3]]
+    if partial:  # a Partial reduction accumulates in fp32 and needs f16/bf16/f32/f64 on both sides
+        pairs = [p for p in pairs if p[0] in FLOATS[:3] and p[1] in FLOATS]
     sdt, tdt = pairs[int(rng.integers(len(pairs)))]
     n_src = math.prod(src_mesh)
     # overlapping rank sets create LOCAL chunks; their wire dtype is the target dtype (as in the reference), so

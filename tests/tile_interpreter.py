@@ -15,7 +15,9 @@ import numpy as np
 from oracle import c_oracle as co
 
 THREADS = 256
-_CODE_RAW = {0: np.uint16, 1: np.uint16, 2: np.uint32, 3: np.uint64}
+_CODE_RAW = {0: np.uint16, 1: np.uint16, 2: np.uint32, 3: np.uint64,  # f16 bf16 f32 f64
+             8: np.uint8, 9: np.uint8, 10: np.uint16, 11: np.uint32, 12: np.uint64, 13: np.uint8, 14: np.uint8, 15: np.uint8}
+_CODE_SIZE = {k: np.dtype(v).itemsize for k, v in _CODE_RAW.items()}
 
 
 class HostArena:
@@ -150,9 +152,12 @@ def _execute(table, arena, direction, first, count, peers, ordered) -> None:
             # (for reduce tiles the a side is an offset from each peer's base: checked against the real addresses below)
             assert reduce or skew_a or np.all(a[sel] % ua == 0), "misaligned vector access on the a side"
             assert skew_b or np.all(b[sel] % ub == 0), "misaligned vector access on the b side"
+            generic = bool(int(m) & (1 << 20))  # an integer, bool or 8-bit float side: one element per unit
             if cvt and not reduce:  # typed accesses: every element must sit at a multiple of its size, skewed or not
-                esz = {0: 2, 1: 2, 2: 4, 3: 8}
-                assert np.all(a[sel] % esz[dta] == 0) and np.all(b[sel] % esz[dtb] == 0), "misaligned element"
+                assert np.all(a[sel] % _CODE_SIZE[dta] == 0) and np.all(b[sel] % _CODE_SIZE[dtb] == 0), "misaligned element"
+                assert generic == (dta > 3 or dtb > 3)
+                if generic:
+                    assert (ua, ub) == (_CODE_SIZE[dta], _CODE_SIZE[dtb]) and not vec
             if reduce:
                 _reduce_units(arena, mem, row_tiles, row_idx[sel], a[sel], b[sel], ua, ub, dta, dtb, peers, skew_a)
                 continue
