@@ -4,6 +4,7 @@ environment, derive the two paths, create the client."""
 from __future__ import annotations
 
 import ctypes
+import errno
 import logging
 import os
 from collections.abc import Callable
@@ -23,8 +24,12 @@ def setup_ptrace() -> None:
     libc.prctl.argtypes = [ctypes.c_int, ctypes.c_ulong, ctypes.c_ulong, ctypes.c_ulong, ctypes.c_ulong]
     if libc.prctl(PR_SET_PTRACER, pr_set_ptracer_any, 0, 0, 0) != 0:
         err = ctypes.get_errno()
-        # without Yama ptrace restrictions the call is not needed and fails with EINVAL: hipIPC still works
-        logger.warning("[Bootstrap] prctl(PR_SET_PTRACER, ANY) failed: errno %d (%s)", err, os.strerror(err))
+        if err == errno.EINVAL:
+            # a kernel without the Yama module does not know the option: there is no ptrace restriction to lift,
+            # and another process can open this one's allocations anyway
+            logger.info("[Bootstrap] prctl(PR_SET_PTRACER) is not known to this kernel (no ptrace restriction to lift)")
+        else:
+            logger.warning("[Bootstrap] prctl(PR_SET_PTRACER, ANY) failed: errno %d (%s)", err, os.strerror(err))
 
 
 @dataclass
