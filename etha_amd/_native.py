@@ -253,6 +253,16 @@ class Table:
             res.append(arr)
         return res[0], res[1]
 
+    def ordered_gather(self, first: int, count: int) -> np.ndarray:
+        """Piece addresses of the gather tiles of an optimized range (``peer_first`` of such a tile indexes it)."""
+        need = c_uint64()
+        _check("etha_table_read_ordered", lib().etha_table_read_ordered(self._h, first, count, 3, None, 0, byref(need)))
+        arr = np.zeros(need.value // 8, dtype=np.uint64)
+        if need.value:
+            _check("etha_table_read_ordered",
+                   lib().etha_table_read_ordered(self._h, first, count, 3, arr.ctypes.data, need.value, byref(need)))
+        return arr
+
     def pack(self, first: int, count: int, stream: int = 0, flags: int = 0) -> None:
         _check("etha_pack_bucket", lib().etha_pack_bucket(self._h, first, count, c_void_p(stream), flags))
 

@@ -83,7 +83,8 @@ struct RowTile {     // walks rows of `run` units; covers units [c0, c0+n) count
   uint32_t peer_first;  // reduce tiles: index of the first peer base in the peers array
   uint32_t n_peers;     // 0 = plain tile
   uint32_t reduce_op;
-  uint32_t via;         // reduce tiles: 0, or 1 + ETHA_* dtype the result is rounded to before the b-side dtype
+  uint32_t via;         // reduce tiles: 0, or 1 + ETHA_* dtype the result is rounded to before the b-side dtype;
+                        // gather tiles: units per piece
 };
 static_assert(sizeof(RowTile) == 64, "RowTile layout");
 
@@ -136,6 +137,10 @@ constexpr uint32_t kMetaSkew = 1u << 18;  // a-side addresses are not all multip
 constexpr uint32_t kMetaSkewB = 1u << 19; // same for the b side (both are bookkeeping for checkers: the kernel's
                                           // accesses are legal at any element-aligned address)
 constexpr uint32_t kMetaGeneric = 1u << 20;  // converting move with an integer, bool or 8-bit float side: one element per unit
+// Row tile of a write-ordered range whose rows are assembled from several chunks (unpack only): a row of `run`
+// units is n_peers pieces of `via` units each, piece p read at gather[peer_first + p] + row * b_pitch.  The a
+// side is addressed as in any row tile, so one wavefront writes whole destination lines.
+constexpr uint32_t kMetaGather = 1u << 21;
 
 // ---- typed vector access ----------------------------------------------------------------------
 typedef uint32_t u32x2 __attribute__((ext_vector_type(2)));
@@ -405,7 +410,8 @@ __device__ __forceinline__ void row_position(const RowTile& t, uint32_t tid, uin
 // pack (REV = false): a -> b.   unpack (REV = true): b -> a.
 template <bool REV>
 __global__ __launch_bounds__(ETHA_BLOCK_THREADS) void etha_tile_kernel(const RunTile* __restrict__ run_tiles, uint32_t n_run,
-                                                                        const RowTile* __restrict__ row_tiles) {
+                                                                        const RowTile* __restrict__ row_tiles,
+                                                                        const uint64_t* __restrict__ gather) {
   const uint32_t bid = blockIdx.x / kBlocksPerTile;
   const uint32_t tid = (blockIdx.x % kBlocksPerTile) * kBlockThreads + threadIdx.x;
   uint64_t a, b;
@@ -423,7 +429,13 @@ __global__ __launch_bounds__(ETHA_BLOCK_THREADS) void etha_tile_kernel(const Run
     uint32_t r, c;
     row_position(t, tid, r, c);
     a = t.a + (uint64_t)((int64_t)r * t.a_pitch) + ((uint64_t)c << ((meta >> kMetaUaShift) & 15u));
-    b = t.b + (uint64_t)((int64_t)r * t.b_pitch) + ((uint64_t)c << ((meta >> kMetaUbShift) & 15u));
+    if (REV && (meta & kMetaGather)) {
+      if (tid >= n) return;
+      const uint32_t p = c / t.via;
+      b = gather[t.peer_first + p] + (uint64_t)((int64_t)r * t.b_pitch) + ((uint64_t)(c - p * t.via) << ((meta >> kMetaUbShift) & 15u));
+    } else {
+      b = t.b + (uint64_t)((int64_t)r * t.b_pitch) + ((uint64_t)c << ((meta >> kMetaUbShift) & 15u));
+    }
   }
   if (tid >= n) return;
   move_unit<REV>(meta, a, b);
@@ -872,6 +884,7 @@ struct Builder {
   uint64_t payload_bytes = 0;
 };
 
+constexpr uint64_t kShortRowUnits = 64;  // rows of at most this many units never straddle a tile
 constexpr uint64_t kMaxTiles = 0x7fff0000ull / kBlocksPerTile;  // grid.x limit with margin
 
 struct ReduceSpec {
@@ -1138,11 +1151,14 @@ class PairCompiler {
         const uint64_t rows = k_ > 0 ? (uint64_t)n_[k_ - 1] : 1;
         const int64_t pa = k_ > 0 ? sa_[k_ - 1] : 0, pb = k_ > 0 ? sb_[k_ - 1] : 0;
         const uint64_t total = rows * run_units;
-        for (uint64_t q = 0; q < total; q += kTileThreads) {
+        // tiles of short rows hold whole rows (a few lanes of the last workgroup stay idle): such tiles can be
+        // regrouped row-wise with the tiles of neighbouring chunks when a range is ordered by written address
+        const uint64_t step = rows > 1 && run_units <= kShortRowUnits ? (kTileThreads / run_units) * run_units : kTileThreads;
+        for (uint64_t q = 0; q < total; q += step) {
           RowTile t;
           memset(&t, 0, sizeof(t));
           const uint64_t left = total - q;
-          t.n = (uint32_t)(left < kTileThreads ? left : kTileThreads);
+          t.n = (uint32_t)(left < step ? left : step);
           t.meta = meta;
           if (rows == 1) {  // one (possibly very long) run: address the tile directly
             t.a = a0 + q * ua;
@@ -1215,8 +1231,10 @@ struct EthaTable {
   struct Ordered {
     std::vector<RunTile> h_run;
     std::vector<RowTile> h_row;
+    std::vector<uint64_t> h_gather;  // piece addresses of the gather tiles
     RunTile* d_run = nullptr;
     RowTile* d_row = nullptr;
+    uint64_t* d_gather = nullptr;
   };
   std::map<std::pair<uint32_t, uint32_t>, Ordered> ordered;
 };
@@ -1261,6 +1279,7 @@ void free_table(EthaTable* t) {
   for (auto& kv : t->ordered) {
     if (kv.second.d_run) (void)hipFree(kv.second.d_run);
     if (kv.second.d_row) (void)hipFree(kv.second.d_row);
+    if (kv.second.d_gather) (void)hipFree(kv.second.d_gather);
   }
   delete t;
 }
@@ -1315,7 +1334,7 @@ template <bool REV>
 int launch_tiles(const EthaTable* t, uint32_t first, uint32_t count, void* stream, uint32_t flags) {
   const uint32_t r0 = t->run_begin[first], r1 = t->run_begin[first + count];
   const uint32_t w0 = t->row_begin[first], w1 = t->row_begin[first + count];
-  const uint32_t n_run = r1 - r0, n_row = w1 - w0;
+  uint32_t n_run = r1 - r0, n_row = w1 - w0;
   const uint32_t x0 = t->trans_begin[first], n_trans = t->trans_begin[first + count] - x0;
   if (n_trans) {  // transposing chunks run in their own kernel (it needs LDS)
     launch_kernel(etha_transpose_kernel<REV>, dim3(n_trans), dim3(kTransThreads), t->trans_lds, stream, flags,
@@ -1326,15 +1345,19 @@ int launch_tiles(const EthaTable* t, uint32_t first, uint32_t count, void* strea
   if (n_run + n_row == 0) return ETHA_OK;
   const RunTile* d_run = t->d_run + r0;
   const RowTile* d_row = t->d_row + w0;
+  const uint64_t* d_gather = nullptr;
   if (REV == (t->kind == 0)) {  // the direction that writes the a side (unpack) / b side (self-copy) of an ordered range
     auto it = t->ordered.find(std::make_pair(first, count));
     if (it != t->ordered.end()) {
       d_run = it->second.d_run;
       d_row = it->second.d_row;
+      d_gather = it->second.d_gather;
+      n_run = (uint32_t)it->second.h_run.size();  // gathering regroups row tiles: their number may differ
+      n_row = (uint32_t)it->second.h_row.size();
     }
   }
   launch_kernel(etha_tile_kernel<REV>, dim3((n_run + n_row) * kBlocksPerTile), dim3(kBlockThreads), 0, stream, flags, d_run,
-                n_run, d_row);
+                n_run, d_row, d_gather);
   HIP_TRY(hipGetLastError());
   return ETHA_OK;
 }
@@ -1346,6 +1369,62 @@ int launch_reduce(const EthaTable* t, uint32_t first, uint32_t count, void* stre
                 (const RowTile*)(t->d_row + w0), (const uint64_t*)t->d_peers);
   HIP_TRY(hipGetLastError());
   return ETHA_OK;
+}
+
+// Short pieces of one destination row that arrive through different chunks (a target row assembled from
+// several source ranks' column blocks): written one piece per tile, every 64-byte DRAM burst is written in parts
+// by different workgroups, which costs more than half the bandwidth at 32-byte pieces.  In a write-ordered range
+// the tiles of such sibling chunks are neighbours (same rows, adjacent columns).  P of them, each covering R rows,
+// are replaced by about P gather tiles that cover about R / P rows each but all P pieces of every row, so that one
+// wavefront writes whole lines and reads P short streams.  Bytes moved are the same.
+constexpr uint32_t kGatherMaxPieceBytes = 64;
+constexpr uint32_t kGatherMaxPieces = 8;
+
+void gather_short_pieces(std::vector<RowTile>& rows, std::vector<uint64_t>& gather) {
+  std::vector<RowTile> out;
+  out.reserve(rows.size());
+  size_t i = 0;
+  while (i < rows.size()) {
+    const RowTile& x = rows[i];
+    const uint32_t ua = (x.meta >> kMetaUaShift) & 15u;
+    const uint64_t piece = (uint64_t)x.run << ua;
+    bool ok = x.n_peers == 0 && x.c0 == 0 && x.run < kTileThreads && x.n % x.run == 0 && piece <= kGatherMaxPieceBytes &&
+              x.a_pitch > 0 && !(x.meta & kMetaGather);
+    uint32_t have = 1;
+    if (ok) {
+      while (have < kGatherMaxPieces && i + have < rows.size()) {
+        const RowTile& y = rows[i + have];
+        if (y.n_peers != 0 || y.c0 != 0 || y.n != x.n || y.run != x.run || y.meta != x.meta || y.a_pitch != x.a_pitch ||
+            y.b_pitch != x.b_pitch || y.a != x.a + have * piece || (uint64_t)(have + 1) * piece > (uint64_t)x.a_pitch ||
+            (uint64_t)(have + 1) * x.run > kTileThreads)
+          break;
+        have++;
+      }
+    }
+    const uint32_t n_rows = ok ? x.n / x.run : 0, pieces = have;
+    if (!ok || pieces < 2) {
+      out.push_back(x);
+      i++;
+      continue;
+    }
+    const uint32_t rows_cap = kTileThreads / (x.run * pieces);  // rows one gather tile can hold
+    for (uint32_t row0 = 0; row0 < n_rows; row0 += rows_cap) {
+      RowTile g = x;
+      g.a = x.a + (uint64_t)row0 * (uint64_t)x.a_pitch;
+      g.b = (uint64_t)((int64_t)x.b + (int64_t)row0 * x.b_pitch);  // piece 0, for inspection only
+      g.meta = x.meta | kMetaGather;
+      g.run = x.run * pieces;
+      g.n = (n_rows - row0 < rows_cap ? n_rows - row0 : rows_cap) * g.run;
+      g.peer_first = (uint32_t)gather.size();
+      g.n_peers = pieces;
+      g.via = x.run;
+      for (uint32_t p2 = 0; p2 < pieces; p2++)
+        gather.push_back((uint64_t)((int64_t)rows[i + p2].b + (int64_t)row0 * x.b_pitch));
+      out.push_back(g);
+    }
+    i += pieces;
+  }
+  rows.swap(out);
 }
 
 int check_flags(uint32_t flags) {
@@ -1583,19 +1662,24 @@ int etha_table_optimize_range(EthaTable* t, uint32_t first, uint32_t count) {
     const uint64_t px = (by_a ? x.a : x.b) + x.c0 * unit(x.meta, by_a), py = (by_a ? y.a : y.b) + y.c0 * unit(y.meta, by_a);
     return px < py;
   });
+  if (by_a) gather_short_pieces(o.h_row, o.h_gather);
   if (t->uploaded) {
     const size_t run_bytes = o.h_run.size() * sizeof(RunTile), row_bytes = o.h_row.size() * sizeof(RowTile);
+    const size_t gather_bytes = o.h_gather.size() * sizeof(uint64_t);
     hipError_t e = hipSuccess;
     if (run_bytes) e = hipMalloc(&o.d_run, run_bytes);
     if (e == hipSuccess && run_bytes) e = hipMemcpy(o.d_run, o.h_run.data(), run_bytes, hipMemcpyHostToDevice);
     if (e == hipSuccess && row_bytes) e = hipMalloc(&o.d_row, row_bytes);
     if (e == hipSuccess && row_bytes) e = hipMemcpy(o.d_row, o.h_row.data(), row_bytes, hipMemcpyHostToDevice);
+    if (e == hipSuccess && gather_bytes) e = hipMalloc(&o.d_gather, gather_bytes);
+    if (e == hipSuccess && gather_bytes) e = hipMemcpy(o.d_gather, o.h_gather.data(), gather_bytes, hipMemcpyHostToDevice);
     if (e != hipSuccess) {
       if (o.d_run) (void)hipFree(o.d_run);
       if (o.d_row) (void)hipFree(o.d_row);
+      if (o.d_gather) (void)hipFree(o.d_gather);
       return fail(ETHA_ERR_HIP, "uploading the ordered range: %s", hipGetErrorString(e));
     }
-    t->device_bytes += run_bytes + row_bytes;
+    t->device_bytes += run_bytes + row_bytes + gather_bytes;
   }
   t->ordered.emplace(key, std::move(o));
   return ETHA_OK;
@@ -1606,9 +1690,13 @@ int etha_table_read_ordered(const EthaTable* t, uint32_t first, uint32_t count, 
   if (!t || !need_bytes) return fail(ETHA_ERR_INVALID, "null argument");
   auto it = t->ordered.find(std::make_pair(first, count));
   if (it == t->ordered.end()) return fail(ETHA_ERR_INVALID, "range [%u,+%u) has not been optimized", first, count);
-  if (which != 0 && which != 1) return fail(ETHA_ERR_INVALID, "which must be 0 or 1");
-  const void* src = which == 0 ? (const void*)it->second.h_run.data() : (const void*)it->second.h_row.data();
-  const uint64_t bytes = which == 0 ? it->second.h_run.size() * sizeof(RunTile) : it->second.h_row.size() * sizeof(RowTile);
+  if (which != 0 && which != 1 && which != 3) return fail(ETHA_ERR_INVALID, "which must be 0, 1 or 3");
+  const void* src = which == 0   ? (const void*)it->second.h_run.data()
+                    : which == 1 ? (const void*)it->second.h_row.data()
+                                 : (const void*)it->second.h_gather.data();
+  const uint64_t bytes = which == 0   ? it->second.h_run.size() * sizeof(RunTile)
+                         : which == 1 ? it->second.h_row.size() * sizeof(RowTile)
+                                      : it->second.h_gather.size() * sizeof(uint64_t);
   *need_bytes = bytes;
   if (out && bytes) memcpy(out, src, bytes < cap_bytes ? bytes : cap_bytes);
   return ETHA_OK;
@@ -1752,7 +1840,7 @@ int etha_copy_regions_noalloc(const EthaChunkDesc* src, const EthaChunkDesc* dst
   const uint32_t n_run = (uint32_t)bld.run.size(), n_row = (uint32_t)bld.row.size();
   if (n_run + n_row) {
     launch_kernel(etha_tile_kernel<false>, dim3((n_run + n_row) * kBlocksPerTile), dim3(kBlockThreads), 0, stream, 0,
-                  (const RunTile*)base, n_run, (const RowTile*)(base + row_off));
+                  (const RunTile*)base, n_run, (const RowTile*)(base + row_off), (const uint64_t*)nullptr);
     HIP_TRY(hipGetLastError());
   }
   return ETHA_OK;

@@ -894,3 +894,25 @@ def test_large_resident_set_70b_shapes(gpu_device):
         del glob, want
     del job
     torch.cuda.empty_cache()  # hand the 150 GB back before the multi-process tests start
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("pool", ["ring", "resident"])
+@pytest.mark.parametrize("cols,src_dtype,tgt_dtype", [(64, torch.bfloat16, None), (32, torch.bfloat16, None),
+                                                      (48, torch.float32, torch.bfloat16), (32, torch.bfloat16, torch.float32)])
+def test_short_pieces_from_several_ranks_are_gathered_per_row(gpu_device, pool, cols, src_dtype, tgt_dtype):
+    """Every target row is four short pieces from four source ranks' buckets.  Merged unpack launches run from the
+    write-ordered copy of their range, where such pieces are assembled row by row by gather tiles."""
+    from etha_amd.comm.comm_methods import _UNPACK
+
+    specs = [TensorSpec(f"t{i}", (2048 + 512 * i, cols), [[0, 1, 2, 3]], (Replicate(), Shard(1)), [4], (Replicate(),),
+                        src_dtype, tgt_dtype, seed=40 + i, std=1.0) for i in range(3)]
+    job, _ = gpu_vs_oracle(specs, gpu_device, 256 * 1024, merge_launches=True, pool=pool)
+    job.run(merge_launches=True)  # the schedule repeats: by now every recurring merged range has its ordered copy
+    plan = job.wire.plan(job.recv_buckets[4])
+    ranges = plan._ordered_ranges if pool == "ring" else {(k, f, c) for k, f, c, s in plan.merged_steps if len(s) > 1}
+    gathered = sum(len(plan.recv_table.ordered_gather(f, c)) for k, f, c in ranges if k == _UNPACK)
+    assert gathered > 0
+    for i, spec in enumerate(specs):
+        want = expected_target(spec, job.globals_[i].cpu(), 4)
+        assert_bit_equal(job.target_locals[i][4], want, spec.name)

@@ -260,6 +260,60 @@ def test_optimized_range_is_a_write_ordered_permutation():
         table.ordered_tiles(0, 2)
 
 
+@pytest.mark.parametrize("rows,cols,blocks,tdt,wdt", [
+    (1024, 64, 4, nat.BF16, nat.BF16),   # 32-byte pieces: four per 128-byte row
+    (1024, 64, 8, nat.BF16, nat.BF16),   # 16-byte pieces: one unit each
+    (1500, 96, 3, nat.BF16, nat.BF16),   # 64-byte pieces, three siblings, a last tile with fewer rows
+    (640, 96, 4, nat.F32, nat.BF16),     # converting: 96-byte pieces on the tensor side are left alone ...
+    (640, 48, 6, nat.F32, nat.BF16),     # ... 32-byte ones are gathered (16 bytes each in the bucket)
+    (333, 40, 5, nat.B8, nat.B8),        # 8-byte pieces of byte elements
+    (1000, 36, 3, nat.BF16, nat.BF16),   # 24-byte pieces: three 8-byte units, tiles hold whole rows
+    (777, 48, 3, nat.BF16, nat.BF16),    # three 32-byte pieces per 96-byte row
+    (515, 35, 7, nat.B8, nat.B8),        # 5-byte pieces: byte units
+])
+def test_short_pieces_of_one_row_are_gathered_in_an_ordered_range(rows, cols, blocks, tdt, wdt):
+    """Column blocks of one tensor arrive through different buckets.  When the pieces are short, the ordered range
+    holds gather tiles: each assembles whole rows from the pieces of several chunks.  Same bytes as the plain
+    tiles, every destination byte written exactly once."""
+    from tile_interpreter import GATHER
+
+    es_t, es_w = ES[tdt], ES[wdt]
+    piece = cols // blocks
+    results = []
+    for ordered in (False, True):
+        arena = HostArena(rows * cols * (es_t + es_w) + 65536)
+        t = arena.alloc(rows * cols * es_t)
+        descs = []
+        seed = np.random.RandomState(11)
+        for j in range(blocks):
+            nb = rows * piece * es_w
+            b = arena.alloc(nb)
+            if wdt == nat.BF16:  # finite values, so that a conversion has something to show
+                vals = seed.randn(rows * piece).astype(np.float32)
+                arena.bytes_at(b, nb)[:] = (vals.view(np.uint32) >> 16).astype(np.uint16).view(np.uint8)
+            else:
+                arena.bytes_at(b, nb)[:] = seed.randint(0, 256, nb)
+            descs.append(_mk_desc(t, t, t + rows * cols * es_t, b, b, b + nb, (0, j * piece), (rows, piece), (cols, 1), tdt, wdt))
+        table = nat.Table.create(np.stack(descs), upload=False)
+        if ordered:
+            table.optimize_range(0, blocks)
+            _, o_row = table.ordered_tiles(0, blocks)
+            gathered = (o_row["meta"] & GATHER) != 0
+            assert gathered.any() == (piece * es_t <= 64)
+            if gathered.any():
+                g = o_row[gathered]
+                assert np.all(g["n_peers"] >= 2) and np.all(g["run"] == g["via"] * g["n_peers"])
+                assert len(table.ordered_gather(0, blocks)) == int(g["n_peers"].sum())
+                # the plain tiles of the range are untouched: another range, or a pack, still uses them
+                assert not np.any(table.tiles()[1]["meta"] & GATHER)
+        arena.writes = np.zeros(arena.nbytes, dtype=np.int32)
+        execute(table, arena, "unpack", 0, blocks, ordered=ordered)
+        counts = arena.writes[arena.offsets(np.array([t]), 1)[0]:][: rows * cols * es_t]
+        assert np.all(counts == 1)
+        results.append(arena.bytes_at(t, rows * cols * es_t).copy())
+    assert np.array_equal(results[0], results[1])
+
+
 @pytest.mark.parametrize("dt", [nat.B8, nat.BF16, nat.F32, nat.B64])
 def test_transposed_parent_uses_lds_blocks(dt):
     """A chunk of a transposed view: the tensor side is contiguous along dim 0, the bucket along dim 1."""

@@ -67,7 +67,10 @@ class AbsoluteMemory:
         return off
 
 
-def _unit_positions(run_tiles, row_tiles):
+GATHER = 1 << 21  # row tile that assembles each row from pieces of several chunks (ordered unpack ranges only)
+
+
+def _unit_positions(run_tiles, row_tiles, gather=None):
     """Per active work-item: (a address, b address, meta, tile kind, row-tile index)."""
     out = []
     if len(run_tiles):
@@ -93,6 +96,13 @@ def _unit_positions(run_tiles, row_tiles):
         assert np.all(c < run) and np.all(c >= 0)
         a = t["a"].astype(np.int64) + r * t["a_pitch"] + (c << (meta & 15))
         b = t["b"].astype(np.int64) + r * t["b_pitch"] + (c << ((meta >> 4) & 15))
+        g = (meta & GATHER) != 0
+        if g.any():
+            assert gather is not None and np.all(t["n_peers"][g] >= 2) and np.all(t["via"][g] > 0)
+            assert np.all(t["run"][g] == t["via"][g] * t["n_peers"][g]) and np.all(t["c0"][g] == 0)
+            piece = c[g] // t["via"][g].astype(np.int64)
+            base = gather[t["peer_first"][g].astype(np.int64) + piece].astype(np.int64)
+            b[g] = base + r[g] * t["b_pitch"][g] + ((c[g] - piece * t["via"][g].astype(np.int64)) << ((meta[g] >> 4) & 15))
         out.append((a, b, meta, rep))
     return out
 
@@ -127,8 +137,11 @@ def _execute(table, arena, direction, first, count, peers, ordered) -> None:
     run_begin, row_begin = table.ranges()
     if count is None:
         count = len(run_begin) - 1 - first
+    gather = None
     if ordered:
         run_tiles, row_tiles = table.ordered_tiles(first, count)
+        gather = table.ordered_gather(first, count)
+        assert direction == "unpack" or not np.any(row_tiles["meta"] & GATHER)
     else:
         run_tiles, row_tiles = table.tiles()
         run_tiles = run_tiles[run_begin[first] : run_begin[first + count]]
@@ -141,14 +154,14 @@ def _execute(table, arena, direction, first, count, peers, ordered) -> None:
     assert np.all(run_tiles["n"] > 0) and np.all(row_tiles["n"] > 0)
     rev = direction == "unpack"
     mem = arena.buf[arena.pad : arena.pad + arena.nbytes]
-    for a, b, meta, row_idx in _unit_positions(run_tiles, row_tiles):
+    for a, b, meta, row_idx in _unit_positions(run_tiles, row_tiles, gather):
         for m in np.unique(meta):
             sel = meta == m
             ua, ub = 1 << (int(m) & 15), 1 << ((int(m) >> 4) & 15)
             dta, dtb = (int(m) >> 8) & 15, (int(m) >> 12) & 15
             cvt, vec = bool(int(m) & (1 << 16)), bool(int(m) & (1 << 17))
             skew_a, skew_b = bool(int(m) & (1 << 18)), bool(int(m) & (1 << 19))
-            reduce = row_idx[sel][0] >= 0 and int(row_tiles["n_peers"][row_idx[sel][0]]) > 0
+            reduce = row_idx[sel][0] >= 0 and int(row_tiles["n_peers"][row_idx[sel][0]]) > 0 and not (int(m) & GATHER)
             # (for reduce tiles the a side is an offset from each peer's base: checked against the real addresses below)
             assert reduce or skew_a or np.all(a[sel] % ua == 0), "misaligned vector access on the a side"
             assert skew_b or np.all(b[sel] % ub == 0), "misaligned vector access on the b side"
