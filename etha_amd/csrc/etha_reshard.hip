@@ -141,6 +141,8 @@ constexpr uint32_t kMetaGeneric = 1u << 20;  // converting move with an integer,
 // units is n_peers pieces of `via` units each, piece p read at gather[peer_first + p] + row * b_pitch.  The a
 // side is addressed as in any row tile, so one wavefront writes whole destination lines.
 constexpr uint32_t kMetaGather = 1u << 21;
+constexpr uint32_t kGatherMaxPieceBytes = 64;  // longer pieces already write whole lines: gathering them costs more than it gives
+constexpr uint32_t kGatherMaxPieces = 8;       // the kernel reads this many piece addresses per tile (the list is padded)
 
 // ---- typed vector access ----------------------------------------------------------------------
 typedef uint32_t u32x2 __attribute__((ext_vector_type(2)));
@@ -432,7 +434,18 @@ __global__ __launch_bounds__(ETHA_BLOCK_THREADS) void etha_tile_kernel(const Run
     if (REV && (meta & kMetaGather)) {
       if (tid >= n) return;
       const uint32_t p = c / t.via;
-      b = gather[t.peer_first + p] + (uint64_t)((int64_t)r * t.b_pitch) + ((uint64_t)(c - p * t.via) << ((meta >> kMetaUbShift) & 15u));
+      // the tile's piece addresses are the same for every lane: fetched through the scalar path, picked per lane
+      const uint64_t* pieces = gather + t.peer_first;
+      uint64_t base = 0;
+#pragma unroll
+      for (uint32_t j = 0; j < kGatherMaxPieces; j++) {
+        const uint64_t v = pieces[j];  // readfirstlane keeps each of these a scalar load of its own
+        // (the builtin returns a signed int: go through uint32_t, or the low word would be sign-extended)
+        const uint64_t u = ((uint64_t)(uint32_t)__builtin_amdgcn_readfirstlane((int)(uint32_t)(v >> 32)) << 32) |
+                           (uint64_t)(uint32_t)__builtin_amdgcn_readfirstlane((int)(uint32_t)v);
+        base = p == j ? u : base;
+      }
+      b = base + (uint64_t)((int64_t)r * t.b_pitch) + ((uint64_t)(c - p * t.via) << ((meta >> kMetaUbShift) & 15u));
     } else {
       b = t.b + (uint64_t)((int64_t)r * t.b_pitch) + ((uint64_t)c << ((meta >> kMetaUbShift) & 15u));
     }
@@ -884,7 +897,10 @@ struct Builder {
   uint64_t payload_bytes = 0;
 };
 
-constexpr uint64_t kShortRowUnits = 64;  // rows of at most this many units never straddle a tile
+#ifndef ETHA_SHORT_ROW_UNITS
+#define ETHA_SHORT_ROW_UNITS 64
+#endif
+constexpr uint64_t kShortRowUnits = ETHA_SHORT_ROW_UNITS;  // rows of at most this many units never straddle a tile
 constexpr uint64_t kMaxTiles = 0x7fff0000ull / kBlocksPerTile;  // grid.x limit with margin
 
 struct ReduceSpec {
@@ -1377,8 +1393,6 @@ int launch_reduce(const EthaTable* t, uint32_t first, uint32_t count, void* stre
 // the tiles of such sibling chunks are neighbours (same rows, adjacent columns).  P of them, each covering R rows,
 // are replaced by about P gather tiles that cover about R / P rows each but all P pieces of every row, so that one
 // wavefront writes whole lines and reads P short streams.  Bytes moved are the same.
-constexpr uint32_t kGatherMaxPieceBytes = 64;
-constexpr uint32_t kGatherMaxPieces = 8;
 
 void gather_short_pieces(std::vector<RowTile>& rows, std::vector<uint64_t>& gather) {
   std::vector<RowTile> out;
@@ -1425,6 +1439,7 @@ void gather_short_pieces(std::vector<RowTile>& rows, std::vector<uint64_t>& gath
     i += pieces;
   }
   rows.swap(out);
+  if (!gather.empty()) gather.insert(gather.end(), kGatherMaxPieces, 0);  // a tile's fetch may run past its own pieces
 }
 
 int check_flags(uint32_t flags) {
