@@ -36,6 +36,9 @@ def parse_args():
                     help="strictly one launch per bucket (default: buckets that become ready together and are neighbours "
                          "in their table share a launch)")
     ap.add_argument("--in-order", action="store_true", help="issue every launch ordered after the previous one")
+    ap.add_argument("--no-sets", action="store_true",
+                    help="one kernel launch per bucket step instead of shared launches for independent steps "
+                         "(implied by --per-bucket)")
     ap.add_argument("--fanout", type=int, default=1, help="side streams for per-bucket launches (resident pool only)")
     ap.add_argument("--zero-copy", action="store_true",
                     help="lend contiguous single-chunk buckets to the consumer instead of packing them")
@@ -240,13 +243,17 @@ def time_steps(job, steps, run):
 
 
 def launches_per_step(job, run):
+    """(kernel launches, bucket steps, bucket steps issued unordered) of one step."""
     import torch
 
+    from etha_amd import _native
+
     log = job.wire.launch_log = []
+    before = _native.kernel_launches()
     run()
     torch.cuda.synchronize()
     job.wire.launch_log = None
-    return len(log), sum(1 for entry in log if entry[3] & 1)
+    return _native.kernel_launches() - before, len(log), sum(1 for entry in log if entry[3] & 1)
 
 
 def main():
@@ -281,6 +288,8 @@ def main():
     t0 = time.time()
     job = make_job(args.pool, args.max_in_flight)
     job.wire.unordered_launches = not args.in_order
+    sets = not (args.no_sets or args.per_bucket)
+    job.wire.group_launches = sets
     for _ in range(max(args.warmup, 1)):  # plans (compiles the tile programs) + warm-up
         job.run(merge_launches=merge, fanout=args.fanout)
     setup_s = time.time() - t0
@@ -294,12 +303,11 @@ def main():
         graph.replay()
     step = graph.replay if graph is not None else (lambda: job.run(merge_launches=merge, fanout=args.fanout, synchronize=False))
     dev_ms, step_ms = time_steps(job, args.steps, step)
-    if args.pool == "ring":
-        n_launch, n_unordered = launches_per_step(job, lambda: job.run(merge_launches=merge, synchronize=False))
-    else:
+    n_launch, n_steps, n_unordered = launches_per_step(
+        job, lambda: job.run(merge_launches=merge, fanout=args.fanout, synchronize=False))
+    if args.pool != "ring":
         plans = [job.wire.plan(b) for bs in (job.send_buckets, job.recv_buckets) for b in bs.values()]
-        n_launch = sum(1 for p in plans for s in (p.merged_steps if merge else p.steps) if s[0] != "lend")
-        n_unordered = 0
+        n_steps = sum(1 for p in plans for s in (p.merged_steps if merge else p.steps) if s[0] != "lend")
 
     kernels = []
     tables = [t for p in (job.wire.plan(b) for bs in (job.send_buckets, job.recv_buckets) for b in bs.values())
@@ -312,8 +320,9 @@ def main():
     if kinds & {"reduce_pack", "direct_reduce"}:
         kernels.insert(0, "etha_reduce_kernel")
     granularity = ("bucket" if not merge else
-                   "buckets ready together" if args.pool == "ring" else "run of buckets")
-    mode = f"{args.pool}/{'bucket' if not merge else 'runs'}"
+                   "run of buckets" if args.pool != "ring" else
+                   "independent steps share launches" if sets else "buckets ready together")
+    mode = f"{args.pool}/{'bucket' if not merge else 'sets' if sets and args.pool == 'ring' else 'runs'}"
     element = str(specs[0].source_dtype).replace("torch.", "")
     achieved = total_bytes / (dev_ms * 1e-3) / 1e9
     traffic = None if (args.zero_copy or args.direct or args.graph or args.fanout > 1 or args.in_order
@@ -350,7 +359,8 @@ def main():
         "pct_of_hbm_peak": round(100.0 * achieved / HBM_PEAK_GBS, 2),
         "algorithmic_bytes_per_step": {"pack": pack_bytes, "unpack": unpack_bytes, "of_which_self_copy": self_bytes},
         "launches_per_step": n_launch,
-        "unordered_launches_per_step": n_unordered,
+        "bucket_steps_per_step": n_steps,
+        "unordered_bucket_steps_per_step": n_unordered,
         "roofline": {
             "bound": "hbm",
             "kernel": " + ".join(kernels),
@@ -391,18 +401,26 @@ def main():
     if plain and args.pool == "ring":
         # the same step in its other forms, for comparison (none of them is `value`)
         pool_bytes = job.wire.pool.reserved_bytes if job.wire.pool is not None else 0
-        other = not merge
-        ms = leg(job, merge_launches=other)
-        n, _ = launches_per_step(job, lambda: job.run(merge_launches=other, synchronize=False))
-        out["one_launch_per_bucket" if merge else "buckets_ready_together"] = describe(ms, n, pool_bytes)
-        job.wire.unordered_launches = False
-        out["every_launch_in_order"] = describe(leg(job, merge_launches=merge), n_launch, pool_bytes)
-        job.wire.unordered_launches = True
+        def other_leg(merge_, sets_, unordered=True):
+            job.wire.group_launches, job.wire.unordered_launches = sets_, unordered
+            ms = leg(job, merge_launches=merge_)
+            n = launches_per_step(job, lambda: job.run(merge_launches=merge_, synchronize=False))[0]
+            job.wire.group_launches, job.wire.unordered_launches = sets, True
+            return describe(ms, n, pool_bytes)
+
+        if merge or sets:
+            out["one_launch_per_bucket"] = other_leg(False, False)
+        if not (merge and not sets):
+            out["one_launch_per_run_of_buckets"] = other_leg(True, False)
+        if not (merge and sets):
+            out["independent_steps_share_launches"] = other_leg(True, True)
+        out["every_launch_in_order"] = other_leg(merge, False, unordered=False)
         del job
         torch.cuda.empty_cache()
         deeper = make_job("ring", 2 * args.max_in_flight)
+        deeper.wire.group_launches = sets
         ms = leg(deeper, merge_launches=merge)
-        n, _ = launches_per_step(deeper, lambda: deeper.run(merge_launches=merge, synchronize=False))
+        n = launches_per_step(deeper, lambda: deeper.run(merge_launches=merge, synchronize=False))[0]
         out[f"ring_of_{2 * args.max_in_flight}_slots"] = describe(ms, n, deeper.wire.pool.reserved_bytes if deeper.wire.pool else 0)
         del deeper
         torch.cuda.empty_cache()

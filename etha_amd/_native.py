@@ -14,8 +14,10 @@ import numpy as np
 from .build import LIB_PATH
 
 ETHA_MAX_NDIM = 8
-ABI_VERSION = 4
+ABI_VERSION = 5
 LAUNCH_UNORDERED = 1  # ETHA_LAUNCH_UNORDERED
+SEG_PACK, SEG_UNPACK, SEG_REDUCE_PACK, SEG_SELFCOPY = 0, 1, 2, 3  # ETHA_SEG_*
+MAX_SEGMENTS = 16
 
 # element type codes (include/etha_reshard.h)
 F16, BF16, F32, F64, B8, B16, B32, B64, I8, U8, I16, I32, I64, BOOL, F8E4M3, F8E5M2 = range(16)
@@ -68,6 +70,12 @@ TRANS_TILE = np.dtype([("a", "<u8"), ("b", "<u8"), ("a_pitch", "<i8"), ("b_pitch
 assert RUN_TILE.itemsize == 24 and ROW_TILE.itemsize == 64 and TRANS_TILE.itemsize == 48
 
 
+class Segment(ctypes.Structure):
+    """EthaSegment: one chunk range of one table, run as the entry point named by ``kind`` would."""
+
+    _fields_ = [("table", c_void_p), ("kind", c_uint32), ("first", c_uint32), ("count", c_uint32), ("reserved", c_uint32)]
+
+
 class TableInfo(ctypes.Structure):
     _fields_ = [
         ("n_chunks", c_uint32),
@@ -112,6 +120,8 @@ _SIGNATURES = {
     "etha_unpack_bucket": (c_int, [c_void_p, c_uint32, c_uint32, c_void_p, c_uint32]),
     "etha_reduce_pack_bucket": (c_int, [c_void_p, c_uint32, c_uint32, c_void_p, c_uint32]),
     "etha_selfcopy_bucket": (c_int, [c_void_p, c_uint32, c_uint32, c_void_p, c_uint32]),
+    "etha_launch_segments": (c_int, [c_void_p, c_uint32, c_void_p, c_uint32]),
+    "etha_kernel_launches": (c_uint64, []),
     "etha_noalloc_setup": (c_int, []),
     "etha_copy_regions_noalloc": (c_int, [c_void_p, c_void_p, c_uint32, c_void_p]),
     "etha_arena_create": (c_int, [c_uint64, POINTER(c_void_p)]),
@@ -320,6 +330,20 @@ def ipc_export(ptr: int) -> bytes:
     h = IpcHandle()
     _check("etha_ipc_export", lib().etha_ipc_export(c_void_p(ptr), byref(h)))
     return bytes(h)
+
+
+def kernel_launches() -> int:
+    """Kernels launched through the library by this process so far."""
+    return int(lib().etha_kernel_launches())
+
+
+def launch_segments(segments, stream: int = 0, flags: int = 0) -> None:
+    """Issue ``segments`` - ``(table, kind, first, count)`` with ``kind`` one of ``SEG_*`` - as one set of launches
+    that do not depend on each other (``etha_launch_segments``)."""
+    arr = (Segment * max(len(segments), 1))()
+    for i, (table, kind, first, count) in enumerate(segments):
+        arr[i].table, arr[i].kind, arr[i].first, arr[i].count = table._h, kind, first, count
+    _check("etha_launch_segments", lib().etha_launch_segments(arr, len(segments), c_void_p(stream), flags))
 
 
 def ipc_open(handle_bytes: bytes) -> int:

@@ -288,6 +288,18 @@ class TransferPlan:
         elif kind in (_SELF, _SELF_REDUCE, _DIRECT, _DIRECT_REDUCE):
             self.local_table.selfcopy(first, count, stream, flags)
 
+    def segment(self, kind: str, first: int, count: int) -> tuple:
+        """The same launch as an entry of a set for ``_native.launch_segments``."""
+        from .. import _native as nat
+
+        if kind == _PACK:
+            return (self.send_table, nat.SEG_PACK, first, count)
+        if kind == _REDUCE:
+            return (self.send_table, nat.SEG_REDUCE_PACK, first, count)
+        if kind == _UNPACK:
+            return (self.recv_table, nat.SEG_UNPACK, first, count)
+        return (self.local_table, nat.SEG_SELFCOPY, first, count)
+
     # ---- resident pool: the bucket list in list order -------------------------------------------------
     def run(self, stream: int | None = None, merge_launches: bool = False, fanout: int = 1) -> None:
         """Enqueue this bucket list's launches in list order (resident pool only: with a ring the list's

@@ -136,6 +136,11 @@ class LoopbackWire:
         # launches that do not depend on each other are issued without ordering between them
         # (ETHA_LAUNCH_UNORDERED), which hides the gap between one bucket's kernel and the next one's
         self.unordered_launches = True
+        # launches that do not depend on each other are handed to the library as one set (etha_launch_segments):
+        # what a sweep over all pipelines prepares and finalizes shares kernel launches
+        self.group_launches = True
+        self._group: list = []  # (plan, kind, first, count) of the set being collected
+        self._group_flags = 0
         # host inspection: called as ``on_launch(plan, kind, first, count, flags)`` instead of launching
         self.on_launch = None
         self.launch_log: list | None = None  # when a list: (kind, first, count, flags) of every launch
@@ -396,14 +401,17 @@ class LoopbackWire:
         self._ordered_next = True
         self._epoch_reads, self._epoch_writes = set(), set()
         with torch.cuda.device(self.device) if cuda else _no_context():
-            moved = True
-            while moved:
-                moved = False
-                for program in list(self._programs):
-                    if program.sweep(self):
-                        moved = True
-                    if program.finished:
-                        self._programs.remove(program)
+            try:
+                moved = True
+                while moved:
+                    moved = False
+                    for program in list(self._programs):
+                        if program.sweep(self):
+                            moved = True
+                        if program.finished:
+                            self._programs.remove(program)
+            finally:
+                self._flush()  # what was issued is marked as sent / received: it must reach the stream
         self._carried = bool(self._programs)
 
     def idle(self) -> bool:
@@ -468,7 +476,31 @@ class LoopbackWire:
             return
         if plan.device is None or plan.device.type != "cuda":
             raise RuntimeError("this plan was compiled for host inspection; the executor only runs on a GPU (there is no CPU path)")
-        plan.launch_step(kind, first, count, self._stream.cuda_stream, flags)
+        if not self.group_launches:
+            plan.launch_step(kind, first, count, self._stream.cuda_stream, flags)
+            return
+        # an ordered launch closes the set before it and opens the next one; an unordered launch depends on
+        # nothing since the last ordered one, members of the open set included, so it joins the set
+        if ordered:
+            self._flush()
+            self._group_flags = 0
+        elif not self._group:
+            self._group_flags = nat.LAUNCH_UNORDERED
+        self._group.append((plan, kind, first, count))
+
+    def _flush(self) -> None:
+        """Hand the collected set of independent launches to the library."""
+        if not self._group:
+            return
+        from .. import _native as nat
+
+        group, self._group = self._group, []
+        if len(group) == 1:
+            plan, kind, first, count = group[0]
+            plan.launch_step(kind, first, count, self._stream.cuda_stream, self._group_flags)
+            return
+        nat.launch_segments([plan.segment(kind, first, count) for plan, kind, first, count in group],
+                            self._stream.cuda_stream, self._group_flags)
 
 
 _default_wire: LoopbackWire | None = None

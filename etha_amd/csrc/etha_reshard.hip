@@ -19,6 +19,7 @@
 #include <cstdio>
 #include <algorithm>
 #include <array>
+#include <atomic>
 #include <cstring>
 #include <map>
 #include <mutex>
@@ -411,11 +412,9 @@ __device__ __forceinline__ void row_position(const RowTile& t, uint32_t tid, uin
 
 // pack (REV = false): a -> b.   unpack (REV = true): b -> a.
 template <bool REV>
-__global__ __launch_bounds__(ETHA_BLOCK_THREADS) void etha_tile_kernel(const RunTile* __restrict__ run_tiles, uint32_t n_run,
-                                                                        const RowTile* __restrict__ row_tiles,
-                                                                        const uint64_t* __restrict__ gather) {
-  const uint32_t bid = blockIdx.x / kBlocksPerTile;
-  const uint32_t tid = (blockIdx.x % kBlocksPerTile) * kBlockThreads + threadIdx.x;
+__device__ __forceinline__ void tile_body(const RunTile* __restrict__ run_tiles, uint32_t n_run,
+                                          const RowTile* __restrict__ row_tiles, const uint64_t* __restrict__ gather,
+                                          uint32_t bid, uint32_t tid) {
   uint64_t a, b;
   uint32_t n, meta;
   if (bid < n_run) {
@@ -452,6 +451,45 @@ __global__ __launch_bounds__(ETHA_BLOCK_THREADS) void etha_tile_kernel(const Run
   }
   if (tid >= n) return;
   move_unit<REV>(meta, a, b);
+}
+
+template <bool REV>
+__global__ __launch_bounds__(ETHA_BLOCK_THREADS) void etha_tile_kernel(const RunTile* __restrict__ run_tiles, uint32_t n_run,
+                                                                        const RowTile* __restrict__ row_tiles,
+                                                                        const uint64_t* __restrict__ gather) {
+  tile_body<REV>(run_tiles, n_run, row_tiles, gather, blockIdx.x / kBlocksPerTile,
+                 (blockIdx.x % kBlocksPerTile) * kBlockThreads + threadIdx.x);
+}
+
+// Several chunk ranges of one direction in one launch: blockIdx.y picks the range, blockIdx.x walks its tiles
+// (workgroups past the end of a shorter range leave at once).  The ranges run one after the other in dispatch
+// order, as their own launches would, without the gap between launches.
+struct alignas(32) Seg2D {
+  const RunTile* run;
+  const RowTile* row;
+  const uint64_t* gather;
+  uint32_t n_run;
+  uint32_t n_tiles;
+};
+struct Args2D {
+  Seg2D seg[ETHA_MAX_SEGMENTS];
+};
+
+template <bool REV>
+__global__ __launch_bounds__(ETHA_BLOCK_THREADS) void etha_tile_kernel_2d(const Args2D args) {
+  typedef uint32_t u32x8 __attribute__((ext_vector_type(8)));
+  const u32x8 raw = *reinterpret_cast<const u32x8*>(&args.seg[blockIdx.y]);  // the whole entry in one scalar load
+  const uint32_t bid = blockIdx.x / kBlocksPerTile;
+  if (bid >= raw[7]) return;
+  // (pointers rebuilt from integers must be told that they point to device memory, or they are dereferenced
+  // with per-lane generic loads instead of scalar loads: measured 7 % slower)
+  typedef const __attribute__((address_space(1))) RunTile* GlobalRun;
+  typedef const __attribute__((address_space(1))) RowTile* GlobalRow;
+  typedef const __attribute__((address_space(1))) uint64_t* GlobalU64;
+  const RunTile* run = (const RunTile*)(GlobalRun)(((uint64_t)raw[1] << 32) | raw[0]);
+  const RowTile* row = (const RowTile*)(GlobalRow)(((uint64_t)raw[3] << 32) | raw[2]);
+  const uint64_t* gather = (const uint64_t*)(GlobalU64)(((uint64_t)raw[5] << 32) | raw[4]);
+  tile_body<REV>(run, raw[6], row, gather, bid, (blockIdx.x % kBlocksPerTile) * kBlockThreads + threadIdx.x);
 }
 
 // ---- transposing chunks: staged through LDS -----------------------------------------------------
@@ -1337,8 +1375,11 @@ int check_range(const EthaTable* t, uint32_t first, uint32_t count, int kind) {
 // clears that wait for this one dispatch: the kernel may start while earlier launches are still running,
 // which removes the drain/ramp bubble between launches that do not depend on each other.  The next
 // ordinary launch on the stream again waits for everything before it, unordered launches included.
+std::atomic<uint64_t> g_kernel_launches{0};
+
 template <typename... Args, typename F>
 void launch_kernel(F kernel, dim3 grid, dim3 block, size_t lds, void* stream, uint32_t flags, Args... args) {
+  g_kernel_launches.fetch_add(1, std::memory_order_relaxed);
   if (flags & ETHA_LAUNCH_UNORDERED)
     hipExtLaunchKernelGGL(kernel, grid, block, (uint32_t)lds, (hipStream_t)stream, nullptr, nullptr, hipExtAnyOrderLaunch,
                           args...);
@@ -1346,36 +1387,85 @@ void launch_kernel(F kernel, dim3 grid, dim3 block, size_t lds, void* stream, ui
     hipLaunchKernelGGL(kernel, grid, block, lds, (hipStream_t)stream, args...);
 }
 
+// the plain (run and row) tiles of a chunk range, as the tile kernels take them
+Seg2D tile_range(const EthaTable* t, uint32_t first, uint32_t count, bool rev) {
+  const uint32_t r0 = t->run_begin[first], w0 = t->row_begin[first];
+  Seg2D g{t->d_run + r0, t->d_row + w0, nullptr, t->run_begin[first + count] - r0, 0};
+  g.n_tiles = g.n_run + (t->row_begin[first + count] - w0);
+  if (rev == (t->kind == 0)) {  // the direction that writes the a side (unpack) / b side (self-copy) of an ordered range
+    auto it = t->ordered.find(std::make_pair(first, count));
+    if (it != t->ordered.end()) {
+      g.run = it->second.d_run;
+      g.row = it->second.d_row;
+      g.gather = it->second.d_gather;
+      g.n_run = (uint32_t)it->second.h_run.size();  // gathering regroups row tiles: their number may differ
+      g.n_tiles = g.n_run + (uint32_t)it->second.h_row.size();
+    }
+  }
+  return g;
+}
+
+// transposing chunks run in their own kernel (it needs LDS); true when one was launched
+bool launch_trans(const EthaTable* t, uint32_t first, uint32_t count, bool rev, void* stream, uint32_t flags) {
+  const uint32_t x0 = t->trans_begin[first], n_trans = t->trans_begin[first + count] - x0;
+  if (!n_trans) return false;
+  if (rev)
+    launch_kernel(etha_transpose_kernel<true>, dim3(n_trans), dim3(kTransThreads), t->trans_lds, stream, flags,
+                  (const TransTile*)(t->d_trans + x0));
+  else
+    launch_kernel(etha_transpose_kernel<false>, dim3(n_trans), dim3(kTransThreads), t->trans_lds, stream, flags,
+                  (const TransTile*)(t->d_trans + x0));
+  return true;
+}
+
+void launch_plain(const Seg2D& g, bool rev, void* stream, uint32_t flags) {
+  if (rev)
+    launch_kernel(etha_tile_kernel<true>, dim3(g.n_tiles * kBlocksPerTile), dim3(kBlockThreads), 0, stream, flags, g.run, g.n_run,
+                  g.row, g.gather);
+  else
+    launch_kernel(etha_tile_kernel<false>, dim3(g.n_tiles * kBlocksPerTile), dim3(kBlockThreads), 0, stream, flags, g.run, g.n_run,
+                  g.row, g.gather);
+}
+
 template <bool REV>
 int launch_tiles(const EthaTable* t, uint32_t first, uint32_t count, void* stream, uint32_t flags) {
-  const uint32_t r0 = t->run_begin[first], r1 = t->run_begin[first + count];
-  const uint32_t w0 = t->row_begin[first], w1 = t->row_begin[first + count];
-  uint32_t n_run = r1 - r0, n_row = w1 - w0;
-  const uint32_t x0 = t->trans_begin[first], n_trans = t->trans_begin[first + count] - x0;
-  if (n_trans) {  // transposing chunks run in their own kernel (it needs LDS)
-    launch_kernel(etha_transpose_kernel<REV>, dim3(n_trans), dim3(kTransThreads), t->trans_lds, stream, flags,
-                  (const TransTile*)(t->d_trans + x0));
+  if (launch_trans(t, first, count, REV, stream, flags)) {
     HIP_TRY(hipGetLastError());
     flags |= ETHA_LAUNCH_UNORDERED;  // the two kernels of one call touch different chunks
   }
-  if (n_run + n_row == 0) return ETHA_OK;
-  const RunTile* d_run = t->d_run + r0;
-  const RowTile* d_row = t->d_row + w0;
-  const uint64_t* d_gather = nullptr;
-  if (REV == (t->kind == 0)) {  // the direction that writes the a side (unpack) / b side (self-copy) of an ordered range
-    auto it = t->ordered.find(std::make_pair(first, count));
-    if (it != t->ordered.end()) {
-      d_run = it->second.d_run;
-      d_row = it->second.d_row;
-      d_gather = it->second.d_gather;
-      n_run = (uint32_t)it->second.h_run.size();  // gathering regroups row tiles: their number may differ
-      n_row = (uint32_t)it->second.h_row.size();
-    }
-  }
-  launch_kernel(etha_tile_kernel<REV>, dim3((n_run + n_row) * kBlocksPerTile), dim3(kBlockThreads), 0, stream, flags, d_run,
-                n_run, d_row, d_gather);
+  const Seg2D g = tile_range(t, first, count, REV);
+  if (g.n_tiles == 0) return ETHA_OK;
+  launch_plain(g, REV, stream, flags);
   HIP_TRY(hipGetLastError());
   return ETHA_OK;
+}
+
+// Plain-tile segments of one direction: those of similar size share a launch (the workgroups a shorter
+// segment leaves unused still cost a dispatch slot each, about 0.2 ns; a launch of its own costs about
+// 1.8 us, i.e. some 8000 workgroups).
+constexpr uint32_t kGroupSlackTiles = 8192 / kBlocksPerTile;
+
+void launch_group(std::vector<Seg2D>& segs, bool rev, void* stream, uint32_t& flags) {
+  std::stable_sort(segs.begin(), segs.end(), [](const Seg2D& x, const Seg2D& y) { return x.n_tiles > y.n_tiles; });
+  size_t i = 0;
+  while (i < segs.size()) {
+    size_t j = i + 1;
+    while (j < segs.size() && j - i < ETHA_MAX_SEGMENTS && segs[i].n_tiles - segs[j].n_tiles <= kGroupSlackTiles) j++;
+    if (j - i == 1) {
+      launch_plain(segs[i], rev, stream, flags);
+    } else {
+      Args2D args;
+      memset(&args, 0, sizeof(args));
+      for (size_t k = i; k < j; k++) args.seg[k - i] = segs[k];
+      const dim3 grid(segs[i].n_tiles * kBlocksPerTile, (uint32_t)(j - i));
+      if (rev)
+        launch_kernel(etha_tile_kernel_2d<true>, grid, dim3(kBlockThreads), 0, stream, flags, args);
+      else
+        launch_kernel(etha_tile_kernel_2d<false>, grid, dim3(kBlockThreads), 0, stream, flags, args);
+    }
+    flags |= ETHA_LAUNCH_UNORDERED;  // what follows belongs to the same set of independent segments
+    i = j;
+  }
 }
 
 int launch_reduce(const EthaTable* t, uint32_t first, uint32_t count, void* stream, uint32_t flags) {
@@ -1455,6 +1545,7 @@ extern "C" {
 #define ETHA_SOURCE_HASH "unknown"
 #endif
 int etha_abi_version(void) { return ETHA_ABI_VERSION; }
+uint64_t etha_kernel_launches(void) { return g_kernel_launches.load(std::memory_order_relaxed); }
 // the marker lets a build script find the digest in the file without loading the library
 static const char kSourceDigest[] = "etha-source-digest:" ETHA_SOURCE_HASH;
 const char* etha_source_hash(void) { return kSourceDigest + sizeof("etha-source-digest:") - 1; }
@@ -1752,6 +1843,48 @@ int etha_selfcopy_bucket(const EthaTable* t, uint32_t first, uint32_t count, voi
   if (n_reduce == 0) return launch_tiles<false>(t, first, count, stream, flags);
   if (n_reduce != count) return fail(ETHA_ERR_INVALID, "range mixes Partial and plain chunks; launch them separately");
   return launch_reduce(t, first, count, stream, flags);
+}
+
+int etha_launch_segments(const EthaSegment* segs, uint32_t n_segments, void* stream, uint32_t flags) {
+  int rc = check_flags(flags);
+  if (rc != ETHA_OK) return rc;
+  if (n_segments == 0) return ETHA_OK;
+  if (!segs) return fail(ETHA_ERR_INVALID, "null segment list");
+  for (uint32_t i = 0; i < n_segments; i++) {  // validate everything before the first launch
+    const EthaSegment& g = segs[i];
+    if (g.kind > ETHA_SEG_SELFCOPY) return fail(ETHA_ERR_INVALID, "segment %u: unknown kind %u", i, g.kind);
+    rc = check_range(g.table, g.first, g.count, g.kind == ETHA_SEG_SELFCOPY ? 1 : 0);
+    if (rc != ETHA_OK) return rc;
+    const uint32_t n_reduce = g.table->reduce_prefix[g.first + g.count] - g.table->reduce_prefix[g.first];
+    if ((g.kind == ETHA_SEG_PACK || g.kind == ETHA_SEG_UNPACK) && n_reduce)
+      return fail(ETHA_ERR_INVALID, "segment %u: range holds Partial chunks", i);
+    if (g.kind == ETHA_SEG_REDUCE_PACK && n_reduce != g.count)
+      return fail(ETHA_ERR_INVALID, "segment %u: range holds chunks that are not Partial chunks", i);
+    if (g.kind == ETHA_SEG_SELFCOPY && n_reduce && n_reduce != g.count)
+      return fail(ETHA_ERR_INVALID, "segment %u: range mixes Partial and plain chunks; launch them separately", i);
+  }
+  std::vector<Seg2D> forward, reverse;
+  for (uint32_t i = 0; i < n_segments; i++) {
+    const EthaSegment& g = segs[i];
+    const EthaTable* t = g.table;
+    if (t->reduce_prefix[g.first + g.count] != t->reduce_prefix[g.first]) {
+      const uint32_t w0 = t->row_begin[g.first], w1 = t->row_begin[g.first + g.count];
+      if (w1 != w0) {
+        launch_kernel(etha_reduce_kernel, dim3((w1 - w0) * kBlocksPerTile), dim3(kBlockThreads), 0, stream, flags,
+                      (const RowTile*)(t->d_row + w0), (const uint64_t*)t->d_peers);
+        flags |= ETHA_LAUNCH_UNORDERED;
+      }
+      continue;
+    }
+    const bool rev = g.kind == ETHA_SEG_UNPACK;
+    if (launch_trans(t, g.first, g.count, rev, stream, flags)) flags |= ETHA_LAUNCH_UNORDERED;
+    const Seg2D r = tile_range(t, g.first, g.count, rev);
+    if (r.n_tiles) (rev ? reverse : forward).push_back(r);
+  }
+  launch_group(forward, false, stream, flags);
+  launch_group(reverse, true, stream, flags);
+  HIP_TRY(hipGetLastError());
+  return ETHA_OK;
 }
 
 // ---- region copies for callers that cannot allocate --------------------------------------------

@@ -31,7 +31,7 @@
 extern "C" {
 #endif
 
-#define ETHA_ABI_VERSION 4
+#define ETHA_ABI_VERSION 5
 #define ETHA_MAX_NDIM 8
 
 /* status codes */
@@ -136,6 +136,9 @@ const char* etha_last_error(void);
 /* digest of the sources (kernel file + this header) the library was built from, as the build recipe passed it;
  * lets a harness notice a library that is older than the tree.  No counterpart in the reference. */
 const char* etha_source_hash(void);
+/* kernels this process has launched through the library so far (one call may launch several); for benchmarks
+ * that report time per launch.  No counterpart in the reference. */
+uint64_t etha_kernel_launches(void);
 
 /*
  * Compile chunk descriptors into a tile program.
@@ -225,6 +228,32 @@ int etha_reduce_pack_bucket(const EthaTable* table, uint32_t first, uint32_t cou
 
 /* Run chunks [first, first+count) of a self-copy or direct table.  One kernel launch. */
 int etha_selfcopy_bucket(const EthaTable* table, uint32_t first, uint32_t count, void* stream, uint32_t flags);
+
+/*
+ * Several bucket launches that do not depend on each other, issued as one unit: what one sweep of the
+ * reference's bucket_comm loop prepares and finalizes over all its channels (comm_methods.py:85-116) -
+ * packs of the next candidates, unpacks of the arrived buckets, same-rank copies - in as few kernel
+ * launches as possible.  Segment i runs chunks [first, first+count) of its table as the entry point named
+ * by kind would (ETHA_SEG_PACK = etha_pack_bucket, ...).  No byte written by one segment may be read or
+ * written by another: the segments run concurrently.  flags apply to the set as a whole (with
+ * ETHA_LAUNCH_UNORDERED the whole set is unordered against earlier launches of the stream).  Segments of one
+ * direction and of similar size share a launch (up to ETHA_MAX_SEGMENTS each; the segment is picked by the
+ * workgroup's second grid index); transposing and reduce tiles keep their own kernels.  Saves the cost of a
+ * launch (about 1.8 us) per segment that joins another's launch.  No counterpart in the reference, whose
+ * buckets are many small ATen launches each.
+ */
+#define ETHA_SEG_PACK 0u
+#define ETHA_SEG_UNPACK 1u
+#define ETHA_SEG_REDUCE_PACK 2u
+#define ETHA_SEG_SELFCOPY 3u
+#define ETHA_MAX_SEGMENTS 16u
+typedef struct EthaSegment {
+  const EthaTable* table;
+  uint32_t kind; /* ETHA_SEG_* */
+  uint32_t first, count;
+  uint32_t reserved; /* 0 */
+} EthaSegment;
+int etha_launch_segments(const EthaSegment* segments, uint32_t n_segments, void* stream, uint32_t flags);
 
 /*
  * Region copies for callers that cannot allocate device memory (code under HIP graph capture, tight serving
