@@ -604,6 +604,32 @@ __global__ __launch_bounds__(ETHA_TRANS_THREADS) void etha_transpose_kernel(cons
   }
 }
 
+// several tables' transposing tiles in one launch: blockIdx.y picks the list, as in etha_tile_kernel_2d
+struct alignas(16) TransSeg {
+  const TransTile* tiles;
+  uint32_t n;
+  uint32_t reserved;
+};
+struct TransArgs {
+  TransSeg seg[ETHA_MAX_SEGMENTS];
+};
+
+template <bool REV>
+__global__ __launch_bounds__(ETHA_TRANS_THREADS) void etha_transpose_kernel_2d(const TransArgs args) {
+  extern __shared__ __attribute__((aligned(16))) uint8_t lds_bytes[];
+  const u32x4 raw = *reinterpret_cast<const u32x4*>(&args.seg[blockIdx.y]);
+  if (blockIdx.x >= raw[2]) return;  // the whole workgroup leaves: no barrier is skipped by part of it
+  typedef const __attribute__((address_space(1))) TransTile* GlobalTrans;
+  const TransTile* tiles = (const TransTile*)(GlobalTrans)(((uint64_t)raw[1] << 32) | raw[0]);
+  const TransTile t = tiles[blockIdx.x];
+  switch (t.es_log2) {
+    case 0: transpose_block<uint8_t, REV>(t, lds_bytes); break;
+    case 1: transpose_block<uint16_t, REV>(t, lds_bytes); break;
+    case 2: transpose_block<uint32_t, REV>(t, lds_bytes); break;
+    default: transpose_block<uint64_t, REV>(t, lds_bytes); break;
+  }
+}
+
 // ---- Partial reduce-pack ------------------------------------------------------------------------
 template <typename ACC>
 __device__ __forceinline__ ACC combine(uint32_t op, ACC x, ACC y) {
@@ -1845,6 +1871,35 @@ int etha_selfcopy_bucket(const EthaTable* t, uint32_t first, uint32_t count, voi
   return launch_reduce(t, first, count, stream, flags);
 }
 
+// the same for transposing tiles (one workgroup of kTransThreads work-items per tile)
+constexpr uint32_t kTransGroupSlackTiles = 64;
+
+void launch_trans_group(std::vector<TransSeg>& segs, bool rev, uint32_t lds, void* stream, uint32_t& flags) {
+  std::stable_sort(segs.begin(), segs.end(), [](const TransSeg& x, const TransSeg& y) { return x.n > y.n; });
+  size_t i = 0;
+  while (i < segs.size()) {
+    size_t j = i + 1;
+    while (j < segs.size() && j - i < ETHA_MAX_SEGMENTS && segs[i].n - segs[j].n <= kTransGroupSlackTiles) j++;
+    if (j - i == 1) {
+      if (rev)
+        launch_kernel(etha_transpose_kernel<true>, dim3(segs[i].n), dim3(kTransThreads), lds, stream, flags, segs[i].tiles);
+      else
+        launch_kernel(etha_transpose_kernel<false>, dim3(segs[i].n), dim3(kTransThreads), lds, stream, flags, segs[i].tiles);
+    } else {
+      TransArgs args;
+      memset(&args, 0, sizeof(args));
+      for (size_t k = i; k < j; k++) args.seg[k - i] = segs[k];
+      const dim3 grid(segs[i].n, (uint32_t)(j - i));
+      if (rev)
+        launch_kernel(etha_transpose_kernel_2d<true>, grid, dim3(kTransThreads), lds, stream, flags, args);
+      else
+        launch_kernel(etha_transpose_kernel_2d<false>, grid, dim3(kTransThreads), lds, stream, flags, args);
+    }
+    flags |= ETHA_LAUNCH_UNORDERED;
+    i = j;
+  }
+}
+
 int etha_launch_segments(const EthaSegment* segs, uint32_t n_segments, void* stream, uint32_t flags) {
   int rc = check_flags(flags);
   if (rc != ETHA_OK) return rc;
@@ -1864,6 +1919,8 @@ int etha_launch_segments(const EthaSegment* segs, uint32_t n_segments, void* str
       return fail(ETHA_ERR_INVALID, "segment %u: range mixes Partial and plain chunks; launch them separately", i);
   }
   std::vector<Seg2D> forward, reverse;
+  std::vector<TransSeg> trans_forward, trans_reverse;
+  uint32_t trans_lds = 0;
   for (uint32_t i = 0; i < n_segments; i++) {
     const EthaSegment& g = segs[i];
     const EthaTable* t = g.table;
@@ -1877,10 +1934,16 @@ int etha_launch_segments(const EthaSegment* segs, uint32_t n_segments, void* str
       continue;
     }
     const bool rev = g.kind == ETHA_SEG_UNPACK;
-    if (launch_trans(t, g.first, g.count, rev, stream, flags)) flags |= ETHA_LAUNCH_UNORDERED;
+    const uint32_t x0 = t->trans_begin[g.first], n_trans = t->trans_begin[g.first + g.count] - x0;
+    if (n_trans) {
+      (rev ? trans_reverse : trans_forward).push_back(TransSeg{t->d_trans + x0, n_trans, 0});
+      if (t->trans_lds > trans_lds) trans_lds = t->trans_lds;
+    }
     const Seg2D r = tile_range(t, g.first, g.count, rev);
     if (r.n_tiles) (rev ? reverse : forward).push_back(r);
   }
+  launch_trans_group(trans_forward, false, trans_lds, stream, flags);
+  launch_trans_group(trans_reverse, true, trans_lds, stream, flags);
   launch_group(forward, false, stream, flags);
   launch_group(reverse, true, stream, flags);
   HIP_TRY(hipGetLastError());
