@@ -234,12 +234,16 @@ def time_steps(job, steps, run):
         for k in range(steps):
             run()
             ev[k + 1].record(stream)
+        HOST_MS["issue"] = (time.perf_counter() - wall0) * 1e3 / steps  # the host's share: planning sweeps + launch calls
         torch.cuda.synchronize()
         wall = time.perf_counter() - wall0
     finally:
         gc.enable()
     dev = [ev[k].elapsed_time(ev[k + 1]) for k in range(steps)]
     return sum(dev) / steps, wall * 1e3 / steps
+
+
+HOST_MS: dict = {}
 
 
 def launches_per_step(job, run):
@@ -303,6 +307,7 @@ def main():
         graph.replay()
     step = graph.replay if graph is not None else (lambda: job.run(merge_launches=merge, fanout=args.fanout, synchronize=False))
     dev_ms, step_ms = time_steps(job, args.steps, step)
+    host_ms = HOST_MS.get("issue")
     n_launch, n_steps, n_unordered = launches_per_step(
         job, lambda: job.run(merge_launches=merge, fanout=args.fanout, synchronize=False))
     if args.pool != "ring":
@@ -356,6 +361,7 @@ def main():
             **job.counts(),
         },
         "device_ms_per_step": round(dev_ms, 4),
+        "host_issue_ms_per_step": round(host_ms, 4),
         "pct_of_hbm_peak": round(100.0 * achieved / HBM_PEAK_GBS, 2),
         "algorithmic_bytes_per_step": {"pack": pack_bytes, "unpack": unpack_bytes, "of_which_self_copy": self_bytes},
         "launches_per_step": n_launch,

@@ -1466,32 +1466,74 @@ int launch_tiles(const EthaTable* t, uint32_t first, uint32_t count, void* strea
   return ETHA_OK;
 }
 
-// Plain-tile segments of one direction: those of similar size share a launch (the workgroups a shorter
-// segment leaves unused still cost a dispatch slot each, about 0.2 ns; a launch of its own costs about
-// 1.8 us, i.e. some 8000 workgroups).
-constexpr uint32_t kGroupSlackTiles = 8192 / kBlocksPerTile;
+// Segments of one direction, largest first: those of (nearly) the same size share a launch.  A workgroup that a
+// shorter segment leaves unused is not free - with no limit on them the config-2 step took 6.0 instead of 4.9 ms -
+// while a launch of its own costs about 1.8 us: a segment joins the open launch only while the unused
+// workgroups it adds stay below a few thousand.  Equal-sized buckets, the usual case, add none.
+constexpr uint64_t kJoinMaxIdleTiles = 6000 / kBlocksPerTile;
 
-void launch_group(std::vector<Seg2D>& segs, bool rev, void* stream, uint32_t& flags) {
-  std::stable_sort(segs.begin(), segs.end(), [](const Seg2D& x, const Seg2D& y) { return x.n_tiles > y.n_tiles; });
+template <typename SEG, typename COUNT, typename LAUNCH>
+void launch_neighbours(std::vector<SEG>& segs, uint64_t max_idle, COUNT count_of, LAUNCH launch, uint32_t& flags) {
+  std::stable_sort(segs.begin(), segs.end(), [&](const SEG& x, const SEG& y) { return count_of(x) > count_of(y); });
   size_t i = 0;
   while (i < segs.size()) {
+    uint64_t top = count_of(segs[i]), sum = top;
     size_t j = i + 1;
-    while (j < segs.size() && j - i < ETHA_MAX_SEGMENTS && segs[i].n_tiles - segs[j].n_tiles <= kGroupSlackTiles) j++;
-    if (j - i == 1) {
-      launch_plain(segs[i], rev, stream, flags);
-    } else {
-      Args2D args;
-      memset(&args, 0, sizeof(args));
-      for (size_t k = i; k < j; k++) args.seg[k - i] = segs[k];
-      const dim3 grid(segs[i].n_tiles * kBlocksPerTile, (uint32_t)(j - i));
-      if (rev)
-        launch_kernel(etha_tile_kernel_2d<true>, grid, dim3(kBlockThreads), 0, stream, flags, args);
-      else
-        launch_kernel(etha_tile_kernel_2d<false>, grid, dim3(kBlockThreads), 0, stream, flags, args);
+    while (j < segs.size() && j - i < ETHA_MAX_SEGMENTS) {
+      const uint64_t n = count_of(segs[j]), new_top = n > top ? n : top;
+      const uint64_t idle_now = top * (j - i) - sum, idle_then = new_top * (j - i + 1) - (sum + n);
+      if (idle_then - idle_now > max_idle) break;
+      top = new_top;
+      sum += n;
+      j++;
     }
+    launch(i, j, (uint32_t)top, flags);
     flags |= ETHA_LAUNCH_UNORDERED;  // what follows belongs to the same set of independent segments
     i = j;
   }
+}
+
+void launch_group(std::vector<Seg2D>& segs, bool rev, void* stream, uint32_t& flags) {
+  launch_neighbours(
+      segs, kJoinMaxIdleTiles, [](const Seg2D& g) { return (uint64_t)g.n_tiles; },
+      [&](size_t i, size_t j, uint32_t top, uint32_t fl) {
+        if (j - i == 1) return launch_plain(segs[i], rev, stream, fl);
+        Args2D args;
+        memset(&args, 0, sizeof(args));
+        for (size_t k = i; k < j; k++) args.seg[k - i] = segs[k];
+        const dim3 grid(top * kBlocksPerTile, (uint32_t)(j - i));
+        if (rev)
+          launch_kernel(etha_tile_kernel_2d<true>, grid, dim3(kBlockThreads), 0, stream, fl, args);
+        else
+          launch_kernel(etha_tile_kernel_2d<false>, grid, dim3(kBlockThreads), 0, stream, fl, args);
+      },
+      flags);
+}
+
+// the same for transposing tiles (one workgroup of kTransThreads work-items per tile)
+constexpr uint64_t kTransJoinMaxIdleTiles = 64;
+
+void launch_trans_group(std::vector<TransSeg>& segs, bool rev, uint32_t lds, void* stream, uint32_t& flags) {
+  launch_neighbours(
+      segs, kTransJoinMaxIdleTiles, [](const TransSeg& g) { return (uint64_t)g.n; },
+      [&](size_t i, size_t j, uint32_t top, uint32_t fl) {
+        if (j - i == 1) {
+          if (rev)
+            launch_kernel(etha_transpose_kernel<true>, dim3(segs[i].n), dim3(kTransThreads), lds, stream, fl, segs[i].tiles);
+          else
+            launch_kernel(etha_transpose_kernel<false>, dim3(segs[i].n), dim3(kTransThreads), lds, stream, fl, segs[i].tiles);
+          return;
+        }
+        TransArgs args;
+        memset(&args, 0, sizeof(args));
+        for (size_t k = i; k < j; k++) args.seg[k - i] = segs[k];
+        const dim3 grid(top, (uint32_t)(j - i));
+        if (rev)
+          launch_kernel(etha_transpose_kernel_2d<true>, grid, dim3(kTransThreads), lds, stream, fl, args);
+        else
+          launch_kernel(etha_transpose_kernel_2d<false>, grid, dim3(kTransThreads), lds, stream, fl, args);
+      },
+      flags);
 }
 
 int launch_reduce(const EthaTable* t, uint32_t first, uint32_t count, void* stream, uint32_t flags) {
@@ -1869,35 +1911,6 @@ int etha_selfcopy_bucket(const EthaTable* t, uint32_t first, uint32_t count, voi
   if (n_reduce == 0) return launch_tiles<false>(t, first, count, stream, flags);
   if (n_reduce != count) return fail(ETHA_ERR_INVALID, "range mixes Partial and plain chunks; launch them separately");
   return launch_reduce(t, first, count, stream, flags);
-}
-
-// the same for transposing tiles (one workgroup of kTransThreads work-items per tile)
-constexpr uint32_t kTransGroupSlackTiles = 64;
-
-void launch_trans_group(std::vector<TransSeg>& segs, bool rev, uint32_t lds, void* stream, uint32_t& flags) {
-  std::stable_sort(segs.begin(), segs.end(), [](const TransSeg& x, const TransSeg& y) { return x.n > y.n; });
-  size_t i = 0;
-  while (i < segs.size()) {
-    size_t j = i + 1;
-    while (j < segs.size() && j - i < ETHA_MAX_SEGMENTS && segs[i].n - segs[j].n <= kTransGroupSlackTiles) j++;
-    if (j - i == 1) {
-      if (rev)
-        launch_kernel(etha_transpose_kernel<true>, dim3(segs[i].n), dim3(kTransThreads), lds, stream, flags, segs[i].tiles);
-      else
-        launch_kernel(etha_transpose_kernel<false>, dim3(segs[i].n), dim3(kTransThreads), lds, stream, flags, segs[i].tiles);
-    } else {
-      TransArgs args;
-      memset(&args, 0, sizeof(args));
-      for (size_t k = i; k < j; k++) args.seg[k - i] = segs[k];
-      const dim3 grid(segs[i].n, (uint32_t)(j - i));
-      if (rev)
-        launch_kernel(etha_transpose_kernel_2d<true>, grid, dim3(kTransThreads), lds, stream, flags, args);
-      else
-        launch_kernel(etha_transpose_kernel_2d<false>, grid, dim3(kTransThreads), lds, stream, flags, args);
-    }
-    flags |= ETHA_LAUNCH_UNORDERED;
-    i = j;
-  }
 }
 
 int etha_launch_segments(const EthaSegment* segs, uint32_t n_segments, void* stream, uint32_t flags) {
