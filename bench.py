@@ -35,6 +35,9 @@ def parse_args():
     ap.add_argument("--per-bucket", action="store_true",
                     help="strictly one launch per bucket (default: buckets that become ready together and are neighbours "
                          "in their table share a launch)")
+    ap.add_argument("--bucket-segments", action="store_true",
+                    help="every bucket stays a launch segment of its own (no merging of neighbouring buckets), "
+                         "independent segments still share launches")
     ap.add_argument("--in-order", action="store_true", help="issue every launch ordered after the previous one")
     ap.add_argument("--no-sets", action="store_true",
                     help="one kernel launch per bucket step instead of shared launches for independent steps "
@@ -280,7 +283,7 @@ def main():
     dev = torch.device("cuda:0")
     torch.cuda.set_device(dev)
     specs, targets, bucket = workloads.WORKLOADS[args.workload]()
-    merge = not args.per_bucket
+    merge = not (args.per_bucket or args.bucket_segments)
     if args.fanout > 1 and args.pool != "resident":
         print("--fanout needs --pool resident (side streams run a bucket list in list order)", file=sys.stderr)
         sys.exit(2)
@@ -324,10 +327,11 @@ def main():
         kernels.append("etha_tile_kernel")
     if kinds & {"reduce_pack", "direct_reduce"}:
         kernels.insert(0, "etha_reduce_kernel")
-    granularity = ("bucket" if not merge else
+    granularity = ("bucket" if not merge and not sets else
+                   "one segment per bucket, independent segments share launches" if not merge else
                    "run of buckets" if args.pool != "ring" else
                    "independent steps share launches" if sets else "buckets ready together")
-    mode = f"{args.pool}/{'bucket' if not merge else 'sets' if sets and args.pool == 'ring' else 'runs'}"
+    mode = f"{args.pool}/{'bucket' if not merge and not sets else 'bucket-sets' if not merge else 'sets' if sets and args.pool == 'ring' else 'runs'}"
     element = str(specs[0].source_dtype).replace("torch.", "")
     achieved = total_bytes / (dev_ms * 1e-3) / 1e9
     traffic = None if (args.zero_copy or args.direct or args.graph or args.fanout > 1 or args.in_order
@@ -416,6 +420,8 @@ def main():
 
         if merge or sets:
             out["one_launch_per_bucket"] = other_leg(False, False)
+        if merge or not sets:
+            out["one_segment_per_bucket"] = other_leg(False, True)
         if not (merge and not sets):
             out["one_launch_per_run_of_buckets"] = other_leg(True, False)
         if not (merge and sets):
