@@ -147,6 +147,9 @@ class LoopbackWire:
         self._group_flags = 0
         # host inspection: called as ``on_launch(plan, kind, first, count, flags)`` instead of launching
         self.on_launch = None
+        # host inspection of the sets: called as ``on_set([(plan, kind, first, count), ...], flags)`` instead of
+        # handing the set to the library (its members may run in any order, or at the same time)
+        self.on_set = None
         self.launch_log: list | None = None  # when a list: (kind, first, count, flags) of every launch
         self._programs: list = []  # bucket pipelines that still have work, in arrival order
         self._epoch_reads: set[int] = set()  # allocations read / written by launches since the last ordered one
@@ -392,7 +395,7 @@ class LoopbackWire:
         up by the call that brings them."""
         if not self._programs:
             return
-        cuda = self.device is not None and self.device.type == "cuda" and self.on_launch is None
+        cuda = self.device is not None and self.device.type == "cuda" and self.on_launch is None and self.on_set is None
         if cuda:
             stream = torch.cuda.current_stream(self.device)
             if self._carried and self._stream is not None and self._stream != stream:
@@ -463,7 +466,7 @@ class LoopbackWire:
     def _issue(self, plan, kind, first, count, reads, writes, excl) -> None:
         ordered = (self._ordered_next or not self.unordered_launches or not self._epoch_writes.isdisjoint(reads)
                    or not self._epoch_reads.isdisjoint(writes) or not self._epoch_writes.isdisjoint(excl))
-        if not ordered and self.on_launch is None and torch.cuda.is_current_stream_capturing():
+        if not ordered and self.on_launch is None and self.on_set is None and torch.cuda.is_current_stream_capturing():
             ordered = True  # a captured stream records its launches as a chain anyway
         if ordered:
             self._epoch_reads, self._epoch_writes = set(reads), set(writes)
@@ -479,11 +482,14 @@ class LoopbackWire:
         if self.on_launch is not None:
             self.on_launch(plan, kind, first, count, flags)
             return
-        if plan.device is None or plan.device.type != "cuda":
+        if self.on_set is None and (plan.device is None or plan.device.type != "cuda"):
             raise RuntimeError("this plan was compiled for host inspection; the executor only runs on a GPU (there is no CPU path)")
         if not self.group_launches or kind in _UNGROUPED:
             self._flush()
-            plan.launch_step(kind, first, count, self._stream.cuda_stream, flags)
+            if self.on_set is not None:
+                self.on_set([(plan, kind, first, count)], flags)
+            else:
+                plan.launch_step(kind, first, count, self._stream.cuda_stream, flags)
             return
         # an ordered launch closes the set before it and opens the next one; an unordered launch depends on
         # nothing since the last ordered one, members of the open set included, so it joins the set
@@ -501,6 +507,9 @@ class LoopbackWire:
         from .. import _native as nat
 
         group, self._group = self._group, []
+        if self.on_set is not None:
+            self.on_set(group, self._group_flags)
+            return
         if len(group) == 1:
             plan, kind, first, count = group[0]
             plan.launch_step(kind, first, count, self._stream.cuda_stream, self._group_flags)

@@ -124,7 +124,7 @@ class _HazardCheck:
             self.reads, self.writes = r, w
 
 
-def _interpret(job, merged: bool):
+def _interpret(job, merged: bool, by_sets: bool = False):
     """What ReshardJob.run would enqueue, executed on the host by the tile interpreter.  With a ring pool the
     wire's own bucket pipelines decide the order (slots are reused, so list order would be wrong); the wire
     hands every launch to the interpreter instead of the GPU."""
@@ -152,11 +152,26 @@ def _interpret(job, merged: bool):
             _run_step(mem, p, kind, first, count, ordered=(kind, first, count) in p._ordered_ranges, touched=touched)
             check.launch(touched, flags)
 
-        job.wire.on_launch = on_launch
+        def on_set(members, flags):
+            # the members of a set run at the same time on the GPU: here in reverse, which must not matter
+            if not flags & 1:
+                check.launch({}, 0)  # an ordered set: everything before it has finished
+            for p, kind, first, count in reversed(members):
+                touched = {}
+                _run_step(mem, p, kind, first, count, ordered=(kind, first, count) in p._ordered_ranges, touched=touched)
+                check.launch(touched, 1)
+            check.sets += 1
+            check.largest = max(check.largest, len(members))
+
+        check.sets = check.largest = 0
+        if by_sets:
+            job.wire.on_set = on_set
+        else:
+            job.wire.on_launch = on_launch
         try:
             job.run(merge_launches=merged)
         finally:
-            job.wire.on_launch = None
+            job.wire.on_launch = job.wire.on_set = None
         return check
     for p in plans:
         steps = p.merged_steps if merged else [(k, f, c, (s,)) for k, f, c, s in p.steps]
@@ -257,7 +272,8 @@ def test_random_batches(seed, spec_fn=None):
         for r in a:
             b[r].copy_(a[r])
     src_before = [{r: t.clone() for r, t in d.items()} for d in job.source_locals]
-    _interpret(job, merged)
+    # the launches one by one in issue order, or set by set with the members of every set in reverse
+    _interpret(job, merged, by_sets=bool(rng.integers(2)))
     run_oracle(ref)
     for i, spec in enumerate(specs):
         for r, t in job.target_locals[i].items():

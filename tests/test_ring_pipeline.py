@@ -52,6 +52,25 @@ def _ring_bound(job, depth):
     return bound
 
 
+@pytest.mark.parametrize("depth", [1, 2, 4])
+@pytest.mark.parametrize("merged", [False, True], ids=["per_bucket", "ready_runs"])
+def test_sets_of_independent_launches(depth, merged):
+    """The wire hands an ordered launch and the unordered ones that follow it to the library as one set, whose
+    members run at the same time: executed in reverse inside every set the result must be the same, no member may
+    touch a byte another one writes, and the eight senders' packs of a sweep must really share sets."""
+    specs, targets, _ = workloads.llama3_8b_fsdp8_to_tp2(n_layers=6, hidden=64, inter=224, kv=16, vocab=136)
+    job, ref = _jobs(specs, 2048, depth, targets)
+    log = job.wire.launch_log = []
+    check = _interpret(job, merged, by_sets=True)
+    run_oracle(ref)
+    _compare(job, ref, specs, f"depth {depth}")
+    assert check.sets < len(log) / 2 and check.largest >= 8
+    job.wire.group_launches = False  # every step a set of its own
+    check = _interpret(job, merged, by_sets=True)
+    assert check.largest == 1
+    _compare(job, ref, specs, f"depth {depth}, ungrouped")
+
+
 @pytest.mark.parametrize("depth", [1, 2, 3])
 @pytest.mark.parametrize("merged", [False, True], ids=["per_bucket", "ready_runs"])
 def test_llama_like_through_a_ring(depth, merged):
