@@ -8,7 +8,8 @@
  * ir.py:300-310 with Chunk.finalize ir.py:134-141).  The host planner describes
  * every chunk once ("plan once, transfer N times"); the library compiles the
  * descriptors into a device-resident tile program and each transfer is then one
- * batched kernel launch per bucket (or per run of buckets).
+ * batched kernel launch per bucket, per run of buckets, or per set of buckets that
+ * do not depend on each other (etha_launch_segments).
  *
  * Conventions
  *  - plain C types only; every function returns 0 on success or a negative
