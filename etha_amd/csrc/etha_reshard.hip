@@ -142,7 +142,11 @@ constexpr uint32_t kMetaGeneric = 1u << 20;  // converting move with an integer,
 // units is n_peers pieces of `via` units each, piece p read at gather[peer_first + p] + row * b_pitch.  The a
 // side is addressed as in any row tile, so one wavefront writes whole destination lines.
 constexpr uint32_t kMetaGather = 1u << 21;
-constexpr uint32_t kGatherMaxPieceBytes = 64;  // longer pieces already write whole lines: gathering them costs more than it gives
+// Pieces up to this size are gathered.  Measured on a four-piece scatter: 32-byte pieces 2.2 -> 6.3 TB/s, 96-byte
+// 3.9 -> 5.2, 160-byte 4.7 -> 5.2, 224-byte 5.0 -> 5.1; from 352 bytes on the plain tiles are as fast or faster
+// (5.3 against 5.1).  Pieces that are whole 128-byte lines already write whole lines and are left alone (6.5).
+constexpr uint32_t kGatherMaxPieceBytes = 256;
+constexpr uint32_t kGatherLineBytes = 128;
 constexpr uint32_t kGatherMaxPieces = 8;       // the kernel reads this many piece addresses per tile (the list is padded)
 
 // ---- typed vector access ----------------------------------------------------------------------
@@ -1555,38 +1559,56 @@ int launch_reduce(const EthaTable* t, uint32_t first, uint32_t count, void* stre
 void gather_short_pieces(std::vector<RowTile>& rows, std::vector<uint64_t>& gather) {
   std::vector<RowTile> out;
   out.reserve(rows.size());
+  // siblings of rows[at]: tiles of the same shape whose pieces follow each other inside one destination row
+  const auto siblings = [&rows](size_t at) -> uint32_t {
+    const RowTile& x = rows[at];
+    const uint64_t piece = (uint64_t)x.run << ((x.meta >> kMetaUaShift) & 15u);
+    if (x.n_peers != 0 || x.c0 != 0 || x.run >= kTileThreads || x.n % x.run != 0 || piece > kGatherMaxPieceBytes ||
+        piece % kGatherLineBytes == 0 ||
+        x.a_pitch <= 0 || (x.meta & kMetaGather))
+      return 1;
+    uint32_t have = 1;
+    while (have < kGatherMaxPieces && at + have < rows.size()) {
+      const RowTile& y = rows[at + have];
+      if (y.n_peers != 0 || y.c0 != 0 || y.n != x.n || y.run != x.run || y.meta != x.meta || y.a_pitch != x.a_pitch ||
+          y.b_pitch != x.b_pitch || y.a != x.a + have * piece || (uint64_t)(have + 1) * piece > (uint64_t)x.a_pitch ||
+          (uint64_t)(have + 1) * x.run > kTileThreads)
+        break;
+      have++;
+    }
+    return have;
+  };
   size_t i = 0;
   while (i < rows.size()) {
-    const RowTile& x = rows[i];
-    const uint32_t ua = (x.meta >> kMetaUaShift) & 15u;
-    const uint64_t piece = (uint64_t)x.run << ua;
-    bool ok = x.n_peers == 0 && x.c0 == 0 && x.run < kTileThreads && x.n % x.run == 0 && piece <= kGatherMaxPieceBytes &&
-              x.a_pitch > 0 && !(x.meta & kMetaGather);
-    uint32_t have = 1;
-    if (ok) {
-      while (have < kGatherMaxPieces && i + have < rows.size()) {
-        const RowTile& y = rows[i + have];
-        if (y.n_peers != 0 || y.c0 != 0 || y.n != x.n || y.run != x.run || y.meta != x.meta || y.a_pitch != x.a_pitch ||
-            y.b_pitch != x.b_pitch || y.a != x.a + have * piece || (uint64_t)(have + 1) * piece > (uint64_t)x.a_pitch ||
-            (uint64_t)(have + 1) * x.run > kTileThreads)
-          break;
-        have++;
-      }
-    }
-    const uint32_t n_rows = ok ? x.n / x.run : 0, pieces = have;
-    if (!ok || pieces < 2) {
+    const RowTile x = rows[i];
+    const uint32_t pieces = siblings(i);
+    if (pieces < 2) {
       out.push_back(x);
       i++;
       continue;
     }
+    // The next groups of siblings often continue the same rows (the following tiles of the same chunks): taken
+    // together, the rows are cut into gather tiles without a short tile at the end of every group.
+    uint64_t n_rows = x.n / x.run;
+    size_t next = i + pieces;
+    while (next < rows.size() && siblings(next) == pieces) {
+      const RowTile& y = rows[next];
+      bool continues = y.run == x.run && y.meta == x.meta && y.a_pitch == x.a_pitch && y.b_pitch == x.b_pitch &&
+                       y.a == x.a + n_rows * (uint64_t)x.a_pitch;
+      for (uint32_t p2 = 0; continues && p2 < pieces; p2++)
+        continues = rows[next + p2].b == (uint64_t)((int64_t)rows[i + p2].b + (int64_t)n_rows * x.b_pitch);
+      if (!continues) break;
+      n_rows += y.n / y.run;
+      next += pieces;
+    }
     const uint32_t rows_cap = kTileThreads / (x.run * pieces);  // rows one gather tile can hold
-    for (uint32_t row0 = 0; row0 < n_rows; row0 += rows_cap) {
+    for (uint64_t row0 = 0; row0 < n_rows; row0 += rows_cap) {
       RowTile g = x;
-      g.a = x.a + (uint64_t)row0 * (uint64_t)x.a_pitch;
+      g.a = x.a + row0 * (uint64_t)x.a_pitch;
       g.b = (uint64_t)((int64_t)x.b + (int64_t)row0 * x.b_pitch);  // piece 0, for inspection only
       g.meta = x.meta | kMetaGather;
       g.run = x.run * pieces;
-      g.n = (n_rows - row0 < rows_cap ? n_rows - row0 : rows_cap) * g.run;
+      g.n = (uint32_t)(n_rows - row0 < rows_cap ? n_rows - row0 : rows_cap) * g.run;
       g.peer_first = (uint32_t)gather.size();
       g.n_peers = pieces;
       g.via = x.run;
@@ -1594,7 +1616,7 @@ void gather_short_pieces(std::vector<RowTile>& rows, std::vector<uint64_t>& gath
         gather.push_back((uint64_t)((int64_t)rows[i + p2].b + (int64_t)row0 * x.b_pitch));
       out.push_back(g);
     }
-    i += pieces;
+    i = next;
   }
   rows.swap(out);
   if (!gather.empty()) gather.insert(gather.end(), kGatherMaxPieces, 0);  // a tile's fetch may run past its own pieces

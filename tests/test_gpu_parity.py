@@ -899,7 +899,8 @@ def test_large_resident_set_70b_shapes(gpu_device):
 @pytest.mark.gpu
 @pytest.mark.parametrize("pool", ["ring", "resident"])
 @pytest.mark.parametrize("cols,src_dtype,tgt_dtype", [(64, torch.bfloat16, None), (32, torch.bfloat16, None),
-                                                      (48, torch.float32, torch.bfloat16), (32, torch.bfloat16, torch.float32)])
+                                                      (48, torch.float32, torch.bfloat16), (32, torch.bfloat16, torch.float32),
+                                                      (320, torch.bfloat16, None), (192, torch.bfloat16, None)])
 def test_short_pieces_from_several_ranks_are_gathered_per_row(gpu_device, pool, cols, src_dtype, tgt_dtype):
     """Every target row is four short pieces from four source ranks' buckets.  Merged unpack launches run from the
     write-ordered copy of their range, where such pieces are assembled row by row by gather tiles."""

@@ -264,8 +264,12 @@ def test_optimized_range_is_a_write_ordered_permutation():
     (1024, 64, 4, nat.BF16, nat.BF16),   # 32-byte pieces: four per 128-byte row
     (1024, 64, 8, nat.BF16, nat.BF16),   # 16-byte pieces: one unit each
     (1500, 96, 3, nat.BF16, nat.BF16),   # 64-byte pieces, three siblings, a last tile with fewer rows
-    (640, 96, 4, nat.F32, nat.BF16),     # converting: 96-byte pieces on the tensor side are left alone ...
-    (640, 48, 6, nat.F32, nat.BF16),     # ... 32-byte ones are gathered (16 bytes each in the bucket)
+    (3000, 240, 3, nat.BF16, nat.BF16),  # 160-byte pieces over several tiles per chunk: the groups continue each other
+    (640, 96, 4, nat.F32, nat.BF16),     # converting: 96-byte pieces on the tensor side (48 bytes each in the bucket)
+    (640, 128, 4, nat.F32, nat.BF16),    # 128-byte pieces already fill whole lines: left alone
+    (300, 512, 4, nat.BF16, nat.BF16),   # 256-byte pieces likewise
+    (300, 576, 4, nat.BF16, nat.BF16),   # 288-byte pieces: too long to gain
+    (640, 48, 6, nat.F32, nat.BF16),     # 32-byte pieces (16 bytes each in the bucket)
     (333, 40, 5, nat.B8, nat.B8),        # 8-byte pieces of byte elements
     (1000, 36, 3, nat.BF16, nat.BF16),   # 24-byte pieces: three 8-byte units, tiles hold whole rows
     (777, 48, 3, nat.BF16, nat.BF16),    # three 32-byte pieces per 96-byte row
@@ -299,7 +303,7 @@ def test_short_pieces_of_one_row_are_gathered_in_an_ordered_range(rows, cols, bl
             table.optimize_range(0, blocks)
             _, o_row = table.ordered_tiles(0, blocks)
             gathered = (o_row["meta"] & GATHER) != 0
-            assert gathered.any() == (piece * es_t <= 64)
+            assert gathered.any() == (piece * es_t <= 256 and piece * es_t % 128 != 0)
             if gathered.any():
                 g = o_row[gathered]
                 assert np.all(g["n_peers"] >= 2) and np.all(g["run"] == g["via"] * g["n_peers"])
@@ -307,6 +311,8 @@ def test_short_pieces_of_one_row_are_gathered_in_an_ordered_range(rows, cols, bl
                 assert len(table.ordered_gather(0, blocks)) == int(g["n_peers"].sum()) + 8
                 # the plain tiles of the range are untouched: another range, or a pack, still uses them
                 assert not np.any(table.tiles()[1]["meta"] & GATHER)
+                # groups that continue each other are cut together: no short tile per group, so about as many tiles
+                assert len(o_row) <= len(table.tiles()[1]) + blocks
         arena.writes = np.zeros(arena.nbytes, dtype=np.int32)
         execute(table, arena, "unpack", 0, blocks, ordered=ordered)
         counts = arena.writes[arena.offsets(np.array([t]), 1)[0]:][: rows * cols * es_t]
