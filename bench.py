@@ -427,6 +427,13 @@ def main():
         if not (merge and sets):
             out["independent_steps_share_launches"] = other_leg(True, True)
         out["every_launch_in_order"] = other_leg(merge, False, unordered=False)
+        # the same launches recorded once into a HIP graph and replayed (a chain of kernel nodes)
+        captured = job.capture(merge_launches=merge)
+        captured.replay()
+        torch.cuda.synchronize()
+        ms, _ = time_steps(job, max(3, min(args.steps, 10)), captured.replay)
+        out["hip_graph_replay"] = describe(ms, n_launch, pool_bytes)
+        del captured
         del job
         torch.cuda.empty_cache()
         deeper = make_job("ring", 2 * args.max_in_flight)

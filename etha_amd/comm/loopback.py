@@ -466,8 +466,6 @@ class LoopbackWire:
     def _issue(self, plan, kind, first, count, reads, writes, excl) -> None:
         ordered = (self._ordered_next or not self.unordered_launches or not self._epoch_writes.isdisjoint(reads)
                    or not self._epoch_reads.isdisjoint(writes) or not self._epoch_writes.isdisjoint(excl))
-        if not ordered and self.on_launch is None and self.on_set is None and torch.cuda.is_current_stream_capturing():
-            ordered = True  # a captured stream records its launches as a chain anyway
         if ordered:
             self._epoch_reads, self._epoch_writes = set(reads), set(writes)
         else:

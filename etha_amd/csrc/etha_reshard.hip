@@ -1410,6 +1410,12 @@ std::atomic<uint64_t> g_kernel_launches{0};
 template <typename... Args, typename F>
 void launch_kernel(F kernel, dim3 grid, dim3 block, size_t lds, void* stream, uint32_t flags, Args... args) {
   g_kernel_launches.fetch_add(1, std::memory_order_relaxed);
+  if (flags & ETHA_LAUNCH_UNORDERED) {
+    // a stream under capture records its kernels as a chain: the flag has no meaning there
+    hipStreamCaptureStatus capture = hipStreamCaptureStatusNone;
+    if (hipStreamIsCapturing((hipStream_t)stream, &capture) != hipSuccess || capture != hipStreamCaptureStatusNone)
+      flags &= ~(uint32_t)ETHA_LAUNCH_UNORDERED;
+  }
   if (flags & ETHA_LAUNCH_UNORDERED)
     hipExtLaunchKernelGGL(kernel, grid, block, (uint32_t)lds, (hipStream_t)stream, nullptr, nullptr, hipExtAnyOrderLaunch,
                           args...);

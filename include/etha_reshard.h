@@ -71,7 +71,8 @@ enum {
  * Launch flags.  By default a launch is ordered after everything enqueued on its stream before it, like any
  * kernel.  ETHA_LAUNCH_UNORDERED declares that this launch depends on none of the launches enqueued on the
  * stream since the last launch without the flag: it may start while they are still running, which hides the
- * drain/ramp gap between kernels.  The next launch without the flag (of this library or any other kernel on
+ * drain/ramp gap between kernels.  (On a stream under capture the flag is ignored: a captured stream records a
+ * chain.)  The next launch without the flag (of this library or any other kernel on
  * the stream) waits for all of them.  The caller owns the dependency analysis: two launches that touch the
  * same bucket buffer, or a launch that reads bytes another one writes, must be separated by an ordered
  * launch.  The reference needs no such notion because each of its buckets is many small ATen launches on one
