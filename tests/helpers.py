@@ -63,7 +63,7 @@ def expected_target(spec: TensorSpec, glob: torch.Tensor, rank: int) -> torch.Te
 
 def bits(t: torch.Tensor) -> torch.Tensor:
     """Raw bytes of a tensor, for bit-exact comparison (NaNs and -0 included)."""
-    return t.detach().cpu().contiguous().view(torch.uint8).reshape(-1)
+    return t.detach().cpu().contiguous().reshape(-1).view(torch.uint8)  # flat first: a size-1 last dim may carry any stride
 
 
 def assert_bit_equal(a: torch.Tensor, b: torch.Tensor, what: str = "") -> None:
