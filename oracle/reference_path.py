@@ -109,7 +109,9 @@ def bucket_prepare_source(bucket) -> torch.Tensor:
     """``Bucket.prepare`` of a producing bucket: returns the uint8 wire buffer (``ir.py:229-264``)."""
     chunks = bucket.chunks
     if len(chunks) == 1:
-        return chunk_prepare(chunks[0]).contiguous().view(torch.uint8).reshape(-1)
+        # (flattened before the byte view: the reference's plain .view(torch.uint8) refuses a last dim of one
+        # element that carries a stride other than 1, which torch reports for some slices; the bytes are the same)
+        return chunk_prepare(chunks[0]).contiguous().reshape(-1).view(torch.uint8)
     offsets = bucket_offsets(bucket)
     total = offsets[-1] + chunks[-1].nbytes
     buffer = torch.empty(total, dtype=torch.uint8)
