@@ -76,6 +76,7 @@ class TransferPlan:
         self.steps: list[tuple[str, int, int, object]] = []
         self.info: list[StepInfo] = []
         self.steps_of: dict[int, list[int]] = {}  # id(bucket) -> indices of its steps
+        self.bucket_steps: dict[int, list] = {}  # id(bucket) -> [(index, kind, info)], filled on first use
         self.lent: set[int] = set()  # ids of source buckets that are consumed straight from their tensor
         self.direct_read_bytes = 0  # bytes the direct steps read from producers' tensors (source dtype)
         self.owned_entries: list = []  # wire entries of this list's send buckets
@@ -514,7 +515,10 @@ class Program:
 
     def _steps(self, bucket):
         plan = self.plan
-        return [(i, plan.steps[i][0], plan.info[i]) for i in plan.steps_of.get(id(bucket), ())]
+        cached = plan.bucket_steps.get(id(bucket))
+        if cached is None:  # the plan's steps never change once it is compiled
+            cached = plan.bucket_steps[id(bucket)] = [(i, plan.steps[i][0], plan.info[i]) for i in plan.steps_of.get(id(bucket), ())]
+        return cached
 
     def _prepare(self, bucket, wire, todo: list) -> bool:
         steps = self._steps(bucket)
