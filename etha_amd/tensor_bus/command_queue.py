@@ -13,6 +13,7 @@ from __future__ import annotations
 import os
 import pickle
 import sqlite3
+import threading
 import time
 from multiprocessing.connection import Client, Connection, Listener
 
@@ -130,6 +131,7 @@ class PersistentCommandQueue:
             raise ValueError("capacity must be positive")
         self.lmdb_path = str(lmdb_path)
         self.capacity = int(capacity)
+        self._lock = threading.Lock()  # one connection, used by several threads: one transaction at a time
         self.env: sqlite3.Connection | None = sqlite3.connect(self.lmdb_path, timeout=30.0, isolation_level=None,
                                                               check_same_thread=False)
         with open(self.lmdb_path + "-lock", "a"):  # the companion file the reference's store keeps beside the data
@@ -140,15 +142,16 @@ class PersistentCommandQueue:
 
     # -- transactions ----------------------------------------------------------------------------
     def _tx(self, sql: str, args: tuple = ()):
-        env = self._env()
-        env.execute("BEGIN IMMEDIATE")
-        try:
-            out = env.execute(sql, args).fetchall()
-            env.execute("COMMIT")
-            return out
-        except BaseException:
-            env.execute("ROLLBACK")
-            raise
+        with self._lock:
+            env = self._env()
+            env.execute("BEGIN IMMEDIATE")
+            try:
+                out = env.execute(sql, args).fetchall()
+                env.execute("COMMIT")
+                return out
+            except BaseException:
+                env.execute("ROLLBACK")
+                raise
 
     def _env(self) -> sqlite3.Connection:
         if self.env is None:
@@ -164,25 +167,31 @@ class PersistentCommandQueue:
         deadline = None if timeout is None else time.monotonic() + timeout
         data = pickle.dumps(msg, protocol=pickle.HIGHEST_PROTOCOL)
         while True:
-            env = self._env()
-            env.execute("BEGIN IMMEDIATE")
-            try:
-                head, tail = self._pointers(env)
-                if tail - head < self.capacity:
-                    env.execute("INSERT OR REPLACE INTO slots VALUES (?, ?)", (tail % self.capacity, data))
-                    env.execute("UPDATE pointers SET value = ? WHERE name = 'tail'", (tail + 1,))
-                    env.execute("COMMIT")
-                    return tail
-                env.execute("ROLLBACK")
-            except BaseException:
-                env.execute("ROLLBACK")
-                raise
+            with self._lock:
+                env = self._env()
+                env.execute("BEGIN IMMEDIATE")
+                try:
+                    head, tail = self._pointers(env)
+                    if tail - head < self.capacity:
+                        env.execute("INSERT OR REPLACE INTO slots VALUES (?, ?)", (tail % self.capacity, data))
+                        env.execute("UPDATE pointers SET value = ? WHERE name = 'tail'", (tail + 1,))
+                        env.execute("COMMIT")
+                        return tail
+                    env.execute("ROLLBACK")
+                except BaseException:
+                    if env.in_transaction:
+                        env.execute("ROLLBACK")
+                    raise
             if not block or (deadline is not None and time.monotonic() >= deadline):
                 raise QueueFullError(f"Queue is full (capacity={self.capacity})")
             time.sleep(self._POLL_S)
 
     # -- consumer --------------------------------------------------------------------------------
     def _take(self, max_count: int, remove: bool = True) -> list:
+        with self._lock:
+            return self._take_locked(max_count, remove)
+
+    def _take_locked(self, max_count: int, remove: bool) -> list:
         env = self._env()
         env.execute("BEGIN IMMEDIATE")
         try:
@@ -221,30 +230,33 @@ class PersistentCommandQueue:
         return got[0] if got else None
 
     def size(self) -> int:
-        head, tail = self._pointers(self._env())
+        with self._lock:
+            head, tail = self._pointers(self._env())
         return tail - head
 
     def is_empty(self) -> bool:
         return self.size() == 0
 
     def clear(self, delete_commands: bool = True) -> None:
-        env = self._env()
-        env.execute("BEGIN IMMEDIATE")
-        try:
-            env.execute("UPDATE pointers SET value = 0")
-            if delete_commands:
-                env.execute("DELETE FROM slots")
-            env.execute("COMMIT")
-        except BaseException:
-            env.execute("ROLLBACK")
-            raise
+        with self._lock:
+            env = self._env()
+            env.execute("BEGIN IMMEDIATE")
+            try:
+                env.execute("UPDATE pointers SET value = 0")
+                if delete_commands:
+                    env.execute("DELETE FROM slots")
+                env.execute("COMMIT")
+            except BaseException:
+                env.execute("ROLLBACK")
+                raise
 
     def close(self, destroy: bool = True) -> None:
         """``destroy=True`` (the default, as in the reference) removes the queue's files; ``destroy=False`` only
         closes this opener's handle.  Safe to call more than once."""
-        if self.env is not None:
-            self.env.close()
-            self.env = None
+        with self._lock:
+            if self.env is not None:
+                self.env.close()
+                self.env = None
         if destroy:
             for suffix in ("", "-lock", "-journal", "-wal", "-shm"):
                 try:
