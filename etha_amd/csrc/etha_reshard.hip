@@ -142,11 +142,6 @@ constexpr uint32_t kMetaGeneric = 1u << 20;  // converting move with an integer,
 // units is n_peers pieces of `via` units each, piece p read at gather[peer_first + p] + row * b_pitch.  The a
 // side is addressed as in any row tile, so one wavefront writes whole destination lines.
 constexpr uint32_t kMetaGather = 1u << 21;
-// Pieces up to this size are gathered.  Measured on a four-piece scatter: 32-byte pieces 2.2 -> 6.3 TB/s, 96-byte
-// 3.9 -> 5.2, 160-byte 4.7 -> 5.2, 224-byte 5.0 -> 5.1; from 352 bytes on the plain tiles are as fast or faster
-// (5.3 against 5.1).  Pieces that are whole 128-byte lines already write whole lines and are left alone (6.5).
-constexpr uint32_t kGatherMaxPieceBytes = 256;
-constexpr uint32_t kGatherLineBytes = 128;
 constexpr uint32_t kGatherMaxPieces = 8;       // the kernel reads this many piece addresses per tile (the list is padded)
 
 // ---- typed vector access ----------------------------------------------------------------------
@@ -415,7 +410,7 @@ __device__ __forceinline__ void row_position(const RowTile& t, uint32_t tid, uin
 }
 
 // pack (REV = false): a -> b.   unpack (REV = true): b -> a.
-template <bool REV>
+template <bool REV, bool GATHER = false>
 __device__ __forceinline__ void tile_body(const RunTile* __restrict__ run_tiles, uint32_t n_run,
                                           const RowTile* __restrict__ row_tiles, const uint64_t* __restrict__ gather,
                                           uint32_t bid, uint32_t tid) {
@@ -434,7 +429,7 @@ __device__ __forceinline__ void tile_body(const RunTile* __restrict__ run_tiles,
     uint32_t r, c;
     row_position(t, tid, r, c);
     a = t.a + (uint64_t)((int64_t)r * t.a_pitch) + ((uint64_t)c << ((meta >> kMetaUaShift) & 15u));
-    if (REV && (meta & kMetaGather)) {
+    if (GATHER && (meta & kMetaGather)) {
       if (tid >= n) return;
       const uint32_t p = c / t.via;
       // the tile's piece addresses are the same for every lane: fetched through the scalar path, picked per lane
@@ -494,6 +489,25 @@ __global__ __launch_bounds__(ETHA_BLOCK_THREADS) void etha_tile_kernel_2d(const 
   const RowTile* row = (const RowTile*)(GlobalRow)(((uint64_t)raw[3] << 32) | raw[2]);
   const uint64_t* gather = (const uint64_t*)(GlobalU64)(((uint64_t)raw[5] << 32) | raw[4]);
   tile_body<REV>(run, raw[6], row, gather, bid, (blockIdx.x % kBlocksPerTile) * kBlockThreads + threadIdx.x);
+}
+
+// The gather tiles of write-ordered unpack ranges (see kMetaGather).  Consecutive 1 KiB pieces of such a tile read
+// source lines that they share with their neighbours (a piece of 96 bytes does not end on a line), so the
+// workgroups of one tile should share an L2: workgroups are dealt to the eight XCDs in turn, and this kernel lets
+// workgroup w of every 128 handle piece w / 8 of tile w % 8 - the sixteen pieces of a tile then run on one XCD,
+// close in time.  Measured on 96- to 480-byte pieces: 5.1-5.3 -> 6.25-6.3 TB/s.  (The same mapping costs plain
+// copies 8 %: it is used for gather tiles only.)
+static_assert(kBlocksPerTile == 16, "the XCD mapping below deals 8 tiles x 16 pieces to 128 workgroups");
+__global__ __launch_bounds__(ETHA_BLOCK_THREADS) void etha_gather_kernel(const Args2D args) {
+  typedef uint32_t u32x8 __attribute__((ext_vector_type(8)));
+  const u32x8 raw = *reinterpret_cast<const u32x8*>(&args.seg[blockIdx.y]);
+  const uint32_t w = blockIdx.x, tile = ((w >> 7) << 3) + (w & 7u), piece = (w & 127u) >> 3;
+  if (tile >= raw[7]) return;
+  typedef const __attribute__((address_space(1))) RowTile* GlobalRow;
+  typedef const __attribute__((address_space(1))) uint64_t* GlobalU64;
+  const RowTile* row = (const RowTile*)(GlobalRow)(((uint64_t)raw[3] << 32) | raw[2]);
+  const uint64_t* gather = (const uint64_t*)(GlobalU64)(((uint64_t)raw[5] << 32) | raw[4]);
+  tile_body<true, true>(nullptr, 0u, row, gather, tile, piece * kBlockThreads + threadIdx.x);
 }
 
 // ---- transposing chunks: staged through LDS -----------------------------------------------------
@@ -965,10 +979,6 @@ struct Builder {
   uint64_t payload_bytes = 0;
 };
 
-#ifndef ETHA_SHORT_ROW_UNITS
-#define ETHA_SHORT_ROW_UNITS 64
-#endif
-constexpr uint64_t kShortRowUnits = ETHA_SHORT_ROW_UNITS;  // rows of at most this many units never straddle a tile
 constexpr uint64_t kMaxTiles = 0x7fff0000ull / kBlocksPerTile;  // grid.x limit with margin
 
 struct ReduceSpec {
@@ -1235,9 +1245,7 @@ class PairCompiler {
         const uint64_t rows = k_ > 0 ? (uint64_t)n_[k_ - 1] : 1;
         const int64_t pa = k_ > 0 ? sa_[k_ - 1] : 0, pb = k_ > 0 ? sb_[k_ - 1] : 0;
         const uint64_t total = rows * run_units;
-        // tiles of short rows hold whole rows (a few lanes of the last workgroup stay idle): such tiles can be
-        // regrouped row-wise with the tiles of neighbouring chunks when a range is ordered by written address
-        const uint64_t step = rows > 1 && run_units <= kShortRowUnits ? (kTileThreads / run_units) * run_units : kTileThreads;
+        const uint64_t step = kTileThreads;
         for (uint64_t q = 0; q < total; q += step) {
           RowTile t;
           memset(&t, 0, sizeof(t));
@@ -1314,7 +1322,8 @@ struct EthaTable {
   // write-ordered copies of the tiles of ranges that are always launched as one unit
   struct Ordered {
     std::vector<RunTile> h_run;
-    std::vector<RowTile> h_row;
+    std::vector<RowTile> h_row;      // plain row tiles, then the gather tiles
+    uint32_t n_plain_rows = 0;
     std::vector<uint64_t> h_gather;  // piece addresses of the gather tiles
     RunTile* d_run = nullptr;
     RowTile* d_row = nullptr;
@@ -1434,11 +1443,33 @@ Seg2D tile_range(const EthaTable* t, uint32_t first, uint32_t count, bool rev) {
       g.run = it->second.d_run;
       g.row = it->second.d_row;
       g.gather = it->second.d_gather;
-      g.n_run = (uint32_t)it->second.h_run.size();  // gathering regroups row tiles: their number may differ
-      g.n_tiles = g.n_run + (uint32_t)it->second.h_row.size();
+      g.n_run = (uint32_t)it->second.h_run.size();
+      g.n_tiles = g.n_run + it->second.n_plain_rows;  // chunks covered by gather tiles have no plain tiles here
     }
   }
   return g;
+}
+
+// the gather tiles of an unpack range that has a write-ordered copy (n_tiles == 0: none)
+Seg2D gather_range(const EthaTable* t, uint32_t first, uint32_t count, bool rev) {
+  Seg2D g{nullptr, nullptr, nullptr, 0, 0};
+  if (!rev || t->kind != 0) return g;
+  auto it = t->ordered.find(std::make_pair(first, count));
+  if (it == t->ordered.end()) return g;
+  g.row = it->second.d_row + it->second.n_plain_rows;
+  g.gather = it->second.d_gather;
+  g.n_tiles = (uint32_t)it->second.h_row.size() - it->second.n_plain_rows;
+  return g;
+}
+
+// workgroups of a gather launch over `tiles` tiles: 8 tiles x 16 pieces per 128 workgroups
+uint32_t gather_grid(uint32_t tiles) { return ((tiles + 7u) / 8u) * 128u; }
+
+void launch_gather(const Seg2D* segs, uint32_t n, uint32_t top, void* stream, uint32_t flags) {
+  Args2D args;
+  memset(&args, 0, sizeof(args));
+  for (uint32_t k = 0; k < n; k++) args.seg[k] = segs[k];
+  launch_kernel(etha_gather_kernel, dim3(gather_grid(top), n), dim3(kBlockThreads), 0, stream, flags, args);
 }
 
 // transposing chunks run in their own kernel (it needs LDS); true when one was launched
@@ -1470,8 +1501,12 @@ int launch_tiles(const EthaTable* t, uint32_t first, uint32_t count, void* strea
     flags |= ETHA_LAUNCH_UNORDERED;  // the two kernels of one call touch different chunks
   }
   const Seg2D g = tile_range(t, first, count, REV);
-  if (g.n_tiles == 0) return ETHA_OK;
-  launch_plain(g, REV, stream, flags);
+  if (g.n_tiles) {
+    launch_plain(g, REV, stream, flags);
+    flags |= ETHA_LAUNCH_UNORDERED;
+  }
+  const Seg2D gathered = gather_range(t, first, count, REV);
+  if (gathered.n_tiles) launch_gather(&gathered, 1, gathered.n_tiles, stream, flags);
   HIP_TRY(hipGetLastError());
   return ETHA_OK;
 }
@@ -1555,76 +1590,96 @@ int launch_reduce(const EthaTable* t, uint32_t first, uint32_t count, void* stre
   return ETHA_OK;
 }
 
-// Short pieces of one destination row that arrive through different chunks (a target row assembled from
-// several source ranks' column blocks): written one piece per tile, every 64-byte DRAM burst is written in parts
-// by different workgroups, which costs more than half the bandwidth at 32-byte pieces.  In a write-ordered range
-// the tiles of such sibling chunks are neighbours (same rows, adjacent columns).  P of them, each covering R rows,
-// are replaced by about P gather tiles that cover about R / P rows each but all P pieces of every row, so that one
-// wavefront writes whole lines and reads P short streams.  Bytes moved are the same.
+// Pieces of one destination row that arrive through different chunks (a target row assembled from several source
+// ranks' column blocks).  When a piece is not a whole number of 128-byte lines, every line at a piece boundary is
+// written in parts by different workgroups, which costs up to two thirds of the bandwidth (2.2 instead of 6.5 TB/s
+// at 32-byte pieces, 5.3 at 352 bytes).  In a write-ordered unpack range such sibling chunks - same rows, same
+// shape, adjacent columns - are taken out of the plain tiles and covered by gather tiles instead: row tiles whose
+// row is all P pieces, so that one wavefront writes whole lines and reads P short streams.
+constexpr uint32_t kGatherLineBytes = 128;
 
-void gather_short_pieces(std::vector<RowTile>& rows, std::vector<uint64_t>& gather) {
-  std::vector<RowTile> out;
-  out.reserve(rows.size());
-  // siblings of rows[at]: tiles of the same shape whose pieces follow each other inside one destination row
-  const auto siblings = [&rows](size_t at) -> uint32_t {
-    const RowTile& x = rows[at];
-    const uint64_t piece = (uint64_t)x.run << ((x.meta >> kMetaUaShift) & 15u);
-    if (x.n_peers != 0 || x.c0 != 0 || x.run >= kTileThreads || x.n % x.run != 0 || piece > kGatherMaxPieceBytes ||
-        piece % kGatherLineBytes == 0 ||
-        x.a_pitch <= 0 || (x.meta & kMetaGather))
-      return 1;
-    uint32_t have = 1;
-    while (have < kGatherMaxPieces && at + have < rows.size()) {
-      const RowTile& y = rows[at + have];
-      if (y.n_peers != 0 || y.c0 != 0 || y.n != x.n || y.run != x.run || y.meta != x.meta || y.a_pitch != x.a_pitch ||
-          y.b_pitch != x.b_pitch || y.a != x.a + have * piece || (uint64_t)(have + 1) * piece > (uint64_t)x.a_pitch ||
-          (uint64_t)(have + 1) * x.run > kTileThreads)
-        break;
-      have++;
-    }
-    return have;
-  };
+struct PieceRows {  // a chunk that is a plain 2-D block of rows: rows x run units at the two pitches
+  uint32_t chunk;
+  uint64_t a, b;
+  int64_t a_pitch, b_pitch;
+  uint32_t run, meta;
+  uint64_t rows;
+};
+
+// the chunk as PieceRows when its tiles are exactly one such block (no run tiles, no transposing tiles, one tile
+// sequence that walks the rows in order)
+bool piece_rows_of(const EthaTable* t, uint32_t c, PieceRows* out) {
+  const uint32_t w0 = t->row_begin[c], w1 = t->row_begin[c + 1];
+  if (w1 == w0 || t->run_begin[c + 1] != t->run_begin[c] || t->trans_begin[c + 1] != t->trans_begin[c]) return false;
+  const RowTile& t0 = t->h_row[w0];
+  if (t0.n_peers != 0 || t0.c0 != 0 || t0.run >= kTileThreads || t0.a_pitch <= 0) return false;
+  uint64_t units = 0;
+  for (uint32_t k = w0; k < w1; k++) {
+    const RowTile& y = t->h_row[k];
+    const uint64_t r = units / t0.run, c0 = units % t0.run;
+    if (y.n_peers != 0 || y.run != t0.run || y.meta != t0.meta || y.a_pitch != t0.a_pitch || y.b_pitch != t0.b_pitch ||
+        y.c0 != c0 || y.a != t0.a + r * (uint64_t)t0.a_pitch || y.b != (uint64_t)((int64_t)t0.b + (int64_t)r * t0.b_pitch))
+      return false;
+    units += y.n;
+  }
+  if (units % t0.run != 0) return false;
+  *out = PieceRows{c, t0.a, t0.b, t0.a_pitch, t0.b_pitch, t0.run, t0.meta, units / t0.run};
+  return true;
+}
+
+// Finds the sibling groups among chunks [first, first + count), appends their gather tiles and piece addresses,
+// and marks the chunks they replace.
+void gather_sibling_chunks(const EthaTable* t, uint32_t first, uint32_t count, std::vector<RowTile>& tiles,
+                           std::vector<uint64_t>& gather, std::vector<char>& replaced) {
+  std::vector<PieceRows> cand;
+  for (uint32_t c = first; c < first + count; c++) {
+    PieceRows p;
+    if (piece_rows_of(t, c, &p)) cand.push_back(p);
+  }
+  std::stable_sort(cand.begin(), cand.end(), [](const PieceRows& x, const PieceRows& y) { return x.a < y.a; });
   size_t i = 0;
-  while (i < rows.size()) {
-    const RowTile x = rows[i];
-    const uint32_t pieces = siblings(i);
+  while (i < cand.size()) {
+    const PieceRows& x = cand[i];
+    const uint64_t piece = (uint64_t)x.run << ((x.meta >> kMetaUaShift) & 15u);
+    uint32_t pieces = 1;
+    if (piece % kGatherLineBytes != 0) {
+      while (pieces < kGatherMaxPieces && i + pieces < cand.size()) {
+        const PieceRows& y = cand[i + pieces];
+        if (y.run != x.run || y.meta != x.meta || y.a_pitch != x.a_pitch || y.b_pitch != x.b_pitch || y.rows != x.rows ||
+            y.a != x.a + pieces * piece || (uint64_t)(pieces + 1) * piece > (uint64_t)x.a_pitch ||
+            (uint64_t)(pieces + 1) * x.run > kTileThreads)
+          break;
+        pieces++;
+      }
+    }
     if (pieces < 2) {
-      out.push_back(x);
       i++;
       continue;
     }
-    // The next groups of siblings often continue the same rows (the following tiles of the same chunks): taken
-    // together, the rows are cut into gather tiles without a short tile at the end of every group.
-    uint64_t n_rows = x.n / x.run;
-    size_t next = i + pieces;
-    while (next < rows.size() && siblings(next) == pieces) {
-      const RowTile& y = rows[next];
-      bool continues = y.run == x.run && y.meta == x.meta && y.a_pitch == x.a_pitch && y.b_pitch == x.b_pitch &&
-                       y.a == x.a + n_rows * (uint64_t)x.a_pitch;
-      for (uint32_t p2 = 0; continues && p2 < pieces; p2++)
-        continues = rows[next + p2].b == (uint64_t)((int64_t)rows[i + p2].b + (int64_t)n_rows * x.b_pitch);
-      if (!continues) break;
-      n_rows += y.n / y.run;
-      next += pieces;
-    }
-    const uint32_t rows_cap = kTileThreads / (x.run * pieces);  // rows one gather tile can hold
-    for (uint64_t row0 = 0; row0 < n_rows; row0 += rows_cap) {
-      RowTile g = x;
+    // the rows of all pieces, `width` units each, are cut into tiles of kTileThreads units like any other rows
+    const uint64_t width = (uint64_t)x.run * pieces, total = x.rows * width;
+    for (uint64_t q = 0; q < total; q += kTileThreads) {
+      const uint64_t row0 = q / width;
+      RowTile g;
+      memset(&g, 0, sizeof(g));
       g.a = x.a + row0 * (uint64_t)x.a_pitch;
       g.b = (uint64_t)((int64_t)x.b + (int64_t)row0 * x.b_pitch);  // piece 0, for inspection only
+      g.a_pitch = x.a_pitch;
+      g.b_pitch = x.b_pitch;
       g.meta = x.meta | kMetaGather;
-      g.run = x.run * pieces;
-      g.n = (uint32_t)(n_rows - row0 < rows_cap ? n_rows - row0 : rows_cap) * g.run;
+      g.run = (uint32_t)width;
+      g.c0 = (uint32_t)(q % width);
+      g.n = (uint32_t)(total - q < kTileThreads ? total - q : kTileThreads);
       g.peer_first = (uint32_t)gather.size();
       g.n_peers = pieces;
       g.via = x.run;
       for (uint32_t p2 = 0; p2 < pieces; p2++)
-        gather.push_back((uint64_t)((int64_t)rows[i + p2].b + (int64_t)row0 * x.b_pitch));
-      out.push_back(g);
+        gather.push_back((uint64_t)((int64_t)cand[i + p2].b + (int64_t)row0 * x.b_pitch));
+      tiles.push_back(g);
     }
-    i = next;
+    for (uint32_t p2 = 0; p2 < pieces; p2++) replaced[cand[i + p2].chunk - first] = 1;
+    i += pieces;
   }
-  rows.swap(out);
   if (!gather.empty()) gather.insert(gather.end(), kGatherMaxPieces, 0);  // a tile's fetch may run past its own pieces
 }
 
@@ -1854,9 +1909,13 @@ int etha_table_optimize_range(EthaTable* t, uint32_t first, uint32_t count) {
   const auto key = std::make_pair(first, count);
   if (t->ordered.count(key)) return ETHA_OK;
   EthaTable::Ordered o;
-  o.h_run.assign(t->h_run.begin() + t->run_begin[first], t->h_run.begin() + t->run_begin[first + count]);
-  o.h_row.assign(t->h_row.begin() + t->row_begin[first], t->h_row.begin() + t->row_begin[first + count]);
   const bool by_a = t->kind == 0;  // unpack writes the tensor (a) side; a self-copy writes its b side
+  std::vector<RowTile> gather_tiles;
+  std::vector<char> replaced(count, 0);
+  if (by_a) gather_sibling_chunks(t, first, count, gather_tiles, o.h_gather, replaced);
+  o.h_run.assign(t->h_run.begin() + t->run_begin[first], t->h_run.begin() + t->run_begin[first + count]);
+  for (uint32_t c = first; c < first + count; c++)
+    if (!replaced[c - first]) o.h_row.insert(o.h_row.end(), t->h_row.begin() + t->row_begin[c], t->h_row.begin() + t->row_begin[c + 1]);
   const auto unit = [](uint32_t meta, bool a_side) { return 1ull << ((meta >> (a_side ? kMetaUaShift : kMetaUbShift)) & 15u); };
   std::stable_sort(o.h_run.begin(), o.h_run.end(),
                    [by_a](const RunTile& x, const RunTile& y) { return by_a ? x.a < y.a : x.b < y.b; });
@@ -1864,7 +1923,8 @@ int etha_table_optimize_range(EthaTable* t, uint32_t first, uint32_t count) {
     const uint64_t px = (by_a ? x.a : x.b) + x.c0 * unit(x.meta, by_a), py = (by_a ? y.a : y.b) + y.c0 * unit(y.meta, by_a);
     return px < py;
   });
-  if (by_a) gather_short_pieces(o.h_row, o.h_gather);
+  o.n_plain_rows = (uint32_t)o.h_row.size();
+  o.h_row.insert(o.h_row.end(), gather_tiles.begin(), gather_tiles.end());  // in address order already
   if (t->uploaded) {
     const size_t run_bytes = o.h_run.size() * sizeof(RunTile), row_bytes = o.h_row.size() * sizeof(RowTile);
     const size_t gather_bytes = o.h_gather.size() * sizeof(uint64_t);
@@ -1959,7 +2019,7 @@ int etha_launch_segments(const EthaSegment* segs, uint32_t n_segments, void* str
     if (g.kind == ETHA_SEG_SELFCOPY && n_reduce && n_reduce != g.count)
       return fail(ETHA_ERR_INVALID, "segment %u: range mixes Partial and plain chunks; launch them separately", i);
   }
-  std::vector<Seg2D> forward, reverse;
+  std::vector<Seg2D> forward, reverse, gathered;
   std::vector<TransSeg> trans_forward, trans_reverse;
   uint32_t trans_lds = 0;
   for (uint32_t i = 0; i < n_segments; i++) {
@@ -1982,11 +2042,16 @@ int etha_launch_segments(const EthaSegment* segs, uint32_t n_segments, void* str
     }
     const Seg2D r = tile_range(t, g.first, g.count, rev);
     if (r.n_tiles) (rev ? reverse : forward).push_back(r);
+    const Seg2D gr = gather_range(t, g.first, g.count, rev);
+    if (gr.n_tiles) gathered.push_back(gr);
   }
   launch_trans_group(trans_forward, false, trans_lds, stream, flags);
   launch_trans_group(trans_reverse, true, trans_lds, stream, flags);
   launch_group(forward, false, stream, flags);
   launch_group(reverse, true, stream, flags);
+  launch_neighbours(
+      gathered, kJoinMaxIdleTiles, [](const Seg2D& x) { return (uint64_t)x.n_tiles; },
+      [&](size_t i, size_t j, uint32_t top, uint32_t fl) { launch_gather(&gathered[i], (uint32_t)(j - i), top, stream, fl); }, flags);
   HIP_TRY(hipGetLastError());
   return ETHA_OK;
 }

@@ -200,7 +200,8 @@ int etha_table_read_trans_ranges(const EthaTable* table, uint32_t* trans_begin);
 int etha_table_optimize_range(EthaTable* table, uint32_t first, uint32_t count);
 /* host copy of an optimized range's tiles, in launch order; same conventions as etha_table_read_tiles, plus
  * which = 3: the piece addresses (uint64) of the range's gather tiles - row tiles that assemble each
- * destination row from short pieces of several chunks, so that whole lines are written at once */
+ * destination row from the pieces of several chunks, so that whole lines are written at once.  They follow
+ * the plain row tiles in which = 1 and run in a kernel of their own. */
 int etha_table_read_ordered(const EthaTable* table, uint32_t first, uint32_t count, int which, void* out,
                             uint64_t cap_bytes, uint64_t* need_bytes);
 

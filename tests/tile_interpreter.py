@@ -99,7 +99,7 @@ def _unit_positions(run_tiles, row_tiles, gather=None):
         g = (meta & GATHER) != 0
         if g.any():
             assert gather is not None and np.all(t["n_peers"][g] >= 2) and np.all(t["via"][g] > 0)
-            assert np.all(t["run"][g] == t["via"][g] * t["n_peers"][g]) and np.all(t["c0"][g] == 0)
+            assert np.all(t["run"][g] == t["via"][g] * t["n_peers"][g])
             piece = c[g] // t["via"][g].astype(np.int64)
             base = gather[t["peer_first"][g].astype(np.int64) + piece].astype(np.int64)
             b[g] = base + r[g] * t["b_pitch"][g] + ((c[g] - piece * t["via"][g].astype(np.int64)) << ((meta[g] >> 4) & 15))
