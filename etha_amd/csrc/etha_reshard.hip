@@ -119,11 +119,20 @@ constexpr uint32_t kTransThreads = ETHA_TRANS_THREADS;
 // 8-byte elements, which keeps the LDS footprint of a block at 16-66 KB
 __host__ __device__ constexpr uint32_t trans_dim_a(uint32_t es) { return es == 8 ? ETHA_TRANS_DIM_A / 2u : (uint32_t)ETHA_TRANS_DIM_A; }
 __host__ __device__ constexpr uint32_t trans_dim_b(uint32_t es) { return es == 8 ? ETHA_TRANS_DIM_B / 2u : (uint32_t)ETHA_TRANS_DIM_B; }
+// Where a chunk is large enough, blocks are kTransPanels(es) times that extent on both sides ("wide" blocks):
+// a 128-element side of 2-byte elements is a run of only 256 bytes, and runs of 512 bytes move faster.  A wide
+// block is loaded whole into registers and goes through LDS one panel of trans_dim columns at a time, so LDS
+// holds a panel, not the block.
+#ifndef ETHA_TRANS_PANELS
+#define ETHA_TRANS_PANELS 2
+#endif
+__host__ __device__ constexpr uint32_t trans_panels(uint32_t es) { return es == 2 ? (uint32_t)ETHA_TRANS_PANELS : 1u; }
 __host__ __device__ constexpr uint32_t trans_pitch(uint32_t dim, uint32_t es) {  // LDS row pitch in elements: an odd number of words
   return dim + (es >= 4 ? 1u : 4u / es);
 }
-__host__ __device__ constexpr uint32_t trans_lds_bytes(uint32_t es) {  // either direction: rows of one side, one row per element of the other
-  const uint32_t fwd = trans_dim_b(es) * trans_pitch(trans_dim_a(es), es) * es, rev = trans_dim_a(es) * trans_pitch(trans_dim_b(es), es) * es;
+__host__ __device__ constexpr uint32_t trans_lds_bytes(uint32_t es) {  // either direction: rows of one side (of a wide block, if any), one row per element of the other
+  const uint32_t p = trans_panels(es);
+  const uint32_t fwd = p * trans_dim_b(es) * trans_pitch(trans_dim_a(es), es) * es, rev = p * trans_dim_a(es) * trans_pitch(trans_dim_b(es), es) * es;
   return fwd > rev ? fwd : rev;
 }
 
@@ -517,63 +526,102 @@ __global__ __launch_bounds__(ETHA_BLOCK_THREADS) void etha_gather_kernel(const A
 // vector gathered element by element from LDS.  Both global sides therefore move whole 16-byte vectors in
 // runs of at least 128 bytes; without the staging one side would touch a different line per element.
 // Blocks at the edge of a chunk (fewer than D elements on a side) take the element-wise path.
+// the vectors q = tid + i * kTransThreads of DY source rows of DX elements each, row by row
+template <typename E, uint32_t DX, uint32_t DY>
+struct TransBlock {
+  static constexpr uint32_t kEs = sizeof(E), kV = 16 / kEs, kVecPerRow = DX / kV, kOutPerRow = DY / kV;
+  static constexpr uint32_t kPitchBytes = trans_pitch(DX, kEs) * kEs;  // a multiple of 4
+  static constexpr uint32_t kVecs = DY * kVecPerRow, kPerThread = (kVecs + kTransThreads - 1) / kTransThreads;
+  static constexpr bool kExact = kVecs % kTransThreads == 0;
+
+  static __device__ __forceinline__ void load(u32x4 (&v)[kPerThread], uint64_t src, int64_t src_pitch) {
+    const uint32_t tid = threadIdx.x;
+#pragma unroll
+    for (uint32_t i = 0; i < kPerThread; i++) {
+      const uint32_t q = tid + i * kTransThreads, y = q / kVecPerRow, xv = q % kVecPerRow;
+      if (kExact || q < kVecs) v[i] = ld_stream<u32x4_any>(src + (uint64_t)((int64_t)y * src_pitch) + xv * 16u);
+    }
+  }
+  static __device__ __forceinline__ void park(const u32x4 (&v)[kPerThread], uint8_t* __restrict__ lds) {
+    const uint32_t tid = threadIdx.x;
+#pragma unroll
+    for (uint32_t i = 0; i < kPerThread; i++) {
+      const uint32_t q = tid + i * kTransThreads, y = q / kVecPerRow, xv = q % kVecPerRow;
+      if (!kExact && q >= kVecs) break;
+      uint32_t* row = reinterpret_cast<uint32_t*>(lds + y * kPitchBytes + xv * 16u);
+      row[0] = v[i][0];
+      row[1] = v[i][1];
+      row[2] = v[i][2];
+      row[3] = v[i][3];
+    }
+  }
+  // writes the DX destination rows (index x) of DY elements out of the parked rows
+  static __device__ __forceinline__ void emit(const uint8_t* __restrict__ lds, uint64_t dst, int64_t dst_pitch) {
+    const uint32_t tid = threadIdx.x;
+    if constexpr (kEs == 2) {
+      // two destination rows at a time: the 32-bit words of 8 source rows hold the elements of columns x and x + 1
+      constexpr uint32_t kPairs = kVecs / 2, kPairsPerThread = (kPairs + kTransThreads - 1) / kTransThreads;
+#pragma unroll
+      for (uint32_t i = 0; i < kPairsPerThread; i++) {
+        const uint32_t q = tid + i * kTransThreads, xp = q / kOutPerRow, yv = q % kOutPerRow;
+        if (kPairs % kTransThreads != 0 && q >= kPairs) break;
+        uint32_t w[8];
+#pragma unroll
+        for (uint32_t e = 0; e < 8; e++) w[e] = *reinterpret_cast<const uint32_t*>(lds + (yv * 8 + e) * kPitchBytes + xp * 4u);
+        u32x4 lo, hi;
+#pragma unroll
+        for (uint32_t p = 0; p < 4; p++) {
+          lo[p] = (w[2 * p] & 0xffffu) | (w[2 * p + 1] << 16);
+          hi[p] = (w[2 * p] >> 16) | (w[2 * p + 1] & 0xffff0000u);
+        }
+        const uint64_t d0 = dst + (uint64_t)((int64_t)(2 * xp) * dst_pitch) + yv * 16u;
+        st_stream<u32x4_any>(d0, lo);
+        st_stream<u32x4_any>(d0 + (uint64_t)dst_pitch, hi);
+      }
+      return;
+    }
+#pragma unroll
+    for (uint32_t i = 0; i < kPerThread; i++) {
+      const uint32_t q = tid + i * kTransThreads, x = q / kOutPerRow, yv = q % kOutPerRow;
+      if (!kExact && q >= kVecs) break;
+      Pack<E, kV> out;
+#pragma unroll
+      for (uint32_t e = 0; e < kV; e++)
+        out.set(e, *reinterpret_cast<const E*>(lds + (yv * kV + e) * kPitchBytes + x * kEs));
+      out.store(dst + (uint64_t)((int64_t)x * dst_pitch) + yv * 16u);
+    }
+  }
+};
+
 template <typename E, uint32_t DX, uint32_t DY>
 __device__ __forceinline__ void transpose_full(uint64_t src, int64_t src_pitch, uint64_t dst, int64_t dst_pitch,
                                                uint8_t* __restrict__ lds) {
   // src: DY rows (index y) of DX elements contiguous along x.  dst: DX rows (index x) of DY elements along y.
-  constexpr uint32_t kEs = sizeof(E), kV = 16 / kEs, kVecPerRow = DX / kV, kOutPerRow = DY / kV;
-  constexpr uint32_t kPitchBytes = trans_pitch(DX, kEs) * kEs;  // a multiple of 4
-  constexpr uint32_t kVecs = DY * kVecPerRow, kPerThread = (kVecs + kTransThreads - 1) / kTransThreads;
-  constexpr bool kExact = kVecs % kTransThreads == 0;
-  const uint32_t tid = threadIdx.x;
-  u32x4 v[kPerThread];
-#pragma unroll
-  for (uint32_t i = 0; i < kPerThread; i++) {
-    const uint32_t q = tid + i * kTransThreads, y = q / kVecPerRow, xv = q % kVecPerRow;
-    if (kExact || q < kVecs) v[i] = ld_stream<u32x4_any>(src + (uint64_t)((int64_t)y * src_pitch) + xv * 16u);
-  }
-#pragma unroll
-  for (uint32_t i = 0; i < kPerThread; i++) {
-    const uint32_t q = tid + i * kTransThreads, y = q / kVecPerRow, xv = q % kVecPerRow;
-    if (!kExact && q >= kVecs) break;
-    uint32_t* row = reinterpret_cast<uint32_t*>(lds + y * kPitchBytes + xv * 16u);
-    row[0] = v[i][0];
-    row[1] = v[i][1];
-    row[2] = v[i][2];
-    row[3] = v[i][3];
-  }
+  typedef TransBlock<E, DX, DY> B;
+  u32x4 v[B::kPerThread];
+  B::load(v, src, src_pitch);
+  B::park(v, lds);
   __syncthreads();
-  if constexpr (kEs == 2) {
-    // two destination rows at a time: the 32-bit words of 8 source rows hold the elements of columns x and x + 1
-    constexpr uint32_t kPairs = kVecs / 2, kPairsPerThread = (kPairs + kTransThreads - 1) / kTransThreads;
+  B::emit(lds, dst, dst_pitch);
+}
+
+// A block of P * DX x DY elements: every load is issued first, then the P column panels of DX elements go
+// through LDS one after the other.  Both global sides then move runs of P * DX and DY elements while LDS holds
+// one panel only.
+template <typename E, uint32_t DX, uint32_t DY, uint32_t P>
+__device__ __forceinline__ void transpose_panels(uint64_t src, int64_t src_pitch, uint64_t dst, int64_t dst_pitch,
+                                                 uint8_t* __restrict__ lds) {
+  typedef TransBlock<E, DX, DY> B;
+  static_assert(B::kExact, "a panel is a whole number of vectors per work-item");
+  u32x4 v[P][B::kPerThread];
 #pragma unroll
-    for (uint32_t i = 0; i < kPairsPerThread; i++) {
-      const uint32_t q = tid + i * kTransThreads, xp = q / kOutPerRow, yv = q % kOutPerRow;
-      if (kPairs % kTransThreads != 0 && q >= kPairs) break;
-      uint32_t w[8];
+  for (uint32_t h = 0; h < P; h++) B::load(v[h], src + h * DX * sizeof(E), src_pitch);
 #pragma unroll
-      for (uint32_t e = 0; e < 8; e++) w[e] = *reinterpret_cast<const uint32_t*>(lds + (yv * 8 + e) * kPitchBytes + xp * 4u);
-      u32x4 lo, hi;
-#pragma unroll
-      for (uint32_t p = 0; p < 4; p++) {
-        lo[p] = (w[2 * p] & 0xffffu) | (w[2 * p + 1] << 16);
-        hi[p] = (w[2 * p] >> 16) | (w[2 * p + 1] & 0xffff0000u);
-      }
-      const uint64_t d0 = dst + (uint64_t)((int64_t)(2 * xp) * dst_pitch) + yv * 16u;
-      st_stream<u32x4_any>(d0, lo);
-      st_stream<u32x4_any>(d0 + (uint64_t)dst_pitch, hi);
-    }
-    return;
-  }
-#pragma unroll
-  for (uint32_t i = 0; i < kPerThread; i++) {
-    const uint32_t q = tid + i * kTransThreads, x = q / kOutPerRow, yv = q % kOutPerRow;
-    if (!kExact && q >= kVecs) break;
-    Pack<E, kV> out;
-#pragma unroll
-    for (uint32_t e = 0; e < kV; e++)
-      out.set(e, *reinterpret_cast<const E*>(lds + (yv * kV + e) * kPitchBytes + x * kEs));
-    out.store(dst + (uint64_t)((int64_t)x * dst_pitch) + yv * 16u);
+  for (uint32_t h = 0; h < P; h++) {
+    if (h) __syncthreads();
+    B::park(v[h], lds);
+    __syncthreads();
+    B::emit(lds, dst + (uint64_t)((int64_t)(h * DX) * dst_pitch), dst_pitch);
   }
 }
 
@@ -604,6 +652,13 @@ __device__ __forceinline__ void transpose_block(const TransTile& t, uint8_t* __r
   const uint64_t src = REV ? t.b : t.a, dst = REV ? t.a : t.b;
   const int64_t src_pitch = REV ? t.b_pitch : t.a_pitch, dst_pitch = REV ? t.a_pitch : t.b_pitch;
   const uint32_t nx = REV ? t.nk : t.nj, ny = REV ? t.nj : t.nk;
+  constexpr uint32_t kP = trans_panels(sizeof(E));
+  if constexpr (kP > 1) {
+    if (nx == kDX * kP && ny == kDY * kP) {  // a wide block
+      transpose_panels<E, kDX, kDY * kP, kP>(src, src_pitch, dst, dst_pitch, lds);
+      return;
+    }
+  }
   if (nx == kDX && ny == kDY)
     transpose_full<E, kDX, kDY>(src, src_pitch, dst, dst_pitch, lds);
   else
@@ -1076,7 +1131,10 @@ class PairCompiler {
     int64_t pos[ETHA_MAX_NDIM] = {0};
     uint64_t off_a = 0, off_b = 0;
     const int64_t kDimJ = (int64_t)trans_dim_a((uint32_t)esa_), kDimK = (int64_t)trans_dim_b((uint32_t)esa_);
-    const int64_t nbj = (n_[j] + kDimJ - 1) / kDimJ, nbk = (n_[kk] + kDimK - 1) / kDimK;
+    // the part of the chunk that whole wide blocks cover; blocks of the plain extent (and edge blocks) cover the rest
+    const int64_t kP = (int64_t)trans_panels((uint32_t)esa_);
+    const int64_t wide_j = kP > 1 ? n_[j] / (kDimJ * kP) * (kDimJ * kP) : 0, wide_k = kP > 1 ? n_[kk] / (kDimK * kP) * (kDimK * kP) : 0;
+    const bool wide = wide_j > 0 && wide_k > 0;
     do {
       // Launch order.  Blocks are grouped into super-blocks of S x S blocks that are emitted together: blocks
       // that are neighbours along j read neighbouring pieces of the same source rows, neighbours along k write
@@ -1084,26 +1142,33 @@ class PairCompiler {
       // open on both sides.  Super-blocks follow diagonals of their grid: row-major order would make everything
       // in flight read (or write) one narrow column stripe of rows that lie a power of two apart, i.e. the same
       // few memory channels.
-      const int64_t S = ETHA_TRANS_SUPER;
-      const int64_t nsj = (nbj + S - 1) / S, nsk = (nbk + S - 1) / S;
-      for (int64_t d = 0; d < nsk; d++)
-        for (int64_t sj = 0; sj < nsj; sj++)
-          for (int64_t ij = 0; ij < S; ij++)
-            for (int64_t ik = 0; ik < S; ik++) {
-          const int64_t bj = sj * S + ij, bk = ((sj + d) % nsk) * S + ik;
-          if (bj >= nbj || bk >= nbk) continue;
-          const int64_t j0 = bj * kDimJ, k0 = bk * kDimK;
-          TransTile t;
-          memset(&t, 0, sizeof(t));
-          t.a = A_.base + off_a + (uint64_t)(j0 * sa_[j]) + (uint64_t)(k0 * sa_[kk]);
-          t.b = B_.base + off_b + (uint64_t)(j0 * sb_[j]) + (uint64_t)(k0 * sb_[kk]);
-          t.a_pitch = sa_[kk];
-          t.b_pitch = sb_[j];
-          t.nj = (uint32_t)(n_[j] - j0 < kDimJ ? n_[j] - j0 : kDimJ);
-          t.nk = (uint32_t)(n_[kk] - k0 < kDimK ? n_[kk] - k0 : kDimK);
-          t.es_log2 = (uint32_t)log2u((uint64_t)esa_);
-          bld_.trans.push_back(t);
-        }
+      auto emit = [&](int64_t dim_j, int64_t dim_k, int64_t j_end, int64_t k_end, int64_t skip_j, int64_t skip_k) {
+        // blocks of dim_j x dim_k over [0, j_end) x [0, k_end), except those inside [0, skip_j) x [0, skip_k)
+        const int64_t S = ETHA_TRANS_SUPER;
+        const int64_t nbj = (j_end + dim_j - 1) / dim_j, nbk = (k_end + dim_k - 1) / dim_k;
+        const int64_t nsj = (nbj + S - 1) / S, nsk = (nbk + S - 1) / S;
+        for (int64_t d = 0; d < nsk; d++)
+          for (int64_t sj = 0; sj < nsj; sj++)
+            for (int64_t ij = 0; ij < S; ij++)
+              for (int64_t ik = 0; ik < S; ik++) {
+                const int64_t bj = sj * S + ij, bk = ((sj + d) % nsk) * S + ik;
+                if (bj >= nbj || bk >= nbk) continue;
+                const int64_t j0 = bj * dim_j, k0 = bk * dim_k;
+                if (j0 < skip_j && k0 < skip_k) continue;
+                TransTile t;
+                memset(&t, 0, sizeof(t));
+                t.a = A_.base + off_a + (uint64_t)(j0 * sa_[j]) + (uint64_t)(k0 * sa_[kk]);
+                t.b = B_.base + off_b + (uint64_t)(j0 * sb_[j]) + (uint64_t)(k0 * sb_[kk]);
+                t.a_pitch = sa_[kk];
+                t.b_pitch = sb_[j];
+                t.nj = (uint32_t)(j_end - j0 < dim_j ? j_end - j0 : dim_j);
+                t.nk = (uint32_t)(k_end - k0 < dim_k ? k_end - k0 : dim_k);
+                t.es_log2 = (uint32_t)log2u((uint64_t)esa_);
+                bld_.trans.push_back(t);
+              }
+      };
+      if (wide) emit(kDimJ * kP, kDimK * kP, wide_j, wide_k, 0, 0);
+      if (!wide || wide_j < n_[j] || wide_k < n_[kk]) emit(kDimJ, kDimK, n_[j], n_[kk], wide ? wide_j : 0, wide ? wide_k : 0);
       const int rc = check_size();
       if (rc != ETHA_OK) return rc;
     } while (next_position(k_, pos, &off_a, &off_b, j, kk));

@@ -527,6 +527,23 @@ def test_transposed_parents_small(gpu_device, dtype, target_transposed):
     assert (recv.n_trans_tiles > 0) == target_transposed
 
 
+@pytest.mark.parametrize("target_transposed", [False, True])
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16, torch.int16])
+def test_transposed_parents_wide_blocks(gpu_device, dtype, target_transposed):
+    """Shards of 2-byte elements large enough for 256 x 256 blocks (each loaded whole, then staged through LDS in
+    two panels), with 128 x 128 blocks and edge blocks around them, against the oracle."""
+    specs, targets, _ = workloads.transposed_parents(n_tensors=2, n=1576, dtype=dtype, target_transposed=target_transposed)
+    for s in specs:
+        s.dist = "bits"
+    job, _ = gpu_vs_oracle(specs, gpu_device, 4 * 1024 * 1024, target_ranks=targets)
+    assert not job.source_locals[0][0].is_contiguous()
+    for b in job.send_buckets.values():
+        tiles = job.wire.plan(b).send_table.trans_tiles()
+        wide = (tiles["nj"] == 256) & (tiles["nk"] == 256)
+        full = (tiles["nj"] == 128) & (tiles["nk"] == 128)
+        assert wide.any() and full.any() and (~wide & ~full).any()
+
+
 def test_transposed_parents_full_size_properties(gpu_device):
     """16 bf16 [8192, 8192] weights handed over as ``.t()`` views: every target shard equals its slice of the
     global tensor, the (non-contiguous) sources are unchanged."""

@@ -323,6 +323,45 @@ def test_short_pieces_of_one_row_are_gathered_in_an_ordered_range(rows, cols, bl
     assert np.array_equal(results[0], results[1])
 
 
+def test_large_transposed_chunk_of_2_byte_elements_uses_wide_blocks():
+    """Where 256 x 256 blocks fit, a transposing chunk of 2-byte elements is covered by them (runs of 512 bytes on
+    both sides); 128 x 128 blocks and element-wise edge blocks cover the rest, every byte exactly once."""
+    rows, cols, es, dt = 720, 540, 2, nat.BF16
+    arena = HostArena(3 * rows * cols * es + 65536)
+    t = arena.alloc(rows * cols * es)
+    arena.bytes_at(t, rows * cols * es)[:] = rs.randint(0, 256, rows * cols * es)
+    nj, nk = 700, 530
+    b = arena.alloc(nj * nk * es)
+    start, cshape, strides = (5, 3), (nj, nk), (1, rows)
+    d = _mk_desc(t, t, t + rows * cols * es, b, b, b + nj * nk * es, start, cshape, strides, dt, dt)
+    table = nat.Table.create(d.reshape(1), upload=False)
+    tiles = table.trans_tiles()
+    wide = (tiles["nj"] == 256) & (tiles["nk"] == 256)
+    full = (tiles["nj"] == 128) & (tiles["nk"] == 128)
+    assert int(wide.sum()) == (nj // 256) * (nk // 256) == 4
+    assert int(full.sum()) == (nj // 128) * (nk // 128) - 16 == 4  # whole 128-blocks outside the 512 x 512 wide part
+    assert int((~wide & ~full).sum()) == 6 * 5 - (nj // 128) * (nk // 128) == 10 and np.all(tiles["nj"][~wide] <= 128) and np.all(tiles["nk"][~wide] <= 128)
+    for direction in ("pack", "unpack"):
+        arena.writes[:] = 0
+        if direction == "unpack":
+            arena.bytes_at(t, rows * cols * es)[:] = 0
+        before = arena.bytes_at(t, rows * cols * es).copy()
+        execute(table, arena, direction)
+        assert arena.writes.max() == 1 and int(arena.writes.sum()) == nj * nk * es
+        if direction == "pack":
+            want = np.zeros(nj * nk * es, dtype=np.uint8)
+            scratch = np.zeros(nj * nk * es, dtype=np.uint8)
+            oc = co.make_chunk(t, start, cshape, strides, dt, dt, bucket_off=0)
+            assert co.lib().oracle_pack_bucket(oc, 1, want.ctypes.data, scratch.ctypes.data) == 0
+            assert np.array_equal(arena.bytes_at(b, nj * nk * es), want)
+            assert np.array_equal(arena.bytes_at(t, rows * cols * es), before)
+        else:
+            want2 = before.copy()
+            oc2 = co.make_chunk(want2.ctypes.data, start, cshape, strides, dt, dt, bucket_off=0)
+            assert co.lib().oracle_unpack_bucket(oc2, 1, want.ctypes.data, scratch.ctypes.data) == 0
+            assert np.array_equal(arena.bytes_at(t, rows * cols * es), want2)
+
+
 @pytest.mark.parametrize("dt", [nat.B8, nat.BF16, nat.F32, nat.B64])
 def test_transposed_parent_uses_lds_blocks(dt):
     """A chunk of a transposed view: the tensor side is contiguous along dim 0, the bucket along dim 1."""
