@@ -119,20 +119,18 @@ constexpr uint32_t kTransThreads = ETHA_TRANS_THREADS;
 // 8-byte elements, which keeps the LDS footprint of a block at 16-66 KB
 __host__ __device__ constexpr uint32_t trans_dim_a(uint32_t es) { return es == 8 ? ETHA_TRANS_DIM_A / 2u : (uint32_t)ETHA_TRANS_DIM_A; }
 __host__ __device__ constexpr uint32_t trans_dim_b(uint32_t es) { return es == 8 ? ETHA_TRANS_DIM_B / 2u : (uint32_t)ETHA_TRANS_DIM_B; }
-// Where a chunk is large enough, blocks are kTransPanels(es) times that extent on both sides ("wide" blocks):
-// a 128-element side of 2-byte elements is a run of only 256 bytes, and runs of 512 bytes move faster.  A wide
-// block is loaded whole into registers and goes through LDS one panel of trans_dim columns at a time, so LDS
-// holds a panel, not the block.
-#ifndef ETHA_TRANS_PANELS
-#define ETHA_TRANS_PANELS 2
-#endif
-__host__ __device__ constexpr uint32_t trans_panels(uint32_t es) { return es == 2 ? (uint32_t)ETHA_TRANS_PANELS : 1u; }
+// Where a chunk is large enough, blocks are trans_wide(es) times that extent on both sides ("wide" blocks): a
+// 128-element side of 1- or 2-byte elements is a run of only 128 or 256 bytes, and longer runs move faster
+// (2-byte elements 5.9 -> 6.1-6.7 TB/s, 1-byte elements 5.1 -> 6.0-6.2).  A wide block is loaded whole into
+// registers and goes through LDS in trans_panels(es) panels of columns, so LDS holds a panel, not the block.
+__host__ __device__ constexpr uint32_t trans_wide(uint32_t es) { return es <= 2 ? 2u : 1u; }
+__host__ __device__ constexpr uint32_t trans_panels(uint32_t es) { return es == 2 ? 2u : 1u; }
 __host__ __device__ constexpr uint32_t trans_pitch(uint32_t dim, uint32_t es) {  // LDS row pitch in elements: an odd number of words
   return dim + (es >= 4 ? 1u : 4u / es);
 }
-__host__ __device__ constexpr uint32_t trans_lds_bytes(uint32_t es) {  // either direction: rows of one side (of a wide block, if any), one row per element of the other
-  const uint32_t p = trans_panels(es);
-  const uint32_t fwd = p * trans_dim_b(es) * trans_pitch(trans_dim_a(es), es) * es, rev = p * trans_dim_a(es) * trans_pitch(trans_dim_b(es), es) * es;
+__host__ __device__ constexpr uint32_t trans_lds_bytes(uint32_t es) {  // either direction: rows of one side (one panel of a wide block), one row per element of the other
+  const uint32_t w = trans_wide(es), p = trans_panels(es);
+  const uint32_t fwd = w * trans_dim_b(es) * trans_pitch(w * trans_dim_a(es) / p, es) * es, rev = w * trans_dim_a(es) * trans_pitch(w * trans_dim_b(es) / p, es) * es;
   return fwd > rev ? fwd : rev;
 }
 
@@ -580,6 +578,33 @@ struct TransBlock {
       }
       return;
     }
+    if constexpr (kEs == 1) {
+      // four destination rows at a time: the 32-bit words of 16 source rows hold the bytes of columns x .. x + 3
+      constexpr uint32_t kQuads = kVecs / 4, kQuadsPerThread = (kQuads + kTransThreads - 1) / kTransThreads;
+#pragma unroll
+      for (uint32_t i = 0; i < kQuadsPerThread; i++) {
+        const uint32_t q = tid + i * kTransThreads, xq = q / kOutPerRow, yv = q % kOutPerRow;
+        if (kQuads % kTransThreads != 0 && q >= kQuads) break;
+        u32x4 col[4];
+#pragma unroll
+        for (uint32_t p = 0; p < 4; p++) {
+          uint32_t w[4];
+#pragma unroll
+          for (uint32_t e = 0; e < 4; e++) w[e] = *reinterpret_cast<const uint32_t*>(lds + (yv * 16 + p * 4 + e) * kPitchBytes + xq * 4u);
+          // 4 x 4 byte transposition; selector bytes 0-3 pick from the second operand, 4-7 from the first
+          const uint32_t a = __builtin_amdgcn_perm(w[1], w[0], 0x05010400u), b = __builtin_amdgcn_perm(w[1], w[0], 0x07030602u);
+          const uint32_t c = __builtin_amdgcn_perm(w[3], w[2], 0x05010400u), d = __builtin_amdgcn_perm(w[3], w[2], 0x07030602u);
+          col[0][p] = __builtin_amdgcn_perm(c, a, 0x05040100u);
+          col[1][p] = __builtin_amdgcn_perm(c, a, 0x07060302u);
+          col[2][p] = __builtin_amdgcn_perm(d, b, 0x05040100u);
+          col[3][p] = __builtin_amdgcn_perm(d, b, 0x07060302u);
+        }
+        const uint64_t d0 = dst + (uint64_t)((int64_t)(4 * xq) * dst_pitch) + yv * 16u;
+#pragma unroll
+        for (uint32_t c = 0; c < 4; c++) st_stream<u32x4_any>(d0 + (uint64_t)((int64_t)c * dst_pitch), col[c]);
+      }
+      return;
+    }
 #pragma unroll
     for (uint32_t i = 0; i < kPerThread; i++) {
       const uint32_t q = tid + i * kTransThreads, x = q / kOutPerRow, yv = q % kOutPerRow;
@@ -652,10 +677,10 @@ __device__ __forceinline__ void transpose_block(const TransTile& t, uint8_t* __r
   const uint64_t src = REV ? t.b : t.a, dst = REV ? t.a : t.b;
   const int64_t src_pitch = REV ? t.b_pitch : t.a_pitch, dst_pitch = REV ? t.a_pitch : t.b_pitch;
   const uint32_t nx = REV ? t.nk : t.nj, ny = REV ? t.nj : t.nk;
-  constexpr uint32_t kP = trans_panels(sizeof(E));
-  if constexpr (kP > 1) {
-    if (nx == kDX * kP && ny == kDY * kP) {  // a wide block
-      transpose_panels<E, kDX, kDY * kP, kP>(src, src_pitch, dst, dst_pitch, lds);
+  constexpr uint32_t kW = trans_wide(sizeof(E)), kP = trans_panels(sizeof(E));
+  if constexpr (kW > 1) {
+    if (nx == kDX * kW && ny == kDY * kW) {  // a wide block
+      transpose_panels<E, kDX * kW / kP, kDY * kW, kP>(src, src_pitch, dst, dst_pitch, lds);
       return;
     }
   }
@@ -1132,7 +1157,7 @@ class PairCompiler {
     uint64_t off_a = 0, off_b = 0;
     const int64_t kDimJ = (int64_t)trans_dim_a((uint32_t)esa_), kDimK = (int64_t)trans_dim_b((uint32_t)esa_);
     // the part of the chunk that whole wide blocks cover; blocks of the plain extent (and edge blocks) cover the rest
-    const int64_t kP = (int64_t)trans_panels((uint32_t)esa_);
+    const int64_t kP = (int64_t)trans_wide((uint32_t)esa_);
     const int64_t wide_j = kP > 1 ? n_[j] / (kDimJ * kP) * (kDimJ * kP) : 0, wide_k = kP > 1 ? n_[kk] / (kDimK * kP) * (kDimK * kP) : 0;
     const bool wide = wide_j > 0 && wide_k > 0;
     do {

@@ -528,10 +528,10 @@ def test_transposed_parents_small(gpu_device, dtype, target_transposed):
 
 
 @pytest.mark.parametrize("target_transposed", [False, True])
-@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16, torch.int16])
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16, torch.int16, torch.int8])
 def test_transposed_parents_wide_blocks(gpu_device, dtype, target_transposed):
-    """Shards of 2-byte elements large enough for 256 x 256 blocks (each loaded whole, then staged through LDS in
-    two panels), with 128 x 128 blocks and edge blocks around them, against the oracle."""
+    """Shards of 1- and 2-byte elements large enough for 256 x 256 blocks (each loaded whole, then staged through
+    LDS in one or two panels), with 128 x 128 blocks and edge blocks around them, against the oracle."""
     specs, targets, _ = workloads.transposed_parents(n_tensors=2, n=1576, dtype=dtype, target_transposed=target_transposed)
     for s in specs:
         s.dist = "bits"
