@@ -123,7 +123,7 @@ typedef struct EthaTableInfo {
   uint32_t tile_threads;  /* units (work-items) per tile; one tile = tile_threads / 64 workgroups of one wavefront */
   uint64_t device_bytes;  /* device memory held by the table */
   uint64_t payload_bytes; /* sum over chunks of numel * wire element size */
-  uint32_t n_trans_tiles; /* square blocks (32-128 elements a side) of transposing chunks, staged through LDS */
+  uint32_t n_trans_tiles; /* square blocks (up to 64-256 elements a side, by element size) of transposing chunks, staged through LDS */
   uint32_t reserved;
 } EthaTableInfo;
 
