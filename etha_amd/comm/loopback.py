@@ -436,9 +436,9 @@ class LoopbackWire:
         return [repr(p) for p in self._programs]
 
     def emit(self, plan, indices: list[int], merge: bool = False) -> None:
-        """Issue steps ``indices`` of ``plan``.  They became ready in the same phase of one pipeline sweep, so they
-        are independent of each other; with ``merge`` those that are neighbours in their table share a launch.
-        Each launch is ordered against earlier launches only where their bytes meet."""
+        """Issue steps ``indices`` of ``plan``, which became ready in the same phase of one pipeline sweep; with
+        ``merge`` those that are neighbours in their table and touch no allocation that the other writes share a
+        launch.  Each launch is ordered against earlier launches only where their bytes meet."""
         todo = []
         for i in indices:
             kind, first, count, _ = plan.steps[i]
@@ -450,7 +450,9 @@ class LoopbackWire:
             runs = [todo[0]]
             for t in todo[1:]:
                 last = runs[-1]
-                if t[0] == last[0] and last[1] + last[2] == t[1]:
+                # steps of one phase are independent except LOCAL buckets inside one tensor, where a later bucket
+                # may read what an earlier one writes: those keep their own launches, in list order
+                if t[0] == last[0] and last[1] + last[2] == t[1] and last[4].isdisjoint(t[3]) and last[3].isdisjoint(t[4]):
                     last[2] += t[2]
                     last[3], last[4], last[5] = last[3] | t[3], last[4] | t[4], last[5] | t[5]
                     last.append(True)  # covers several buckets

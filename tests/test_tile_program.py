@@ -578,3 +578,13 @@ def test_self_copy_buckets_that_feed_each_other_are_not_merged():
     for kind, first, count, _ in plan.merged_steps:
         execute(plan.local_table, mem, "selfcopy", first, count)
     assert torch.equal(t, want)
+    # the ring pipeline with merged launches: both buckets become ready in one sweep, and still get a launch each,
+    # the second one in stream order behind the first
+    from etha_amd.comm import bucket_comm
+
+    wire = LoopbackWire("cpu", host_inspection=True, pool="ring")
+    log = wire.launch_log = []
+    wire.on_launch = lambda *a: None
+    bucket_comm(buckets, wire=wire, merge_launches=True, synchronize=False)
+    assert [(kind, count) for kind, _, count, _ in log] == [("selfcopy", 1), ("selfcopy", 1)]
+    assert log[1][3] == 0 and log[0][1] < log[1][1]
