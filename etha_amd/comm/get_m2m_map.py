@@ -191,9 +191,8 @@ def get_m2m_map(
     target_placements = tuple(target_placements)
     if any(isinstance(p, Partial) for p in target_placements):
         raise NotImplementedError(
-            f"Partial placement in target_placements={target_placements} is not supported. "
-            "Cross-process-group decomposition of a logical tensor into a Partial "
-            "contribution is not uniquely defined; only source-side Partial is supported."
+            f"target_placements={target_placements} contains Partial: how a tensor would be split into partial "
+            "contributions across two process groups has no single answer, so Partial can only appear on the source side."
         )
     src_mesh = _as_rank_array(source_mesh)
     tgt_mesh = _as_rank_array(target_mesh)

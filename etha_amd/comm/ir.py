@@ -31,7 +31,7 @@ REDUCE_OPS = ("sum", "avg", "max", "min", "product")  # ir.py:51-57
 
 @dataclass(frozen=True)
 class Endpoint:
-    """A chunk location: a rank and its cell (multi-index) in the transfer grid."""
+    """Where a chunk lives: the owning rank and the multi-index of its cell in the lcm grid of the transfer."""
 
     rank: int
     cell: tuple[int, ...]
@@ -104,7 +104,7 @@ class PartialGroup:
 
 @dataclass(kw_only=True, eq=False)
 class Chunk:
-    """A shape-dependent transfer descriptor: one tensor region plus its role."""
+    """Descriptor of one region of one tensor and of what this rank does with it (send, receive, both, or reduce only)."""
 
     transport: Transport
     is_source: bool

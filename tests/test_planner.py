@@ -50,7 +50,7 @@ def test_partial_shadows_reach_the_whole_component():
     assert shipping == [(0, [6]), (1, [7])]
     shadows = sorted(r.src.rank for r in m.routes if r.kind == Transport.NONE)
     assert shadows == [2, 3, 4, 5]
-    with pytest.raises(NotImplementedError, match="Partial placement in target"):
+    with pytest.raises(NotImplementedError, match="contains Partial"):
         get_m2m_map([0, 1], (Shard(0),), [2, 3], (Partial(),))
 
 
