@@ -517,6 +517,26 @@ __global__ __launch_bounds__(ETHA_BLOCK_THREADS) void etha_gather_kernel(const A
   tile_body<true, true>(nullptr, 0u, row, gather, tile, piece * kBlockThreads + threadIdx.x);
 }
 
+// An unpack range with both kinds of tile in one launch: the plain tiles first, then (from the next multiple of
+// 128 workgroups on, which keeps the dealing above) the gather tiles.  One launch instead of two that run side by
+// side: two kernels in flight interleave their address streams, and the gather part of a range is short.
+__global__ __launch_bounds__(ETHA_BLOCK_THREADS) void etha_unpack_mixed_kernel(const RunTile* __restrict__ run_tiles,
+                                                                                const RowTile* __restrict__ row_tiles,
+                                                                                const uint64_t* __restrict__ gather,
+                                                                                uint32_t n_run, uint32_t n_plain,
+                                                                                uint32_t n_gather) {
+  const uint32_t w = blockIdx.x, plain_groups = n_plain * kBlocksPerTile;
+  if (w < plain_groups) {
+    tile_body<true>(run_tiles, n_run, row_tiles, gather, w / kBlocksPerTile, (w % kBlocksPerTile) * kBlockThreads + threadIdx.x);
+    return;
+  }
+  const uint32_t base = (plain_groups + 127u) & ~127u;
+  if (w < base) return;
+  const uint32_t g = w - base, tile = ((g >> 7) << 3) + (g & 7u), piece = (g & 127u) >> 3;
+  if (tile >= n_gather) return;
+  tile_body<true, true>(nullptr, 0u, row_tiles + (n_plain - n_run), gather, tile, piece * kBlockThreads + threadIdx.x);
+}
+
 // ---- transposing chunks: staged through LDS -----------------------------------------------------
 // The a side is contiguous along j, the b side along k.  A full block of D x D elements is read with 16-byte
 // vectors along the source's contiguous dim (consecutive work-items cover one row, then the next row),
@@ -1591,12 +1611,16 @@ int launch_tiles(const EthaTable* t, uint32_t first, uint32_t count, void* strea
     flags |= ETHA_LAUNCH_UNORDERED;  // the two kernels of one call touch different chunks
   }
   const Seg2D g = tile_range(t, first, count, REV);
-  if (g.n_tiles) {
-    launch_plain(g, REV, stream, flags);
-    flags |= ETHA_LAUNCH_UNORDERED;
-  }
   const Seg2D gathered = gather_range(t, first, count, REV);
-  if (gathered.n_tiles) launch_gather(&gathered, 1, gathered.n_tiles, stream, flags);
+  if (g.n_tiles && gathered.n_tiles) {  // the gather tiles follow the plain row tiles in the ordered copy
+    const uint32_t groups = ((g.n_tiles * kBlocksPerTile + 127u) & ~127u) + gather_grid(gathered.n_tiles);
+    launch_kernel(etha_unpack_mixed_kernel, dim3(groups), dim3(kBlockThreads), 0, stream, flags, g.run, g.row, g.gather, g.n_run,
+                  g.n_tiles, gathered.n_tiles);
+  } else if (g.n_tiles) {
+    launch_plain(g, REV, stream, flags);
+  } else if (gathered.n_tiles) {
+    launch_gather(&gathered, 1, gathered.n_tiles, stream, flags);
+  }
   HIP_TRY(hipGetLastError());
   return ETHA_OK;
 }
