@@ -66,7 +66,7 @@ ROW_TILE = np.dtype(
     ]
 )
 TRANS_TILE = np.dtype([("a", "<u8"), ("b", "<u8"), ("a_pitch", "<i8"), ("b_pitch", "<i8"), ("nj", "<u4"), ("nk", "<u4"),
-                       ("es_log2", "<u4"), ("pad", "<u4")])
+                       ("es_log2", "<u4"), ("cvt", "<u4")])
 assert RUN_TILE.itemsize == 24 and ROW_TILE.itemsize == 64 and TRANS_TILE.itemsize == 48
 
 

@@ -95,8 +95,8 @@ struct TransTile {   // a 2-D block whose contiguous dim differs between the two
   int64_t a_pitch;   // bytes between consecutive k on the a side
   int64_t b_pitch;   // bytes between consecutive j on the b side
   uint32_t nj, nk;   // extent of the block (<= trans_dim(element size) each)
-  uint32_t es_log2;  // log2 of the element size in bytes
-  uint32_t pad;
+  uint32_t es_log2;  // log2 of the element size in bytes (of the b side, when the block converts)
+  uint32_t cvt;      // 0: same element type on both sides; else (dtype of a << 4) | dtype of b: a holds f32, b f16 or bf16
 };
 static_assert(sizeof(TransTile) == 48, "TransTile layout");
 // A transposing block is D x D elements, handled by one workgroup of kTransThreads work-items.  D is chosen
@@ -689,6 +689,107 @@ __device__ __forceinline__ void transpose_edge(uint64_t src, int64_t src_pitch, 
   }
 }
 
+// Transposing blocks that also convert: the a side holds f32, the b side (the bucket) f16 or bf16.  LDS holds the
+// 16-bit elements, so the staging is that of a 2-byte block: a pack converts while it parks (four f32 of a source
+// row become two words), an unpack while it emits (the eight elements of a gathered vector become two vectors).
+template <typename TB, uint32_t DX, uint32_t DY>
+__device__ __forceinline__ void transpose_cvt_pack(uint64_t src, int64_t src_pitch, uint64_t dst, int64_t dst_pitch,
+                                                   uint8_t* __restrict__ lds) {
+  // src: DY rows of DX f32 contiguous along x.  dst: DX rows of DY 16-bit elements.
+  typedef TransBlock<uint16_t, DX, DY> B;
+  constexpr uint32_t kVecPerRow = DX / 4, kVecs = DY * kVecPerRow, kPerThread = kVecs / kTransThreads;
+  static_assert(kVecs % kTransThreads == 0, "a whole number of f32 vectors per work-item");
+  const uint32_t tid = threadIdx.x;
+  u32x4 v[kPerThread];
+#pragma unroll
+  for (uint32_t i = 0; i < kPerThread; i++) {
+    const uint32_t q = tid + i * kTransThreads, y = q / kVecPerRow, xv = q % kVecPerRow;
+    v[i] = ld_stream<u32x4_any>(src + (uint64_t)((int64_t)y * src_pitch) + xv * 16u);
+  }
+#pragma unroll
+  for (uint32_t i = 0; i < kPerThread; i++) {
+    const uint32_t q = tid + i * kTransThreads, y = q / kVecPerRow, xv = q % kVecPerRow;
+    uint32_t h[4];
+#pragma unroll
+    for (uint32_t e = 0; e < 4; e++) h[e] = from_f32(TB(), to_f32(TagF32(), v[i][e]));
+    uint32_t* row = reinterpret_cast<uint32_t*>(lds + y * B::kPitchBytes + xv * 8u);
+    row[0] = h[0] | (h[1] << 16);
+    row[1] = h[2] | (h[3] << 16);
+  }
+  __syncthreads();
+  B::emit(lds, dst, dst_pitch);
+}
+
+template <typename TB, uint32_t DX, uint32_t DY>
+__device__ __forceinline__ void transpose_cvt_unpack(uint64_t src, int64_t src_pitch, uint64_t dst, int64_t dst_pitch,
+                                                     uint8_t* __restrict__ lds) {
+  // src: DY rows of DX 16-bit elements contiguous along x.  dst: DX rows of DY f32.
+  typedef TransBlock<uint16_t, DX, DY> B;
+  u32x4 v[B::kPerThread];
+  B::load(v, src, src_pitch);
+  B::park(v, lds);
+  __syncthreads();
+  // two destination rows per work-item, four f32 (one vector) of each: the words of 4 source rows hold the elements
+  // of columns x and x + 1, and consecutive work-items write consecutive vectors of a destination row
+  constexpr uint32_t kQuadsPerRow = DY / 4, kItems = (DX / 2) * kQuadsPerRow, kItemsPerThread = (kItems + kTransThreads - 1) / kTransThreads;
+  const uint32_t tid = threadIdx.x;
+#pragma unroll
+  for (uint32_t i = 0; i < kItemsPerThread; i++) {
+    const uint32_t q = tid + i * kTransThreads, xp = q / kQuadsPerRow, y4 = q % kQuadsPerRow;
+    if (kItems % kTransThreads != 0 && q >= kItems) break;
+    u32x4 lo, hi;
+#pragma unroll
+    for (uint32_t e = 0; e < 4; e++) {
+      const uint32_t w = *reinterpret_cast<const uint32_t*>(lds + (y4 * 4 + e) * B::kPitchBytes + xp * 4u);
+      lo[e] = from_f32(TagF32(), to_f32(TB(), (uint16_t)(w & 0xffffu)));
+      hi[e] = from_f32(TagF32(), to_f32(TB(), (uint16_t)(w >> 16)));
+    }
+    const uint64_t d0 = dst + (uint64_t)((int64_t)(2 * xp) * dst_pitch) + y4 * 16u;
+    st_stream<u32x4_any>(d0, lo);
+    st_stream<u32x4_any>(d0 + (uint64_t)dst_pitch, hi);
+  }
+}
+
+template <typename TB, bool REV, uint32_t DX>
+__device__ __forceinline__ void transpose_cvt_edge(uint64_t src, int64_t src_pitch, uint32_t nx, uint64_t dst,
+                                                   int64_t dst_pitch, uint32_t ny, uint8_t* __restrict__ lds) {
+  // nx <= DX elements per source row, ny source rows; one element per access, 16-bit elements in LDS
+  constexpr uint32_t kPitchBytes = trans_pitch(DX, 2) * 2;
+  const uint32_t n = nx * ny;
+  for (uint32_t q = threadIdx.x; q < n; q += kTransThreads) {
+    const uint32_t y = q / nx, x = q - y * nx;
+    const uint64_t at = src + (uint64_t)((int64_t)y * src_pitch);
+    *reinterpret_cast<uint16_t*>(lds + y * kPitchBytes + x * 2u) =
+        REV ? ld_stream<uint16_t>(at + (uint64_t)x * 2u) : from_f32(TB(), to_f32(TagF32(), ld_stream<uint32_t>(at + (uint64_t)x * 4u)));
+  }
+  __syncthreads();
+  for (uint32_t q = threadIdx.x; q < n; q += kTransThreads) {
+    const uint32_t x = q / ny, y = q - x * ny;
+    const uint16_t h = *reinterpret_cast<const uint16_t*>(lds + y * kPitchBytes + x * 2u);
+    const uint64_t at = dst + (uint64_t)((int64_t)x * dst_pitch);
+    if (REV)
+      st_stream<uint32_t>(at + (uint64_t)y * 4u, from_f32(TagF32(), to_f32(TB(), h)));
+    else
+      st_stream<uint16_t>(at + (uint64_t)y * 2u, h);
+  }
+}
+
+template <typename TB, bool REV>
+__device__ __forceinline__ void transpose_block_cvt(const TransTile& t, uint8_t* __restrict__ lds) {
+  constexpr uint32_t kDX = REV ? trans_dim_b(2) : trans_dim_a(2), kDY = REV ? trans_dim_a(2) : trans_dim_b(2);
+  const uint64_t src = REV ? t.b : t.a, dst = REV ? t.a : t.b;
+  const int64_t src_pitch = REV ? t.b_pitch : t.a_pitch, dst_pitch = REV ? t.a_pitch : t.b_pitch;
+  const uint32_t nx = REV ? t.nk : t.nj, ny = REV ? t.nj : t.nk;
+  if (nx == kDX && ny == kDY) {
+    if constexpr (REV)
+      transpose_cvt_unpack<TB, kDX, kDY>(src, src_pitch, dst, dst_pitch, lds);
+    else
+      transpose_cvt_pack<TB, kDX, kDY>(src, src_pitch, dst, dst_pitch, lds);
+  } else {
+    transpose_cvt_edge<TB, REV, kDX>(src, src_pitch, nx, dst, dst_pitch, ny, lds);
+  }
+}
+
 template <typename E, bool REV>
 __device__ __forceinline__ void transpose_block(const TransTile& t, uint8_t* __restrict__ lds) {
   // pack (a -> b): source rows run along j (one row per k); unpack (b -> a): source rows run along k (one per j)
@@ -711,15 +812,27 @@ __device__ __forceinline__ void transpose_block(const TransTile& t, uint8_t* __r
 }
 
 template <bool REV>
+__device__ __forceinline__ void transpose_tile(const TransTile& t, uint8_t* __restrict__ lds) {
+  if (t.cvt) {  // f32 on the a side, f16 or bf16 on the b side
+    if ((t.cvt & 15u) == ETHA_F16)
+      transpose_block_cvt<TagF16, REV>(t, lds);
+    else
+      transpose_block_cvt<TagBF16, REV>(t, lds);
+    return;
+  }
+  switch (t.es_log2) {
+    case 0: transpose_block<uint8_t, REV>(t, lds); break;
+    case 1: transpose_block<uint16_t, REV>(t, lds); break;
+    case 2: transpose_block<uint32_t, REV>(t, lds); break;
+    default: transpose_block<uint64_t, REV>(t, lds); break;
+  }
+}
+
+template <bool REV>
 __global__ __launch_bounds__(ETHA_TRANS_THREADS) void etha_transpose_kernel(const TransTile* __restrict__ tiles) {
   extern __shared__ __attribute__((aligned(16))) uint8_t lds_bytes[];  // trans_lds_bytes(largest element size)
   const TransTile t = tiles[blockIdx.x];
-  switch (t.es_log2) {
-    case 0: transpose_block<uint8_t, REV>(t, lds_bytes); break;
-    case 1: transpose_block<uint16_t, REV>(t, lds_bytes); break;
-    case 2: transpose_block<uint32_t, REV>(t, lds_bytes); break;
-    default: transpose_block<uint64_t, REV>(t, lds_bytes); break;
-  }
+  transpose_tile<REV>(t, lds_bytes);
 }
 
 // several tables' transposing tiles in one launch: blockIdx.y picks the list, as in etha_tile_kernel_2d
@@ -740,12 +853,7 @@ __global__ __launch_bounds__(ETHA_TRANS_THREADS) void etha_transpose_kernel_2d(c
   typedef const __attribute__((address_space(1))) TransTile* GlobalTrans;
   const TransTile* tiles = (const TransTile*)(GlobalTrans)(((uint64_t)raw[1] << 32) | raw[0]);
   const TransTile t = tiles[blockIdx.x];
-  switch (t.es_log2) {
-    case 0: transpose_block<uint8_t, REV>(t, lds_bytes); break;
-    case 1: transpose_block<uint16_t, REV>(t, lds_bytes); break;
-    case 2: transpose_block<uint32_t, REV>(t, lds_bytes); break;
-    default: transpose_block<uint64_t, REV>(t, lds_bytes); break;
-  }
+  transpose_tile<REV>(t, lds_bytes);
 }
 
 // ---- Partial reduce-pack ------------------------------------------------------------------------
@@ -1167,7 +1275,9 @@ class PairCompiler {
   // kernel in blocks of trans_dim_a x trans_dim_b elements; all other dims are unrolled here.
   int try_transposing(bool* done) {
     *done = false;
-    if (!(run_elems_ == 1 && plain_ && k_ >= 2 && sb_[k_ - 1] == esb_ && sa_[k_ - 1] != esa_)) return ETHA_OK;
+    // same element type on both sides, or f32 on the a side with f16 / bf16 in the bucket (converted on the way)
+    const bool converting = cvt_ && red_.n_peers == 0 && dta_ == ETHA_F32 && (dtb_ == ETHA_F16 || dtb_ == ETHA_BF16);
+    if (!(run_elems_ == 1 && (plain_ || converting) && k_ >= 2 && sb_[k_ - 1] == esb_ && sa_[k_ - 1] != esa_)) return ETHA_OK;
     int j = -1;
     for (int i = 0; i < k_ - 1; i++)
       if (sa_[i] == esa_ && n_[i] >= 8) j = i;
@@ -1175,9 +1285,10 @@ class PairCompiler {
     if (j < 0 || n_[kk] < 8 || (A_.base % (uint64_t)esa_) != 0 || (B_.base % (uint64_t)esb_) != 0) return ETHA_OK;
     int64_t pos[ETHA_MAX_NDIM] = {0};
     uint64_t off_a = 0, off_b = 0;
-    const int64_t kDimJ = (int64_t)trans_dim_a((uint32_t)esa_), kDimK = (int64_t)trans_dim_b((uint32_t)esa_);
+    // blocks are sized by the element that goes through LDS: the b side's
+    const int64_t kDimJ = (int64_t)trans_dim_a((uint32_t)esb_), kDimK = (int64_t)trans_dim_b((uint32_t)esb_);
     // the part of the chunk that whole wide blocks cover; blocks of the plain extent (and edge blocks) cover the rest
-    const int64_t kP = (int64_t)trans_wide((uint32_t)esa_);
+    const int64_t kP = converting ? 1 : (int64_t)trans_wide((uint32_t)esb_);
     const int64_t wide_j = kP > 1 ? n_[j] / (kDimJ * kP) * (kDimJ * kP) : 0, wide_k = kP > 1 ? n_[kk] / (kDimK * kP) * (kDimK * kP) : 0;
     const bool wide = wide_j > 0 && wide_k > 0;
     do {
@@ -1208,7 +1319,8 @@ class PairCompiler {
                 t.b_pitch = sb_[j];
                 t.nj = (uint32_t)(j_end - j0 < dim_j ? j_end - j0 : dim_j);
                 t.nk = (uint32_t)(k_end - k0 < dim_k ? k_end - k0 : dim_k);
-                t.es_log2 = (uint32_t)log2u((uint64_t)esa_);
+                t.es_log2 = (uint32_t)log2u((uint64_t)esb_);
+                t.cvt = converting ? (dta_ << 4) | dtb_ : 0u;
                 bld_.trans.push_back(t);
               }
       };

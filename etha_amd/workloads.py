@@ -111,17 +111,24 @@ def moe_experts_row_parallel_w2(n_experts: int = 8, hidden: int = 4096, inter: i
     return specs, [0], 64 * MIB
 
 
-def transposed_parents(n_tensors: int = 16, n: int = 8192, dtype=torch.bfloat16, target_transposed: bool = False):
+def transposed_parents(n_tensors: int = 16, n: int = 8192, dtype=torch.bfloat16, target_transposed: bool = False,
+                       target_dtype=None):
     """16 bf16 [8192, 8192] weights whose source shards are ``.t()`` views (stored [in, out], handed over as
     [out, in]): mesh (4,) Shard(0) -> mesh (2,) Shard(0), one target rank.  The contiguous dim differs between
     shard and bucket, so every chunk goes through the LDS-staged transposing kernel."""
     src, tgt = _mesh(0, (4,)), _mesh(4, (2,))
     specs = [
-        TensorSpec(f"w{i}", (n, n), src, (Shard(0),), tgt, (Shard(0),), dtype, seed=i, source_layout="transposed",
+        TensorSpec(f"w{i}", (n, n), src, (Shard(0),), tgt, (Shard(0),), dtype, target_dtype, seed=i, source_layout="transposed",
                    target_layout="transposed" if target_transposed else "contiguous")
         for i in range(n_tensors)
     ]
     return specs, [4], 64 * MIB
+
+
+def transposed_parents_fp32_to_bf16():
+    """The same with fp32 ``.t()`` sources and bf16 targets (master weights kept [in, out] -> serving weights): the
+    transposing pack converts."""
+    return transposed_parents(dtype=torch.float32, target_dtype=torch.bfloat16)
 
 
 def llama3_8b_fsdp8_to_tp2_fp32_to_bf16():
@@ -139,4 +146,5 @@ WORKLOADS = {
     "moe_experts_and_uneven_vocab": moe_experts_and_uneven_vocab,
     "moe_experts_row_parallel_w2": moe_experts_row_parallel_w2,
     "transposed_parents": transposed_parents,
+    "transposed_parents_fp32_to_bf16": transposed_parents_fp32_to_bf16,
 }

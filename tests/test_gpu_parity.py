@@ -544,6 +544,28 @@ def test_transposed_parents_wide_blocks(gpu_device, dtype, target_transposed):
         assert wide.any() and full.any() and (~wide & ~full).any()
 
 
+@pytest.mark.parametrize("narrow", [torch.bfloat16, torch.float16])
+@pytest.mark.parametrize("direction", ["f32 .t() source -> 16-bit target", "16-bit source -> f32 .t() target"])
+def test_transposed_f32_parents_convert_in_the_transposing_kernel(gpu_device, narrow, direction):
+    """fp32 shards that are ``.t()`` views with a 16-bit wire dtype (master weights stored [in, out] -> serving
+    weights, and back): the transposing blocks convert on the way, full blocks and edge blocks, against the oracle."""
+    src, tgt = mesh_of(0, [4]), mesh_of(4, [2])
+    pack_side = direction.startswith("f32")
+    specs = [TensorSpec(f"w{i}", (776, 776), src, (Shard(0),), tgt, (Shard(0),), torch.float32 if pack_side else narrow,
+                        narrow if pack_side else torch.float32, seed=i,
+                        source_layout="transposed" if pack_side else "contiguous",
+                        target_layout="contiguous" if pack_side else "transposed") for i in range(2)]
+    job, _ = gpu_vs_oracle(specs, gpu_device, 256 * 1024, target_ranks=[4])
+    if pack_side:
+        infos = [job.wire.plan(b).send_table.info() for b in job.send_buckets.values()]
+        tiles = job.wire.plan(job.send_buckets[0]).send_table.trans_tiles()
+    else:
+        infos = [job.wire.plan(job.recv_buckets[4]).recv_table.info()]
+        tiles = job.wire.plan(job.recv_buckets[4]).recv_table.trans_tiles()
+    assert all(i.n_trans_tiles > 0 and i.n_row_tiles == 0 for i in infos)
+    assert np.all(tiles["cvt"] != 0) and ((tiles["nj"] == 128) & (tiles["nk"] == 128)).any() and (tiles["nj"] < 128).any()
+
+
 def test_transposed_parents_full_size_properties(gpu_device):
     """16 bf16 [8192, 8192] weights handed over as ``.t()`` views: every target shard equals its slice of the
     global tensor, the (non-contiguous) sources are unchanged."""
@@ -556,6 +578,20 @@ def test_transposed_parents_full_size_properties(gpu_device):
     for i, d in enumerate(job.source_locals):
         for r, t in d.items():
             assert t.view(torch.int16).sum(dtype=torch.int64).item() == sums[i][r], "source mutated"
+
+
+def test_transposed_parents_fp32_to_bf16_full_size_properties(gpu_device):
+    """16 fp32 [8192, 8192] weights handed over as ``.t()`` views, bf16 targets: every target shard is the RNE bf16 cast
+    of its slice of the fp32 global tensor (torch's device cast is the independent check); all chunks go through the
+    converting transposing blocks."""
+    specs, targets, bucket = workloads.transposed_parents_fp32_to_bf16()
+    job = ReshardJob(specs, device=gpu_device, bucket_size=bucket, target_ranks=targets, keep_globals=True)
+    assert job.payload_bytes() == 16 * 8192 * 4096 * 2
+    for b in job.send_buckets.values():
+        info = job.wire.plan(b).send_table.info()
+        assert info.n_trans_tiles > 0 and info.n_row_tiles == 0 and info.n_run_tiles == 0
+    job.run(merge_launches=True)
+    _check_targets_against_global(job, specs, cast=torch.bfloat16)
 
 
 def test_moe_row_parallel_w2(gpu_device):

@@ -137,6 +137,8 @@ def test_partial_and_self_copy_through_a_ring(op):
     ("transposed_parents", dict(n_tensors=2, n=392, target_transposed=True, dtype=torch.float32)),
     ("transposed_parents", dict(n_tensors=1, n=264, target_transposed=True, dtype=torch.float64)),
     ("transposed_parents", dict(n_tensors=1, n=520, dtype=torch.int8)),
+    ("transposed_parents", dict(n_tensors=2, n=776, dtype=torch.float32, target_dtype=torch.bfloat16)),
+    ("transposed_parents", dict(n_tensors=1, n=600, dtype=torch.float16, target_dtype=torch.float32, target_transposed=True)),
     ("moe_experts_row_parallel_w2", dict(n_experts=8, hidden=64, inter=224)),
 ])
 def test_other_workloads_scaled_down(name, kw):

@@ -362,6 +362,49 @@ def test_large_transposed_chunk_of_2_byte_elements_uses_wide_blocks():
             assert np.array_equal(arena.bytes_at(t, rows * cols * es), want2)
 
 
+@pytest.mark.parametrize("wdt", [nat.BF16, nat.F16])
+def test_transposed_f32_parent_converts_inside_the_lds_blocks(wdt):
+    """An f32 chunk of a transposed view with a 16-bit bucket: the transposing blocks convert (pack: f32 -> wire while
+    parking; unpack: wire -> f32 while emitting) instead of leaving the chunk to strided element tiles."""
+    rows, cols = 310, 280
+    arena = HostArena(2 * rows * cols * 4 + rows * cols * 2 + 65536)
+    t = arena.alloc(rows * cols * 4)   # storage of the [cols, rows] f32 parent; the view is its transpose
+    vals = (rs.randn(rows * cols) * 10.0 ** rs.uniform(-6, 6, rows * cols)).astype(np.float32)
+    vals[:6] = [np.inf, -np.inf, 0.0, -0.0, 65520.0, 1e-41]
+    arena.bytes_at(t, rows * cols * 4)[:] = vals.view(np.uint8)
+    nj, nk = 300, 270
+    b = arena.alloc(nj * nk * 2)
+    start, cshape, strides = (4, 3), (nj, nk), (1, rows)
+    d = _mk_desc(t, t, t + rows * cols * 4, b, b, b + nj * nk * 2, start, cshape, strides, nat.F32, wdt)
+    table = nat.Table.create(d.reshape(1), upload=False)
+    info, tiles = table.info(), table.trans_tiles()
+    assert info.n_run_tiles == 0 and info.n_row_tiles == 0 and info.n_trans_tiles == 9
+    assert np.all(tiles["cvt"] == ((nat.F32 << 4) | wdt)) and np.all(tiles["es_log2"] == 1)
+    assert int(((tiles["nj"] == 128) & (tiles["nk"] == 128)).sum()) == 4 and int(tiles["nj"].max()) == 128
+    before = arena.bytes_at(t, rows * cols * 4).copy()
+    execute(table, arena, "pack")
+    want = np.zeros(nj * nk * 2, dtype=np.uint8)
+    scratch = np.zeros(nj * nk * 4, dtype=np.uint8)
+    oc = co.make_chunk(t, start, cshape, strides, nat.F32, wdt, bucket_off=0)
+    assert co.lib().oracle_pack_bucket(oc, 1, want.ctypes.data, scratch.ctypes.data) == 0
+    assert np.array_equal(arena.bytes_at(b, nj * nk * 2), want)
+    assert np.array_equal(arena.bytes_at(t, rows * cols * 4), before)
+    assert arena.writes.max() == 1 and int(arena.writes.sum()) == nj * nk * 2
+    # and back: the 16-bit bucket widened into a second transposed f32 parent
+    arena.writes[:] = 0
+    t2 = arena.alloc(rows * cols * 4)
+    before2 = arena.bytes_at(t2, rows * cols * 4).copy()
+    d2 = _mk_desc(t2, t2, t2 + rows * cols * 4, b, b, b + nj * nk * 2, start, cshape, strides, nat.F32, wdt)
+    table2 = nat.Table.create(d2.reshape(1), upload=False)
+    assert table2.info().n_trans_tiles == 9
+    execute(table2, arena, "unpack")
+    want2 = before2.copy()
+    oc2 = co.make_chunk(want2.ctypes.data, start, cshape, strides, nat.F32, wdt, bucket_off=0)
+    assert co.lib().oracle_unpack_bucket(oc2, 1, want.ctypes.data, scratch.ctypes.data) == 0
+    assert np.array_equal(arena.bytes_at(t2, rows * cols * 4), want2)
+    assert arena.writes.max() == 1 and int(arena.writes.sum()) == nj * nk * 4
+
+
 @pytest.mark.parametrize("dt", [nat.B8, nat.BF16, nat.F32, nat.B64])
 def test_transposed_parent_uses_lds_blocks(dt):
     """A chunk of a transposed view: the tensor side is contiguous along dim 0, the bucket along dim 1."""

@@ -198,18 +198,27 @@ def _transpose_blocks(arena, trans, rev: bool) -> None:
         es = 1 << int(t["es_log2"])
         nj, nk = int(t["nj"]), int(t["nk"])
         assert 0 < nj <= 512 and 0 < nk <= 512  # block side: a fixed number of bytes per row
+        cvt = int(t["cvt"])
+        dta, dtb = cvt >> 4, cvt & 15
+        if cvt:  # a converting block: f32 on the a side, f16 or bf16 in the bucket; blocks are sized by the b side
+            assert dta == 2 and dtb in (0, 1) and es == 2 and nj <= 128 and nk <= 128
+        esa, esb = (_CODE_SIZE[dta], _CODE_SIZE[dtb]) if cvt else (es, es)
         j, k = np.meshgrid(np.arange(nj), np.arange(nk), indexing="ij")
-        a = int(t["a"]) + j * es + k * int(t["a_pitch"])
-        b = int(t["b"]) + j * int(t["b_pitch"]) + k * es
-        assert np.all(a % es == 0) and np.all(b % es == 0)
-        src, dst = (b, a) if rev else (a, b)
-        so = arena.offsets(src.reshape(-1), es)[:, None] + np.arange(es)
-        do = arena.offsets(dst.reshape(-1), es)[:, None] + np.arange(es)
+        a = int(t["a"]) + j * esa + k * int(t["a_pitch"])
+        b = int(t["b"]) + j * int(t["b_pitch"]) + k * esb
+        assert np.all(a % esa == 0) and np.all(b % esb == 0)
+        src, dst, ess, esd, ds_, dd = (b, a, esb, esa, dtb, dta) if rev else (a, b, esa, esb, dta, dtb)
+        so = arena.offsets(src.reshape(-1), ess)[:, None] + np.arange(ess)
+        do = arena.offsets(dst.reshape(-1), esd)[:, None] + np.arange(esd)
         if arena.writes is not None:
             np.add.at(arena.writes, do.reshape(-1), 1)
         _note("r", so)
         _note("w", do)
-        mem[do] = mem[so]
+        data = mem[so]
+        if cvt:
+            elems = np.ascontiguousarray(data).view(_CODE_RAW[ds_]).reshape(-1)
+            data = co.cast(elems, ds_, dd, _CODE_RAW[dd]).view(np.uint8).reshape(len(so), esd)
+        mem[do] = data
 
 
 def _reduce_units(arena, mem, row_tiles, row_idx, a_off, b, ua, ub, dta, dtb, peers, skew_a=False):
