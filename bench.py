@@ -222,16 +222,19 @@ def time_steps(job, steps, run):
 
     stream = torch.cuda.current_stream(job.device)
     ev = [torch.cuda.Event(enable_timing=True) for _ in range(steps + 1)]
-    # an untimed burst first: the first time steps queue up behind each other without a host synchronisation the
-    # HIP runtime grows its internal pools once (a host stall of tens of milliseconds)
-    for _ in range(min(steps, 5)):
-        run()
-    torch.cuda.synchronize()
     import gc
 
+    # a full collection stalls the host for tens of milliseconds: none inside the timed region, and the one here
+    # comes before the untimed burst, not between it and the first timed step (the GPU would sit idle meanwhile
+    # and the steps after such a pause measured 5-6 % slower on a 1.2 ms step)
     gc.collect()
-    gc.disable()  # a full collection in the middle of the region stalls the host for tens of milliseconds
+    gc.disable()
     try:
+        # an untimed burst first: the first time steps queue up behind each other without a host synchronisation
+        # the HIP runtime grows its internal pools once (a host stall of tens of milliseconds)
+        for _ in range(min(steps, 5)):
+            run()
+        torch.cuda.synchronize()
         wall0 = time.perf_counter()
         ev[0].record(stream)
         for k in range(steps):
@@ -467,6 +470,32 @@ def main():
             out["resident_pool_run_of_buckets"] = d
             del res
             torch.cuda.empty_cache()
+            if args.workload == "llama3_8b_fsdp8_to_tp2":
+                # the Partial collapse has no part in this workload: its rates on config 4, beside pack and unpack above
+                p_specs, p_targets, p_bucket = workloads.WORKLOADS["partial4_to_shard2"]()
+                red = ReshardJob(p_specs, device=dev, bucket_size=p_bucket, target_ranks=p_targets, pool="resident")
+                for _ in range(2):
+                    red.run(merge_launches=True)
+                r_pack, r_unpack = algorithmic_bytes(red)[:2]
+                ev = [[torch.cuda.Event(enable_timing=True) for _ in range(3)] for _ in range(reps)]
+                for k in range(reps):
+                    ev[k][0].record(stream)
+                    red.run_send(True)
+                    ev[k][1].record(stream)
+                    red.run_recv(True)
+                    ev[k][2].record(stream)
+                torch.cuda.synchronize()
+                p_ms = sum(e[0].elapsed_time(e[1]) for e in ev) / reps
+                u_ms = sum(e[1].elapsed_time(e[2]) for e in ev) / reps
+                out["partial_reduce"] = {
+                    "workload": "partial4_to_shard2",
+                    "reduce_pack": {"GB/s": round(r_pack / (p_ms * 1e-3) / 1e9, 1), "ms": round(p_ms, 4),
+                                    "bytes": r_pack, "pool": "resident"},
+                    "unpack": {"GB/s": round(r_unpack / (u_ms * 1e-3) / 1e9, 1), "ms": round(u_ms, 4), "bytes": r_unpack,
+                               "pool": "resident"},
+                }
+                del red
+                torch.cuda.empty_cache()
         except Exception as e:  # an optional leg must not take the measured line with it
             out["extra_legs_error"] = f"{type(e).__name__}: {e}"
 
