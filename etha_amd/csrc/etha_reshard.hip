@@ -125,6 +125,8 @@ __host__ __device__ constexpr uint32_t trans_dim_b(uint32_t es) { return es == 8
 // registers and goes through LDS in trans_panels(es) panels of columns, so LDS holds a panel, not the block.
 __host__ __device__ constexpr uint32_t trans_wide(uint32_t es) { return es <= 2 ? 2u : 1u; }
 __host__ __device__ constexpr uint32_t trans_panels(uint32_t es) { return es == 2 ? 2u : 1u; }
+// wide blocks of chunks that convert between f32 (a side) and a 16-bit wire type: j x k elements
+constexpr uint32_t kTransCvtWideJ = ETHA_TRANS_DIM_A, kTransCvtWideK = 2 * ETHA_TRANS_DIM_B;
 __host__ __device__ constexpr uint32_t trans_pitch(uint32_t dim, uint32_t es) {  // LDS row pitch in elements: an odd number of words
   return dim + (es >= 4 ? 1u : 4u / es);
 }
@@ -780,7 +782,12 @@ __device__ __forceinline__ void transpose_block_cvt(const TransTile& t, uint8_t*
   const uint64_t src = REV ? t.b : t.a, dst = REV ? t.a : t.b;
   const int64_t src_pitch = REV ? t.b_pitch : t.a_pitch, dst_pitch = REV ? t.a_pitch : t.b_pitch;
   const uint32_t nx = REV ? t.nk : t.nj, ny = REV ? t.nj : t.nk;
-  if (nx == kDX && ny == kDY) {
+  if (t.nj == kTransCvtWideJ && t.nk == kTransCvtWideK) {  // runs of 512 bytes on both sides: 128 f32, 256 16-bit elements
+    if constexpr (REV)
+      transpose_cvt_unpack<TB, kTransCvtWideK, kTransCvtWideJ>(src, src_pitch, dst, dst_pitch, lds);
+    else
+      transpose_cvt_pack<TB, kTransCvtWideJ, kTransCvtWideK>(src, src_pitch, dst, dst_pitch, lds);
+  } else if (nx == kDX && ny == kDY) {
     if constexpr (REV)
       transpose_cvt_unpack<TB, kDX, kDY>(src, src_pitch, dst, dst_pitch, lds);
     else
@@ -1288,8 +1295,10 @@ class PairCompiler {
     // blocks are sized by the element that goes through LDS: the b side's
     const int64_t kDimJ = (int64_t)trans_dim_a((uint32_t)esb_), kDimK = (int64_t)trans_dim_b((uint32_t)esb_);
     // the part of the chunk that whole wide blocks cover; blocks of the plain extent (and edge blocks) cover the rest
-    const int64_t kP = converting ? 1 : (int64_t)trans_wide((uint32_t)esb_);
-    const int64_t wide_j = kP > 1 ? n_[j] / (kDimJ * kP) * (kDimJ * kP) : 0, wide_k = kP > 1 ? n_[kk] / (kDimK * kP) * (kDimK * kP) : 0;
+    const int64_t kP = (int64_t)trans_wide((uint32_t)esb_);
+    const int64_t wide_dim_j = converting ? (int64_t)kTransCvtWideJ : kDimJ * kP, wide_dim_k = converting ? (int64_t)kTransCvtWideK : kDimK * kP;
+    const bool has_wide = wide_dim_j > kDimJ || wide_dim_k > kDimK;
+    const int64_t wide_j = has_wide ? n_[j] / wide_dim_j * wide_dim_j : 0, wide_k = has_wide ? n_[kk] / wide_dim_k * wide_dim_k : 0;
     const bool wide = wide_j > 0 && wide_k > 0;
     do {
       // Launch order.  Blocks are grouped into super-blocks of S x S blocks that are emitted together: blocks
@@ -1324,7 +1333,7 @@ class PairCompiler {
                 bld_.trans.push_back(t);
               }
       };
-      if (wide) emit(kDimJ * kP, kDimK * kP, wide_j, wide_k, 0, 0);
+      if (wide) emit(wide_dim_j, wide_dim_k, wide_j, wide_k, 0, 0);
       if (!wide || wide_j < n_[j] || wide_k < n_[kk]) emit(kDimJ, kDimK, n_[j], n_[kk], wide ? wide_j : 0, wide ? wide_k : 0);
       const int rc = check_size();
       if (rc != ETHA_OK) return rc;

@@ -551,7 +551,7 @@ def test_transposed_f32_parents_convert_in_the_transposing_kernel(gpu_device, na
     weights, and back): the transposing blocks convert on the way, full blocks and edge blocks, against the oracle."""
     src, tgt = mesh_of(0, [4]), mesh_of(4, [2])
     pack_side = direction.startswith("f32")
-    specs = [TensorSpec(f"w{i}", (776, 776), src, (Shard(0),), tgt, (Shard(0),), torch.float32 if pack_side else narrow,
+    specs = [TensorSpec(f"w{i}", (904, 904), src, (Shard(0),), tgt, (Shard(0),), torch.float32 if pack_side else narrow,
                         narrow if pack_side else torch.float32, seed=i,
                         source_layout="transposed" if pack_side else "contiguous",
                         target_layout="contiguous" if pack_side else "transposed") for i in range(2)]
@@ -563,7 +563,9 @@ def test_transposed_f32_parents_convert_in_the_transposing_kernel(gpu_device, na
         infos = [job.wire.plan(job.recv_buckets[4]).recv_table.info()]
         tiles = job.wire.plan(job.recv_buckets[4]).recv_table.trans_tiles()
     assert all(i.n_trans_tiles > 0 and i.n_row_tiles == 0 for i in infos)
-    assert np.all(tiles["cvt"] != 0) and ((tiles["nj"] == 128) & (tiles["nk"] == 128)).any() and (tiles["nj"] < 128).any()
+    wide = (tiles["nj"] == 128) & (tiles["nk"] == 256)
+    full = (tiles["nj"] == 128) & (tiles["nk"] == 128)
+    assert np.all(tiles["cvt"] != 0) and wide.any() and full.any() and (~wide & ~full).any()
 
 
 def test_transposed_parents_full_size_properties(gpu_device):

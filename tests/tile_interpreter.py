@@ -201,7 +201,7 @@ def _transpose_blocks(arena, trans, rev: bool) -> None:
         cvt = int(t["cvt"])
         dta, dtb = cvt >> 4, cvt & 15
         if cvt:  # a converting block: f32 on the a side, f16 or bf16 in the bucket; blocks are sized by the b side
-            assert dta == 2 and dtb in (0, 1) and es == 2 and nj <= 128 and nk <= 128
+            assert dta == 2 and dtb in (0, 1) and es == 2 and nj <= 128 and nk <= 256
         esa, esb = (_CODE_SIZE[dta], _CODE_SIZE[dtb]) if cvt else (es, es)
         j, k = np.meshgrid(np.arange(nj), np.arange(nk), indexing="ij")
         a = int(t["a"]) + j * esa + k * int(t["a_pitch"])
