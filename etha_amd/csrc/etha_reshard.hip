@@ -392,6 +392,23 @@ __device__ __forceinline__ void move_unit(uint32_t meta, uint64_t a, uint64_t b)
     }
     return;
   }
+  // The usual converting pairs first - f32 on the a side, bf16 or f16 in the bucket, whole vectors - found with one
+  // compare each and handled by straight-line code: a workgroup lives a few microseconds, and the chain of
+  // dtype switches below (with the jumps across this kernel's code that it takes) sits in front of its load.
+  {
+    constexpr uint32_t kPairMask = (15u << kMetaDtaShift) | (15u << kMetaDtbShift) | kMetaVec | kMetaGeneric;
+    const uint32_t pair = meta & kPairMask;
+    if (pair == (((uint32_t)ETHA_F32 << kMetaDtaShift) | ((uint32_t)ETHA_BF16 << kMetaDtbShift) | kMetaVec)) {
+      constexpr int kN = cvt_elems_per_unit(4, 2);
+      if (REV) cvt_n<TagBF16, TagF32, kN>(src, dst); else cvt_n<TagF32, TagBF16, kN>(src, dst);
+      return;
+    }
+    if (pair == (((uint32_t)ETHA_F32 << kMetaDtaShift) | ((uint32_t)ETHA_F16 << kMetaDtbShift) | kMetaVec)) {
+      constexpr int kN = cvt_elems_per_unit(4, 2);
+      if (REV) cvt_n<TagF16, TagF32, kN>(src, dst); else cvt_n<TagF32, TagF16, kN>(src, dst);
+      return;
+    }
+  }
   const uint32_t dta = (meta >> kMetaDtaShift) & 15u, dtb = (meta >> kMetaDtbShift) & 15u;
   const uint32_t sd = REV ? dtb : dta, dd = REV ? dta : dtb;
   if (meta & kMetaGeneric) {
