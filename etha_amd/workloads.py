@@ -73,6 +73,17 @@ def many_small_2d_to_replicate(n_tensors: int = 256, rows: int = 2048, k_seed: i
     return specs, [8], 64 * MIB
 
 
+def scatter_32_byte_pieces(piece_bytes: int = 32, total_bytes: int = 1 << 29, dtype=torch.bfloat16):
+    """One [rows, 4 * piece] tensor whose four column blocks sit on four source ranks (mesh (1,4), Shard(1)) and
+    are scattered into one replicated target: every target row is four pieces of ``piece_bytes`` from four
+    buckets, 0.5 GiB in all - the shortest rows of ``many_small_2d_to_replicate`` on their own."""
+    es = torch.empty((), dtype=dtype).element_size()
+    cols = piece_bytes // es * 4
+    rows = total_bytes // (piece_bytes * 4)
+    src, tgt = _mesh(0, (1, 4)), _mesh(4, (1,))
+    return [TensorSpec("t", (rows, cols), src, (Replicate(), Shard(1)), tgt, (Replicate(),), dtype, seed=1)], [4], 64 * MIB
+
+
 def partial4_to_shard2(n_tensors: int = 16, n: int = 8192, dtype=torch.bfloat16):
     """16 bf16 [8192,8192], mesh (4,) Partial(sum) -> mesh (2,) Shard(0); one target rank.
     Partial of source rank r of tensor i: normal(0, 0.02) with seed 4*i + r."""
@@ -143,6 +154,7 @@ WORKLOADS = {
     "llama3_8b_fsdp8_to_tp2_fp32_to_bf16": llama3_8b_fsdp8_to_tp2_fp32_to_bf16,
     "many_small_2d_to_replicate": many_small_2d_to_replicate,
     "partial4_to_shard2": partial4_to_shard2,
+    "scatter_32_byte_pieces": scatter_32_byte_pieces,
     "moe_experts_and_uneven_vocab": moe_experts_and_uneven_vocab,
     "moe_experts_row_parallel_w2": moe_experts_row_parallel_w2,
     "transposed_parents": transposed_parents,

@@ -596,6 +596,17 @@ def test_transposed_parents_fp32_to_bf16_full_size_properties(gpu_device):
     _check_targets_against_global(job, specs, cast=torch.bfloat16)
 
 
+@pytest.mark.parametrize("piece_bytes", [32, 96, 1024])
+def test_scatter_of_short_pieces_workload(gpu_device, piece_bytes):
+    """The short-piece scatter workload scaled down (four column blocks from four ranks into one replicated target),
+    merged launches so that the write-ordered range with its gather tiles runs, against the oracle."""
+    specs, targets, _ = workloads.scatter_32_byte_pieces(piece_bytes=piece_bytes, total_bytes=3 << 20)
+    for s in specs:
+        s.dist = "bits"
+    for _ in range(2):  # the second transfer runs the write-ordered copy made during the first
+        gpu_vs_oracle(specs, gpu_device, 256 * 1024, target_ranks=targets, merge_launches=True)
+
+
 def test_moe_row_parallel_w2(gpu_device):
     """The expert layout's second reading - w2 [E, H, I] row-parallel, Shard(0)@8 -> Shard(2)@4 (rows of I/4
     elements at a pitch of I) - scaled down against the oracle, then at full size through the closed form."""
