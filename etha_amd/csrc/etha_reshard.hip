@@ -94,7 +94,7 @@ struct TransTile {   // a 2-D block whose contiguous dim differs between the two
   uint64_t b;        // address of element (j0, k0) on the b side, contiguous along k
   int64_t a_pitch;   // bytes between consecutive k on the a side
   int64_t b_pitch;   // bytes between consecutive j on the b side
-  uint32_t nj, nk;   // extent of the block (<= trans_dim(element size) each)
+  uint32_t nj, nk;   // extent of the block: a wide block, a block of trans_dim_a x trans_dim_b elements, or less at an edge
   uint32_t es_log2;  // log2 of the element size in bytes (of the b side, when the block converts)
   uint32_t cvt;      // 0: same element type on both sides; else (dtype of a << 4) | dtype of b: a holds f32, b f16 or bf16
 };
@@ -563,7 +563,8 @@ __global__ __launch_bounds__(ETHA_BLOCK_THREADS) void etha_unpack_mixed_kernel(c
 // vector gathered element by element from LDS.  Both global sides therefore move whole 16-byte vectors in
 // runs of at least 128 bytes; without the staging one side would touch a different line per element.
 // Blocks at the edge of a chunk (fewer than D elements on a side) take the element-wise path.
-// the vectors q = tid + i * kTransThreads of DY source rows of DX elements each, row by row
+// The steps of one block of DY source rows of DX elements: work-item tid handles vectors q = tid + i * kTransThreads,
+// counted row by row.
 template <typename E, uint32_t DX, uint32_t DY>
 struct TransBlock {
   static constexpr uint32_t kEs = sizeof(E), kV = 16 / kEs, kVecPerRow = DX / kV, kOutPerRow = DY / kV;
