@@ -14,7 +14,7 @@ import numpy as np
 from .build import LIB_PATH
 
 ETHA_MAX_NDIM = 8
-ABI_VERSION = 5
+ABI_VERSION = 6
 LAUNCH_UNORDERED = 1  # ETHA_LAUNCH_UNORDERED
 SEG_PACK, SEG_UNPACK, SEG_REDUCE_PACK, SEG_SELFCOPY = 0, 1, 2, 3  # ETHA_SEG_*
 MAX_SEGMENTS = 16
@@ -76,6 +76,16 @@ class Segment(ctypes.Structure):
     _fields_ = [("table", c_void_p), ("kind", c_uint32), ("first", c_uint32), ("count", c_uint32), ("reserved", c_uint32)]
 
 
+class ScheduleCall(ctypes.Structure):
+    """EthaScheduleCall: one recorded launch call (a set of segments, or one range run by itself)."""
+
+    _fields_ = [("first_segment", c_uint32), ("n_segments", c_uint32), ("flags", c_uint32), ("single", c_uint32)]
+
+
+class ScheduleInfo(ctypes.Structure):
+    _fields_ = [("n_calls", c_uint32), ("n_kernel_launches", c_uint32), ("n_tables", c_uint32), ("reserved", c_uint32)]
+
+
 class TableInfo(ctypes.Structure):
     _fields_ = [
         ("n_chunks", c_uint32),
@@ -121,6 +131,10 @@ _SIGNATURES = {
     "etha_reduce_pack_bucket": (c_int, [c_void_p, c_uint32, c_uint32, c_void_p, c_uint32]),
     "etha_selfcopy_bucket": (c_int, [c_void_p, c_uint32, c_uint32, c_void_p, c_uint32]),
     "etha_launch_segments": (c_int, [c_void_p, c_uint32, c_void_p, c_uint32]),
+    "etha_schedule_create": (c_int, [c_void_p, c_uint32, c_void_p, c_uint32, POINTER(c_void_p)]),
+    "etha_schedule_launch": (c_int, [c_void_p, c_void_p]),
+    "etha_schedule_info": (c_int, [c_void_p, POINTER(ScheduleInfo)]),
+    "etha_schedule_destroy": (c_int, [c_void_p]),
     "etha_kernel_launches": (c_uint64, []),
     "etha_noalloc_setup": (c_int, []),
     "etha_copy_regions_noalloc": (c_int, [c_void_p, c_void_p, c_uint32, c_void_p]),
@@ -344,6 +358,53 @@ def launch_segments(segments, stream: int = 0, flags: int = 0) -> None:
     for i, (table, kind, first, count) in enumerate(segments):
         arr[i].table, arr[i].kind, arr[i].first, arr[i].count = table._h, kind, first, count
     _check("etha_launch_segments", lib().etha_launch_segments(arr, len(segments), c_void_p(stream), flags))
+
+
+class Schedule:
+    """Owner of one recorded transfer (``EthaSchedule*``): launch calls planned once, re-issued with one call.
+
+    ``calls`` is a list of ``(segments, flags, single)`` in issue order, ``segments`` as for :func:`launch_segments`;
+    ``single`` marks a one-segment call that runs as its single-range entry point would.  The tables are kept alive.
+    """
+
+    def __init__(self, calls):
+        n_seg = sum(len(c[0]) for c in calls)
+        segs = (Segment * max(n_seg, 1))()
+        recs = (ScheduleCall * max(len(calls), 1))()
+        self._tables = []
+        k = 0
+        for i, (segments, flags, single) in enumerate(calls):
+            recs[i].first_segment, recs[i].n_segments, recs[i].flags, recs[i].single = k, len(segments), flags, int(bool(single))
+            for table, kind, first, count in segments:
+                segs[k].table, segs[k].kind, segs[k].first, segs[k].count = table._h, kind, first, count
+                self._tables.append(table)
+                k += 1
+        out = c_void_p()
+        _check("etha_schedule_create", lib().etha_schedule_create(segs, n_seg, recs, len(calls), byref(out)))
+        self._h = out
+        self._launch = lib().etha_schedule_launch
+
+    def launch(self, stream: int = 0) -> None:
+        rc = self._launch(self._h, stream)
+        if rc != 0:
+            _check("etha_schedule_launch", rc)
+
+    def info(self) -> ScheduleInfo:
+        info = ScheduleInfo()
+        _check("etha_schedule_info", lib().etha_schedule_info(self._h, byref(info)))
+        return info
+
+    def close(self) -> None:
+        if self._h:
+            lib().etha_schedule_destroy(self._h)
+            self._h = c_void_p()
+        self._tables = []
+
+    def __del__(self):
+        try:
+            self.close()
+        except Exception:
+            pass
 
 
 def ipc_open(handle_bytes: bytes) -> int:

@@ -339,6 +339,10 @@ class TransferPlan:
             with torch.cuda.device(self.device):
                 self._enqueue(steps, lambda i, slots: stream)
             return
+        # buckets stepped by hand move slots outside the pipelines: transfers recorded on this wire no longer
+        # describe what its pipelines would do
+        self.wire.replay_schedules = False
+        self.wire.forget_recorded_transfers()
         with torch.cuda.device(self.device):
             for (kind, first, count, _), info in zip(self.steps, self.info):
                 if kind not in kinds:

@@ -117,6 +117,23 @@ class _no_context:
 # steps that are launched at once: the few, large one-pass copies of the direct wire measured 2 % slower in sets
 _UNGROUPED = ("direct", "direct_reduce")
 
+_DRIVE = ("d",)
+_MAX_TRACE_NODES = 4096
+
+
+class _TraceNode:
+    """One point of a recorded transfer (see :attr:`LoopbackWire.replay_schedules`): reached from its parent by a
+    ``submit`` or a ``drive`` event.  A node reached by a drive holds what that drive issued."""
+
+    __slots__ = ("children", "calls", "schedule", "pending", "recorded")
+
+    def __init__(self):
+        self.children: dict = {}
+        self.calls: list = []  # [(group, flags, single)], group = [(plan, kind, first, count), ...], in issue order
+        self.schedule = None  # the same as one native schedule (built on first replay on a GPU)
+        self.pending: frozenset = frozenset()  # ids of the plans whose pipelines are still waiting after this drive
+        self.recorded = False
+
 
 def wire_key(bucket: Bucket) -> tuple:
     return (bucket.src_rank, tuple(bucket.dst_ranks), bucket.transport.value)
@@ -171,6 +188,23 @@ class LoopbackWire:
         # This is what a pull over a peer mapping does between GPUs, minus the link.  Like a lent bucket,
         # a "sent" tensor must be left alone until the consumer has run.  Only within one process.
         self.direct_same_device = False
+        # True: a transfer that repeats one seen before is not walked through the pipelines again.  The reference
+        # plans once and transfers N times (tensor_bus/batch_state.py:38-40); the pipelines here are deterministic,
+        # so from an idle wire the same sequence of submit / drive calls issues the same launches.  The wire keeps
+        # what every drive of such a sequence issued and, when the sequence recurs, re-issues it with one library
+        # call per drive (etha_schedule_launch) instead of stepping the Python pipelines.  A sequence that departs
+        # from every recorded one falls back to the pipelines (their state is rebuilt first) and is recorded too.
+        self.replay_schedules = True
+        self._trace_root = _TraceNode()
+        self._trace_nodes = 0
+        self._trace_absent: set = set()
+        self._tx_events: list = []  # events of the transfer under way since the wire was last idle
+        self._tx_node: _TraceNode | None = None  # trie node of those events; None: this transfer is not traced
+        self._tx_replaying = False  # the transfer under way follows a recorded one: no pipelines exist for it
+        self._tx_pending: set = set()  # replaying: ids of plans submitted and not yet finished
+        self._tx_calls: list | None = None  # recording: what the drive under way has issued so far
+        self._suppress = False  # rebuilding pipeline state: steps are walked, nothing is launched
+        self.replays = 0  # drives served from a recorded schedule (statistics)
         self.pool: BucketPool | None = None
         # per wire key: sequence number -> (slot, chunk sizes) of every planned send bucket still alive
         self._sent: dict[tuple, dict[int, tuple[Slot, tuple[int, ...]]]] = defaultdict(dict)
@@ -360,6 +394,7 @@ class LoopbackWire:
         plan = self._plans.pop(tuple(id(b) for b in buckets), None)
         if plan is None:
             return
+        self.forget_recorded_transfers()  # they name this plan's tables
         self._programs = [p for p in self._programs if p.plan is not plan]
         for entry in plan.owned_entries:  # sequence numbers are never reused: later plans on this key keep theirs
             self._sent.get(entry.key, {}).pop(entry.seq, None)
@@ -374,29 +409,159 @@ class LoopbackWire:
         self._send_seq.clear()
         self._recv_seq.clear()
         self._programs.clear()
+        self._tx_replaying = False
+        self.forget_recorded_transfers()
+        self._tx_events, self._tx_pending = [], set()
         self.pool = None
+
+    # -- the bucket pipelines of every rank on this wire ---------------------------------------
+    # -- recorded transfers ----------------------------------------------------------------------
+    def _tracing(self) -> bool:
+        if not (self.replay_schedules and self.pool_mode == "ring" and self.on_launch is None and self.launch_log is None
+                and (self.on_set is not None or (self.device is not None and self.device.type == "cuda"))):
+            return False
+        if self.absent_ranks != self._trace_absent:  # who unpacks decides when a slot is free again
+            self.forget_recorded_transfers()
+            self._trace_absent = set(self.absent_ranks)
+        return True
+
+    def forget_recorded_transfers(self) -> None:
+        """Drop every recorded transfer (a plan they name is going away, or the wire was driven by hand).  A transfer
+        under way that was following one goes back to the pipelines."""
+        if self._tx_replaying:
+            self._rebuild_pipelines()
+        self._trace_root = _TraceNode()
+        self._trace_nodes = 0
+        self._tx_node = None
+
+    def _child(self, node: _TraceNode, event) -> _TraceNode | None:
+        child = node.children.get(event)
+        if child is None:
+            if self._trace_nodes >= _MAX_TRACE_NODES:
+                return None
+            child = node.children[event] = _TraceNode()
+            self._trace_nodes += 1
+        return child
+
+    def _rebuild_pipelines(self) -> None:
+        """The transfer under way was following a recorded one and now departs from it: bring the pipelines to the
+        state they would be in, by walking the events so far with launching switched off."""
+        from .comm_methods import Program
+
+        events, self._tx_replaying = self._tx_events, False
+        self._tx_pending = set()
+        self._suppress = True
+        try:
+            for ev in events:
+                if ev[0] == "s":
+                    self._programs.append(Program(ev[1], ev[2], ev[3]))
+                else:
+                    self._drive_pipelines()
+        finally:
+            self._suppress = False
+
+    def _end_of_drive(self, idle: bool) -> None:
+        if idle:  # the transfer is over: the next submit starts a new one
+            self._tx_events, self._tx_node, self._tx_replaying = [], None, False
+            self._tx_pending = set()
 
     # -- the bucket pipelines of every rank on this wire ---------------------------------------
     def submit(self, plan, max_in_flight: int, merge_launches: bool = False):
         """Start one transfer of a planned bucket list: its pipeline joins the ones :meth:`drive` steps."""
         from .comm_methods import Program
 
+        event = ("s", id(plan), max_in_flight, merge_launches, self.unordered_launches, self.group_launches)
+        if not self._programs and not self._tx_events:  # an idle wire: a new transfer begins
+            self._tx_replaying = False
+            self._tx_node = self._trace_root if self._tracing() else None
+            if self._tx_node is not None and event in self._tx_node.children:
+                self._tx_replaying = True
+        if self._tx_replaying:
+            child = self._tx_node.children.get(event) if id(plan) not in self._tx_pending else None
+            if child is not None:
+                self._tx_node = child
+                self._tx_events.append(("s", plan, max_in_flight, merge_launches))
+                self._tx_pending.add(id(plan))
+                return None
+            self._rebuild_pipelines()
         if any(p.plan is plan for p in self._programs):
             raise RuntimeError(
                 "the previous transfer of these buckets has not completed: its receivers have not unpacked yet "
                 "(a real wire would block here)")
         program = Program(plan, max_in_flight, merge_launches)
         self._programs.append(program)
+        self._tx_events.append(("s", plan, max_in_flight, merge_launches))
+        if self._tx_node is not None:
+            self._tx_node = self._child(self._tx_node, event)
         return program
 
     def drive(self) -> None:
         """Step every pending pipeline, in arrival order, until none can move.  Launches go to the current stream
         of the wire's device.  A sender's pipeline that is waiting for its receivers stays pending and is picked
         up by the call that brings them."""
+        if self._tx_replaying and self._drive_recorded():
+            return
         if not self._programs:
             return
+        record = self._tx_node is not None and not self._suppress
+        if record and self.on_set is None and torch.cuda.is_current_stream_capturing():
+            record, self._tx_node = False, None  # what a capture leaves out (uploads) must not end up in a recorded transfer
+        self._tx_calls = [] if record else None
+        try:
+            self._drive_pipelines()
+        except BaseException:
+            self._tx_node, self._tx_calls = None, None
+            raise
+        calls, self._tx_calls = self._tx_calls, None
+        self._tx_events.append(_DRIVE)
+        if record:
+            node = self._tx_node = self._child(self._tx_node, _DRIVE)
+            if node is not None and not node.recorded:
+                node.calls, node.pending, node.recorded = calls, frozenset(id(p.plan) for p in self._programs), True
+        self._end_of_drive(not self._programs)
+
+    def _drive_recorded(self) -> bool:
+        """Serve a drive from the recorded transfer the events so far follow; False when they follow none
+        (the pipelines have then been rebuilt and the caller steps them)."""
+        from .. import _native as nat
+
+        node = self._tx_node.children.get(_DRIVE)
+        if node is None or not node.recorded:
+            self._rebuild_pipelines()
+            return False
+        if self.on_set is not None:
+            for group, flags, _ in node.calls:
+                self.on_set(group, flags)
+        elif node.calls:
+            stream = torch.cuda.current_stream(self.device)
+            if self._carried and self._stream is not None and self._stream != stream:
+                done = torch.cuda.Event()
+                done.record(self._stream)
+                stream.wait_event(done)
+            self._stream = stream
+            try:
+                if node.schedule is None:
+                    node.schedule = nat.Schedule([([plan.segment(kind, first, count) for plan, kind, first, count in group],
+                                                   flags, single) for group, flags, single in node.calls])
+                with torch.cuda.device(self.device):
+                    node.schedule.launch(stream.cuda_stream)
+            except nat.EthaNativeError as e:
+                if "stale schedule" not in str(e):
+                    raise
+                # a table gained a write-ordered range since the recording: nothing was launched; start over
+                self.forget_recorded_transfers()
+                return False
+        self.replays += 1
+        self._tx_node = node
+        self._tx_events.append(_DRIVE)
+        self._tx_pending = set(node.pending)
+        self._carried = bool(node.pending)
+        self._end_of_drive(not node.pending)
+        return True
+
+    def _drive_pipelines(self) -> None:
         cuda = self.device is not None and self.device.type == "cuda" and self.on_launch is None and self.on_set is None
-        if cuda:
+        if cuda and not self._suppress:
             stream = torch.cuda.current_stream(self.device)
             if self._carried and self._stream is not None and self._stream != stream:
                 # work enqueued earlier for pipelines that are still pending sits on another stream
@@ -424,15 +589,21 @@ class LoopbackWire:
 
     def idle(self) -> bool:
         """True when no pipeline is waiting for a peer."""
-        return not self._programs
+        return not self._programs and not (self._tx_replaying and self._tx_pending)
 
     def in_progress(self, buckets: list[Bucket]) -> bool:
         """True while a transfer of this bucket list is still waiting for a peer (a send whose receivers have
         not all unpacked, a receive whose senders have not packed everything yet)."""
         plan = self._plans.get(tuple(id(b) for b in buckets))
-        return plan is not None and any(p.plan is plan for p in self._programs)
+        if plan is None:
+            return False
+        if self._tx_replaying:
+            return id(plan) in self._tx_pending
+        return any(p.plan is plan for p in self._programs)
 
     def pending(self) -> list[str]:
+        if self._tx_replaying:
+            return [f"pipeline of {ev[1].buckets[0]} ..." for ev in self._tx_events if ev[0] == "s" and id(ev[1]) in self._tx_pending]
         return [repr(p) for p in self._programs]
 
     def emit(self, plan, indices: list[int], merge: bool = False) -> None:
@@ -479,6 +650,8 @@ class LoopbackWire:
         flags = 0 if ordered else nat.LAUNCH_UNORDERED
         if self.launch_log is not None:
             self.launch_log.append((kind, first, count, flags))
+        if self._suppress:
+            return
         if self.on_launch is not None:
             self.on_launch(plan, kind, first, count, flags)
             return
@@ -486,6 +659,8 @@ class LoopbackWire:
             raise RuntimeError("this plan was compiled for host inspection; the executor only runs on a GPU (there is no CPU path)")
         if not self.group_launches or kind in _UNGROUPED:
             self._flush()
+            if self._tx_calls is not None:
+                self._tx_calls.append(([(plan, kind, first, count)], flags, True))
             if self.on_set is not None:
                 self.on_set([(plan, kind, first, count)], flags)
             else:
@@ -507,6 +682,8 @@ class LoopbackWire:
         from .. import _native as nat
 
         group, self._group = self._group, []
+        if self._tx_calls is not None:
+            self._tx_calls.append((group, self._group_flags, len(group) == 1))
         if self.on_set is not None:
             self.on_set(group, self._group_flags)
             return

@@ -22,6 +22,7 @@
 #include <atomic>
 #include <cstring>
 #include <map>
+#include <memory>
 #include <mutex>
 #include <new>
 #include <string>
@@ -1093,7 +1094,9 @@ __global__ __launch_bounds__(ETHA_BLOCK_THREADS) void etha_reduce_kernel(const R
 // =================================================================================================
 // Host side: validation and the tile compiler.
 // =================================================================================================
-thread_local std::string g_err;
+// message of the calling thread's last failure; a fixed buffer, so that reporting a failure (out of host memory
+// among them) allocates nothing
+thread_local char g_err[512] = "";
 // An allocation may be opened once per process; several tensors usually share one allocation, so
 // mappings are cached per handle and reference-counted.
 struct IpcMapping {
@@ -1108,13 +1111,26 @@ std::map<void*, IpcKey> g_ipc_ptrs;  // pointer handed out by etha_ipc_open -> i
 std::map<void*, int> g_ipc_ptr_refs;
 
 int fail(int code, const char* fmt, ...) {
-  char buf[512];
   va_list ap;
   va_start(ap, fmt);
-  vsnprintf(buf, sizeof(buf), fmt, ap);
+  vsnprintf(g_err, sizeof(g_err), fmt, ap);
   va_end(ap);
-  g_err = buf;
   return code;
+}
+
+// Body of an entry point that builds host-side containers: no C++ exception leaves the library (the ABI is
+// plain C); running out of host memory becomes ETHA_ERR_NOMEM.
+template <typename F>
+int guarded(const char* what, F&& body) {
+  try {
+    return body();
+  } catch (const std::bad_alloc&) {
+    return fail(ETHA_ERR_NOMEM, "%s: out of host memory", what);
+  } catch (const std::exception& e) {
+    return fail(ETHA_ERR_INVALID, "%s: %s", what, e.what());
+  } catch (...) {
+    return fail(ETHA_ERR_INVALID, "%s: unexpected exception", what);
+  }
 }
 
 #define HIP_TRY(expr)                                                                      \
@@ -1210,9 +1226,29 @@ struct Builder {
   std::vector<uint32_t> run_begin, row_begin, trans_begin;
   std::vector<uint8_t> is_reduce;
   uint64_t payload_bytes = 0;
+  uint64_t max_bytes = 0;  // 0: no limit.  Else the tile program may take at most this many bytes (tiles only)
 };
 
 constexpr uint64_t kMaxTiles = 0x7fff0000ull / kBlocksPerTile;  // grid.x limit with margin
+
+// Called before tiles are appended: refuses a program that would outgrow the grid limit or the builder's byte
+// budget before the host vectors grow, not after.
+int room_for(const Builder& b, uint32_t idx, uint64_t more_run, uint64_t more_row, uint64_t more_trans) {
+  const uint64_t n_run = b.run.size() + more_run, n_row = b.row.size() + more_row, n_trans = b.trans.size() + more_trans;
+#ifdef ETHA_TEST_THROW_AT_TILE
+  // test builds only: stands in for a host allocation that fails while a program is being compiled
+  if (n_run + n_row + n_trans > (uint64_t)(ETHA_TEST_THROW_AT_TILE)) throw std::bad_alloc();
+#endif
+  if (n_run + n_row > kMaxTiles || n_trans > kMaxTiles)
+    return fail(ETHA_ERR_UNSUPPORTED, "chunk %u: tile program too large (> %llu tiles)", idx, (unsigned long long)kMaxTiles);
+  if (b.max_bytes) {
+    const uint64_t bytes = n_run * sizeof(RunTile) + n_row * sizeof(RowTile) + n_trans * sizeof(TransTile);
+    if (bytes > b.max_bytes)
+      return fail(ETHA_ERR_UNSUPPORTED, "chunk %u: the tile program would take more than %llu bytes; this entry point holds at most %llu",
+                  idx, (unsigned long long)bytes, (unsigned long long)b.max_bytes);
+  }
+  return ETHA_OK;
+}
 
 struct ReduceSpec {
   uint32_t n_peers = 0, peer_first = 0, op = 0, via = 0;
@@ -1289,12 +1325,6 @@ class PairCompiler {
     return false;
   }
 
-  int check_size() const {
-    if (bld_.run.size() + bld_.row.size() > kMaxTiles || bld_.trans.size() > kMaxTiles)
-      return fail(ETHA_ERR_UNSUPPORTED, "tile program too large (> %llu tiles)", (unsigned long long)kMaxTiles);
-    return ETHA_OK;
-  }
-
   // Transposing chunk: no common contiguous dim, but the a side is contiguous along some other dim j while
   // the b side is contiguous along the innermost one.  Such chunks go through the LDS-staged transposing
   // kernel in blocks of trans_dim_a x trans_dim_b elements; all other dims are unrolled here.
@@ -1325,11 +1355,13 @@ class PairCompiler {
       // open on both sides.  Super-blocks follow diagonals of their grid: row-major order would make everything
       // in flight read (or write) one narrow column stripe of rows that lie a power of two apart, i.e. the same
       // few memory channels.
-      auto emit = [&](int64_t dim_j, int64_t dim_k, int64_t j_end, int64_t k_end, int64_t skip_j, int64_t skip_k) {
+      auto emit = [&](int64_t dim_j, int64_t dim_k, int64_t j_end, int64_t k_end, int64_t skip_j, int64_t skip_k) -> int {
         // blocks of dim_j x dim_k over [0, j_end) x [0, k_end), except those inside [0, skip_j) x [0, skip_k)
         const int64_t S = ETHA_TRANS_SUPER;
         const int64_t nbj = (j_end + dim_j - 1) / dim_j, nbk = (k_end + dim_k - 1) / dim_k;
         const int64_t nsj = (nbj + S - 1) / S, nsk = (nbk + S - 1) / S;
+        const int rc_room = room_for(bld_, idx_, 0, 0, (uint64_t)nbj * (uint64_t)nbk);
+        if (rc_room != ETHA_OK) return rc_room;
         for (int64_t d = 0; d < nsk; d++)
           for (int64_t sj = 0; sj < nsj; sj++)
             for (int64_t ij = 0; ij < S; ij++)
@@ -1350,10 +1382,11 @@ class PairCompiler {
                 t.cvt = converting ? (dta_ << 4) | dtb_ : 0u;
                 bld_.trans.push_back(t);
               }
+        return ETHA_OK;
       };
-      if (wide) emit(wide_dim_j, wide_dim_k, wide_j, wide_k, 0, 0);
-      if (!wide || wide_j < n_[j] || wide_k < n_[kk]) emit(kDimJ, kDimK, n_[j], n_[kk], wide ? wide_j : 0, wide ? wide_k : 0);
-      const int rc = check_size();
+      int rc = wide ? emit(wide_dim_j, wide_dim_k, wide_j, wide_k, 0, 0) : ETHA_OK;
+      if (rc == ETHA_OK && (!wide || wide_j < n_[j] || wide_k < n_[kk]))
+        rc = emit(kDimJ, kDimK, n_[j], n_[kk], wide ? wide_j : 0, wide ? wide_k : 0);
       if (rc != ETHA_OK) return rc;
     } while (next_position(k_, pos, &off_a, &off_b, j, kk));
     *done = true;
@@ -1427,6 +1460,8 @@ class PairCompiler {
       const uint64_t head = (16 - (b0 & 15)) & 15;
       const uint64_t body_units = (run_bytes - head) / 16;
       const uint64_t tail = run_bytes - head - body_units * 16;
+      const int rc = room_for(bld_, idx_, 2 + (body_units + kTileThreads - 1) / kTileThreads, 0, 0);
+      if (rc != ETHA_OK) return rc;
       narrow(a0, b0, head);
       for (uint64_t q = 0; q < body_units; q += kTileThreads) {
         RunTile t;
@@ -1437,8 +1472,6 @@ class PairCompiler {
         bld_.run.push_back(t);
       }
       narrow(a0 + head + body_units * 16, b0 + head + body_units * 16, tail);
-      const int rc = check_size();
-      if (rc != ETHA_OK) return rc;
     } while (next_position(k_, pos, &off_a, &off_b));
     return ETHA_OK;
   }
@@ -1482,6 +1515,8 @@ class PairCompiler {
     do {
       const uint64_t a0 = base_a + off_a, b0 = base_b + off_b;
       if (!use_rows) {
+        const int rc = room_for(bld_, idx_, (run_units + kTileThreads - 1) / kTileThreads, 0, 0);
+        if (rc != ETHA_OK) return rc;
         for (uint64_t q = 0; q < run_units; q += kTileThreads) {
           RunTile t;
           t.a = a0 + q * ua;
@@ -1495,6 +1530,8 @@ class PairCompiler {
         const int64_t pa = k_ > 0 ? sa_[k_ - 1] : 0, pb = k_ > 0 ? sb_[k_ - 1] : 0;
         const uint64_t total = rows * run_units;
         const uint64_t step = kTileThreads;
+        const int rc = room_for(bld_, idx_, 0, (total + step - 1) / step, 0);
+        if (rc != ETHA_OK) return rc;
         for (uint64_t q = 0; q < total; q += step) {
           RowTile t;
           memset(&t, 0, sizeof(t));
@@ -1522,8 +1559,6 @@ class PairCompiler {
           bld_.row.push_back(t);
         }
       }
-      const int rc = check_size();
-      if (rc != ETHA_OK) return rc;
     } while (next_position(outer, pos, &off_a, &off_b));
     return ETHA_OK;
   }
@@ -1568,6 +1603,10 @@ struct EthaTable {
   uint64_t payload_bytes = 0;
   uint64_t device_bytes = 0;
   bool uploaded = false;
+  // identity for schedules that hold launches of this table: `serial` is unique per table ever created in the
+  // process, `version` changes when the launches of a chunk range change (a range gains a write-ordered copy)
+  uint64_t serial = 0;
+  uint32_t version = 0;
   // write-ordered copies of the tiles of ranges that are always launched as one unit
   struct Ordered {
     std::vector<RunTile> h_run;
@@ -1582,6 +1621,11 @@ struct EthaTable {
 };
 
 namespace {
+
+// tables that exist, by address -> serial; a schedule checks its tables against this before it launches
+std::mutex g_tables_mutex;
+std::map<const EthaTable*, uint64_t> g_live_tables;
+uint64_t g_next_table_serial = 1;
 
 int upload_table(EthaTable* t) {
   if (!t->h_run.empty()) {
@@ -1614,6 +1658,10 @@ int upload_table(EthaTable* t) {
 
 void free_table(EthaTable* t) {
   if (!t) return;
+  {
+    std::lock_guard<std::mutex> lock(g_tables_mutex);
+    g_live_tables.erase(t);
+  }
   if (t->d_run) (void)hipFree(t->d_run);
   if (t->d_row) (void)hipFree(t->d_row);
   if (t->d_peers) (void)hipFree(t->d_peers);
@@ -1626,24 +1674,34 @@ void free_table(EthaTable* t) {
   delete t;
 }
 
-int finish_table(Builder& bld, EthaTable* t, int upload, EthaTable** out) {
-  t->h_run.swap(bld.run);
-  t->h_row.swap(bld.row);
-  t->h_trans.swap(bld.trans);
-  t->run_begin.swap(bld.run_begin);
-  t->row_begin.swap(bld.row_begin);
-  t->trans_begin.swap(bld.trans_begin);
-  for (const TransTile& tt : t->h_trans)
-    if (trans_lds_bytes(1u << tt.es_log2) > t->trans_lds) t->trans_lds = trans_lds_bytes(1u << tt.es_log2);
-  t->reduce_prefix.assign(t->n_chunks + 1, 0);
-  for (uint32_t i = 0; i < t->n_chunks; i++) t->reduce_prefix[i + 1] = t->reduce_prefix[i] + bld.is_reduce[i];
-  t->payload_bytes = bld.payload_bytes;
-  if (upload) {
-    const int rc = upload_table(t);
-    if (rc != ETHA_OK) {
-      free_table(t);
-      return rc;
+// Takes ownership of t: on any failure (an exception included) the table is freed.
+int finish_table(Builder& bld, EthaTable* t, const uint64_t* partial_ptrs, uint32_t n_partial_ptrs, int upload, EthaTable** out) {
+  try {
+    if (partial_ptrs && n_partial_ptrs) t->h_peers.assign(partial_ptrs, partial_ptrs + n_partial_ptrs);
+    t->h_run.swap(bld.run);
+    t->h_row.swap(bld.row);
+    t->h_trans.swap(bld.trans);
+    t->run_begin.swap(bld.run_begin);
+    t->row_begin.swap(bld.row_begin);
+    t->trans_begin.swap(bld.trans_begin);
+    for (const TransTile& tt : t->h_trans)
+      if (trans_lds_bytes(1u << tt.es_log2) > t->trans_lds) t->trans_lds = trans_lds_bytes(1u << tt.es_log2);
+    t->reduce_prefix.assign(t->n_chunks + 1, 0);
+    for (uint32_t i = 0; i < t->n_chunks; i++) t->reduce_prefix[i + 1] = t->reduce_prefix[i] + bld.is_reduce[i];
+    t->payload_bytes = bld.payload_bytes;
+    if (upload) {
+      const int rc = upload_table(t);
+      if (rc != ETHA_OK) {
+        free_table(t);
+        return rc;
+      }
     }
+    std::lock_guard<std::mutex> lock(g_tables_mutex);
+    t->serial = g_next_table_serial++;
+    g_live_tables[t] = t->serial;
+  } catch (...) {
+    free_table(t);
+    throw;
   }
   *out = t;
   return ETHA_OK;
@@ -1668,18 +1726,118 @@ std::atomic<uint64_t> g_kernel_launches{0};
 template <typename... Args, typename F>
 void launch_kernel(F kernel, dim3 grid, dim3 block, size_t lds, void* stream, uint32_t flags, Args... args) {
   g_kernel_launches.fetch_add(1, std::memory_order_relaxed);
-  if (flags & ETHA_LAUNCH_UNORDERED) {
-    // a stream under capture records its kernels as a chain: the flag has no meaning there
-    hipStreamCaptureStatus capture = hipStreamCaptureStatusNone;
-    if (hipStreamIsCapturing((hipStream_t)stream, &capture) != hipSuccess || capture != hipStreamCaptureStatusNone)
-      flags &= ~(uint32_t)ETHA_LAUNCH_UNORDERED;
-  }
   if (flags & ETHA_LAUNCH_UNORDERED)
     hipExtLaunchKernelGGL(kernel, grid, block, (uint32_t)lds, (hipStream_t)stream, nullptr, nullptr, hipExtAnyOrderLaunch,
                           args...);
   else
     hipLaunchKernelGGL(kernel, grid, block, lds, (hipStream_t)stream, args...);
 }
+
+// One kernel launch with everything resolved: which kernel, its grid and its arguments.  Every entry point
+// first plans its launches into a list of these and then issues the list; a schedule (etha_schedule_create)
+// keeps such lists, so that re-issuing a whole transfer is a loop over ready-made launches.
+enum : uint32_t { kKernelTile = 0, kKernelTile2D, kKernelGather, kKernelMixed, kKernelTrans, kKernelTrans2D, kKernelReduce };
+const char* const kKernelNames[] = {"etha_tile_kernel", "etha_tile_kernel_2d", "etha_gather_kernel", "etha_unpack_mixed_kernel",
+                                    "etha_transpose_kernel", "etha_transpose_kernel_2d", "etha_reduce_kernel"};
+
+struct PreparedLaunch {
+  uint32_t kernel;  // kKernel*
+  uint32_t rev;     // direction of the tile and transposing kernels (unpack = 1)
+  uint32_t flags;   // ETHA_LAUNCH_UNORDERED or 0
+  uint32_t gx, gy, block, lds;
+  union Args {
+    struct {  // kKernelTile, kKernelMixed
+      const RunTile* run;
+      const RowTile* row;
+      const uint64_t* gather;
+      uint32_t n_run, n_plain, n_gather;
+    } tile;
+    struct {
+      const TransTile* tiles;
+    } trans;
+    struct {
+      const RowTile* row;
+      const uint64_t* peers;
+    } reduce;
+    Args2D a2d;     // kKernelTile2D, kKernelGather
+    TransArgs t2d;  // kKernelTrans2D
+  } u;
+};
+
+PreparedLaunch new_launch(uint32_t kernel, bool rev, uint32_t flags, uint32_t gx, uint32_t gy, uint32_t block, uint32_t lds) {
+  PreparedLaunch p;
+  memset(&p, 0, sizeof(p));
+  p.kernel = kernel;
+  p.rev = rev ? 1u : 0u;
+  p.flags = flags;
+  p.gx = gx;
+  p.gy = gy;
+  p.block = block;
+  p.lds = lds;
+  return p;
+}
+
+void issue_one(const PreparedLaunch& p, void* stream, uint32_t flags) {
+  const dim3 grid(p.gx, p.gy), block(p.block);
+  switch (p.kernel) {
+    case kKernelTile:
+      if (p.rev)
+        launch_kernel(etha_tile_kernel<true>, grid, block, 0, stream, flags, p.u.tile.run, p.u.tile.n_run, p.u.tile.row, p.u.tile.gather);
+      else
+        launch_kernel(etha_tile_kernel<false>, grid, block, 0, stream, flags, p.u.tile.run, p.u.tile.n_run, p.u.tile.row, p.u.tile.gather);
+      break;
+    case kKernelTile2D:
+      if (p.rev)
+        launch_kernel(etha_tile_kernel_2d<true>, grid, block, 0, stream, flags, p.u.a2d);
+      else
+        launch_kernel(etha_tile_kernel_2d<false>, grid, block, 0, stream, flags, p.u.a2d);
+      break;
+    case kKernelGather:
+      launch_kernel(etha_gather_kernel, grid, block, 0, stream, flags, p.u.a2d);
+      break;
+    case kKernelMixed:
+      launch_kernel(etha_unpack_mixed_kernel, grid, block, 0, stream, flags, p.u.tile.run, p.u.tile.row, p.u.tile.gather,
+                    p.u.tile.n_run, p.u.tile.n_plain, p.u.tile.n_gather);
+      break;
+    case kKernelTrans:
+      if (p.rev)
+        launch_kernel(etha_transpose_kernel<true>, grid, block, p.lds, stream, flags, p.u.trans.tiles);
+      else
+        launch_kernel(etha_transpose_kernel<false>, grid, block, p.lds, stream, flags, p.u.trans.tiles);
+      break;
+    case kKernelTrans2D:
+      if (p.rev)
+        launch_kernel(etha_transpose_kernel_2d<true>, grid, block, p.lds, stream, flags, p.u.t2d);
+      else
+        launch_kernel(etha_transpose_kernel_2d<false>, grid, block, p.lds, stream, flags, p.u.t2d);
+      break;
+    default:
+      launch_kernel(etha_reduce_kernel, grid, block, 0, stream, flags, p.u.reduce.row, p.u.reduce.peers);
+      break;
+  }
+}
+
+// Issues the launches in list order; each one is checked, so that a failure names the launch it belongs to.
+// A stream under capture records its kernels as a chain: the unordered flag has no meaning there and is dropped.
+int issue_all(const PreparedLaunch* list, size_t n, void* stream) {
+  bool capturing = false;
+  for (size_t i = 0; i < n; i++)
+    if (list[i].flags & ETHA_LAUNCH_UNORDERED) {
+      hipStreamCaptureStatus capture = hipStreamCaptureStatusNone;
+      capturing = hipStreamIsCapturing((hipStream_t)stream, &capture) != hipSuccess || capture != hipStreamCaptureStatusNone;
+      break;
+    }
+  for (size_t i = 0; i < n; i++) {
+    issue_one(list[i], stream, capturing ? 0u : list[i].flags);
+    const hipError_t e = hipGetLastError();
+    if (e != hipSuccess)
+      return fail(ETHA_ERR_HIP, "launch %zu of %zu (%s, grid %u x %u): %s", i + 1, n, kKernelNames[list[i].kernel], list[i].gx,
+                  list[i].gy, hipGetErrorString(e));
+  }
+  return ETHA_OK;
+}
+
+typedef std::vector<PreparedLaunch> LaunchList;
 
 // the plain (run and row) tiles of a chunk range, as the tile kernels take them
 Seg2D tile_range(const EthaTable* t, uint32_t first, uint32_t count, bool rev) {
@@ -1714,54 +1872,61 @@ Seg2D gather_range(const EthaTable* t, uint32_t first, uint32_t count, bool rev)
 // workgroups of a gather launch over `tiles` tiles: 8 tiles x 16 pieces per 128 workgroups
 uint32_t gather_grid(uint32_t tiles) { return ((tiles + 7u) / 8u) * 128u; }
 
-void launch_gather(const Seg2D* segs, uint32_t n, uint32_t top, void* stream, uint32_t flags) {
-  Args2D args;
-  memset(&args, 0, sizeof(args));
-  for (uint32_t k = 0; k < n; k++) args.seg[k] = segs[k];
-  launch_kernel(etha_gather_kernel, dim3(gather_grid(top), n), dim3(kBlockThreads), 0, stream, flags, args);
+void plan_gather(const Seg2D* segs, uint32_t n, uint32_t top, uint32_t flags, LaunchList& out) {
+  PreparedLaunch p = new_launch(kKernelGather, true, flags, gather_grid(top), n, kBlockThreads, 0);
+  for (uint32_t k = 0; k < n; k++) p.u.a2d.seg[k] = segs[k];
+  out.push_back(p);
 }
 
-// transposing chunks run in their own kernel (it needs LDS); true when one was launched
-bool launch_trans(const EthaTable* t, uint32_t first, uint32_t count, bool rev, void* stream, uint32_t flags) {
+void plan_plain(const Seg2D& g, bool rev, uint32_t flags, LaunchList& out) {
+  PreparedLaunch p = new_launch(kKernelTile, rev, flags, g.n_tiles * kBlocksPerTile, 1, kBlockThreads, 0);
+  p.u.tile.run = g.run;
+  p.u.tile.row = g.row;
+  p.u.tile.gather = g.gather;
+  p.u.tile.n_run = g.n_run;
+  out.push_back(p);
+}
+
+void plan_trans(const TransTile* tiles, uint32_t n, bool rev, uint32_t lds, uint32_t flags, LaunchList& out) {
+  PreparedLaunch p = new_launch(kKernelTrans, rev, flags, n, 1, kTransThreads, lds);
+  p.u.trans.tiles = tiles;
+  out.push_back(p);
+}
+
+// One chunk range as the single-range entry points run it: the transposing tiles in their kernel, then the
+// plain tiles - and, for an unpack range with a write-ordered copy, its gather tiles in the same launch.
+void plan_tiles(const EthaTable* t, uint32_t first, uint32_t count, bool rev, uint32_t flags, LaunchList& out) {
   const uint32_t x0 = t->trans_begin[first], n_trans = t->trans_begin[first + count] - x0;
-  if (!n_trans) return false;
-  if (rev)
-    launch_kernel(etha_transpose_kernel<true>, dim3(n_trans), dim3(kTransThreads), t->trans_lds, stream, flags,
-                  (const TransTile*)(t->d_trans + x0));
-  else
-    launch_kernel(etha_transpose_kernel<false>, dim3(n_trans), dim3(kTransThreads), t->trans_lds, stream, flags,
-                  (const TransTile*)(t->d_trans + x0));
-  return true;
-}
-
-void launch_plain(const Seg2D& g, bool rev, void* stream, uint32_t flags) {
-  if (rev)
-    launch_kernel(etha_tile_kernel<true>, dim3(g.n_tiles * kBlocksPerTile), dim3(kBlockThreads), 0, stream, flags, g.run, g.n_run,
-                  g.row, g.gather);
-  else
-    launch_kernel(etha_tile_kernel<false>, dim3(g.n_tiles * kBlocksPerTile), dim3(kBlockThreads), 0, stream, flags, g.run, g.n_run,
-                  g.row, g.gather);
-}
-
-template <bool REV>
-int launch_tiles(const EthaTable* t, uint32_t first, uint32_t count, void* stream, uint32_t flags) {
-  if (launch_trans(t, first, count, REV, stream, flags)) {
-    HIP_TRY(hipGetLastError());
+  if (n_trans) {
+    plan_trans(t->d_trans + x0, n_trans, rev, t->trans_lds, flags, out);
     flags |= ETHA_LAUNCH_UNORDERED;  // the two kernels of one call touch different chunks
   }
-  const Seg2D g = tile_range(t, first, count, REV);
-  const Seg2D gathered = gather_range(t, first, count, REV);
+  const Seg2D g = tile_range(t, first, count, rev);
+  const Seg2D gathered = gather_range(t, first, count, rev);
   if (g.n_tiles && gathered.n_tiles) {  // the gather tiles follow the plain row tiles in the ordered copy
     const uint32_t groups = ((g.n_tiles * kBlocksPerTile + 127u) & ~127u) + gather_grid(gathered.n_tiles);
-    launch_kernel(etha_unpack_mixed_kernel, dim3(groups), dim3(kBlockThreads), 0, stream, flags, g.run, g.row, g.gather, g.n_run,
-                  g.n_tiles, gathered.n_tiles);
+    PreparedLaunch p = new_launch(kKernelMixed, true, flags, groups, 1, kBlockThreads, 0);
+    p.u.tile.run = g.run;
+    p.u.tile.row = g.row;
+    p.u.tile.gather = g.gather;
+    p.u.tile.n_run = g.n_run;
+    p.u.tile.n_plain = g.n_tiles;
+    p.u.tile.n_gather = gathered.n_tiles;
+    out.push_back(p);
   } else if (g.n_tiles) {
-    launch_plain(g, REV, stream, flags);
+    plan_plain(g, rev, flags, out);
   } else if (gathered.n_tiles) {
-    launch_gather(&gathered, 1, gathered.n_tiles, stream, flags);
+    plan_gather(&gathered, 1, gathered.n_tiles, flags, out);
   }
-  HIP_TRY(hipGetLastError());
-  return ETHA_OK;
+}
+
+void plan_reduce(const EthaTable* t, uint32_t first, uint32_t count, uint32_t flags, LaunchList& out) {
+  const uint32_t w0 = t->row_begin[first], w1 = t->row_begin[first + count];
+  if (w1 == w0) return;
+  PreparedLaunch p = new_launch(kKernelReduce, false, flags, (w1 - w0) * kBlocksPerTile, 1, kBlockThreads, 0);
+  p.u.reduce.row = t->d_row + w0;
+  p.u.reduce.peers = t->d_peers;
+  out.push_back(p);
 }
 
 // Segments of one direction, largest first: those of (nearly) the same size share a launch.  A workgroup that a
@@ -1771,7 +1936,7 @@ int launch_tiles(const EthaTable* t, uint32_t first, uint32_t count, void* strea
 constexpr uint64_t kJoinMaxIdleTiles = 6000 / kBlocksPerTile;
 
 template <typename SEG, typename COUNT, typename LAUNCH>
-void launch_neighbours(std::vector<SEG>& segs, uint64_t max_idle, COUNT count_of, LAUNCH launch, uint32_t& flags) {
+void plan_neighbours(std::vector<SEG>& segs, uint64_t max_idle, COUNT count_of, LAUNCH launch, uint32_t& flags) {
   std::stable_sort(segs.begin(), segs.end(), [&](const SEG& x, const SEG& y) { return count_of(x) > count_of(y); });
   size_t i = 0;
   while (i < segs.size()) {
@@ -1791,19 +1956,14 @@ void launch_neighbours(std::vector<SEG>& segs, uint64_t max_idle, COUNT count_of
   }
 }
 
-void launch_group(std::vector<Seg2D>& segs, bool rev, void* stream, uint32_t& flags) {
-  launch_neighbours(
+void plan_group(std::vector<Seg2D>& segs, bool rev, uint32_t& flags, LaunchList& out) {
+  plan_neighbours(
       segs, kJoinMaxIdleTiles, [](const Seg2D& g) { return (uint64_t)g.n_tiles; },
       [&](size_t i, size_t j, uint32_t top, uint32_t fl) {
-        if (j - i == 1) return launch_plain(segs[i], rev, stream, fl);
-        Args2D args;
-        memset(&args, 0, sizeof(args));
-        for (size_t k = i; k < j; k++) args.seg[k - i] = segs[k];
-        const dim3 grid(top * kBlocksPerTile, (uint32_t)(j - i));
-        if (rev)
-          launch_kernel(etha_tile_kernel_2d<true>, grid, dim3(kBlockThreads), 0, stream, fl, args);
-        else
-          launch_kernel(etha_tile_kernel_2d<false>, grid, dim3(kBlockThreads), 0, stream, fl, args);
+        if (j - i == 1) return plan_plain(segs[i], rev, fl, out);
+        PreparedLaunch p = new_launch(kKernelTile2D, rev, fl, top * kBlocksPerTile, (uint32_t)(j - i), kBlockThreads, 0);
+        for (size_t k = i; k < j; k++) p.u.a2d.seg[k - i] = segs[k];
+        out.push_back(p);
       },
       flags);
 }
@@ -1811,36 +1971,16 @@ void launch_group(std::vector<Seg2D>& segs, bool rev, void* stream, uint32_t& fl
 // the same for transposing tiles (one workgroup of kTransThreads work-items per tile)
 constexpr uint64_t kTransJoinMaxIdleTiles = 64;
 
-void launch_trans_group(std::vector<TransSeg>& segs, bool rev, uint32_t lds, void* stream, uint32_t& flags) {
-  launch_neighbours(
+void plan_trans_group(std::vector<TransSeg>& segs, bool rev, uint32_t lds, uint32_t& flags, LaunchList& out) {
+  plan_neighbours(
       segs, kTransJoinMaxIdleTiles, [](const TransSeg& g) { return (uint64_t)g.n; },
       [&](size_t i, size_t j, uint32_t top, uint32_t fl) {
-        if (j - i == 1) {
-          if (rev)
-            launch_kernel(etha_transpose_kernel<true>, dim3(segs[i].n), dim3(kTransThreads), lds, stream, fl, segs[i].tiles);
-          else
-            launch_kernel(etha_transpose_kernel<false>, dim3(segs[i].n), dim3(kTransThreads), lds, stream, fl, segs[i].tiles);
-          return;
-        }
-        TransArgs args;
-        memset(&args, 0, sizeof(args));
-        for (size_t k = i; k < j; k++) args.seg[k - i] = segs[k];
-        const dim3 grid(top, (uint32_t)(j - i));
-        if (rev)
-          launch_kernel(etha_transpose_kernel_2d<true>, grid, dim3(kTransThreads), lds, stream, fl, args);
-        else
-          launch_kernel(etha_transpose_kernel_2d<false>, grid, dim3(kTransThreads), lds, stream, fl, args);
+        if (j - i == 1) return plan_trans(segs[i].tiles, segs[i].n, rev, lds, fl, out);
+        PreparedLaunch p = new_launch(kKernelTrans2D, rev, fl, top, (uint32_t)(j - i), kTransThreads, lds);
+        for (size_t k = i; k < j; k++) p.u.t2d.seg[k - i] = segs[k];
+        out.push_back(p);
       },
       flags);
-}
-
-int launch_reduce(const EthaTable* t, uint32_t first, uint32_t count, void* stream, uint32_t flags) {
-  const uint32_t w0 = t->row_begin[first], w1 = t->row_begin[first + count];
-  if (w1 == w0) return ETHA_OK;
-  launch_kernel(etha_reduce_kernel, dim3((w1 - w0) * kBlocksPerTile), dim3(kBlockThreads), 0, stream, flags,
-                (const RowTile*)(t->d_row + w0), (const uint64_t*)t->d_peers);
-  HIP_TRY(hipGetLastError());
-  return ETHA_OK;
 }
 
 // Pieces of one destination row that arrive through different chunks (a target row assembled from several source
@@ -1945,7 +2085,92 @@ int check_flags(uint32_t flags) {
   return ETHA_OK;
 }
 
+int check_segment(const EthaSegment& g, uint32_t i) {
+  if (g.kind > ETHA_SEG_SELFCOPY) return fail(ETHA_ERR_INVALID, "segment %u: unknown kind %u", i, g.kind);
+  const int rc = check_range(g.table, g.first, g.count, g.kind == ETHA_SEG_SELFCOPY ? 1 : 0);
+  if (rc != ETHA_OK) return rc;
+  const uint32_t n_reduce = g.table->reduce_prefix[g.first + g.count] - g.table->reduce_prefix[g.first];
+  if ((g.kind == ETHA_SEG_PACK || g.kind == ETHA_SEG_UNPACK) && n_reduce)
+    return fail(ETHA_ERR_INVALID, "segment %u: range holds Partial chunks", i);
+  if (g.kind == ETHA_SEG_REDUCE_PACK && n_reduce != g.count)
+    return fail(ETHA_ERR_INVALID, "segment %u: range holds chunks that are not Partial chunks", i);
+  if (g.kind == ETHA_SEG_SELFCOPY && n_reduce && n_reduce != g.count)
+    return fail(ETHA_ERR_INVALID, "segment %u: range mixes Partial and plain chunks; launch them separately", i);
+  return ETHA_OK;
+}
+
+// The launches of one chunk range run by itself, as the entry point named by g.kind would run it.
+void plan_single(const EthaSegment& g, uint32_t flags, LaunchList& out) {
+  const EthaTable* t = g.table;
+  if (t->reduce_prefix[g.first + g.count] != t->reduce_prefix[g.first])
+    plan_reduce(t, g.first, g.count, flags, out);
+  else
+    plan_tiles(t, g.first, g.count, g.kind == ETHA_SEG_UNPACK, flags, out);
+}
+
+// The launches of a set of segments that do not depend on each other (validated by the caller).
+void plan_segments(const EthaSegment* segs, uint32_t n_segments, uint32_t flags, LaunchList& out) {
+  std::vector<Seg2D> forward, reverse, gathered;
+  std::vector<TransSeg> trans_forward, trans_reverse;
+  uint32_t trans_lds = 0;
+  for (uint32_t i = 0; i < n_segments; i++) {
+    const EthaSegment& g = segs[i];
+    const EthaTable* t = g.table;
+    if (t->reduce_prefix[g.first + g.count] != t->reduce_prefix[g.first]) {
+      const size_t before = out.size();
+      plan_reduce(t, g.first, g.count, flags, out);
+      if (out.size() != before) flags |= ETHA_LAUNCH_UNORDERED;
+      continue;
+    }
+    const bool rev = g.kind == ETHA_SEG_UNPACK;
+    const uint32_t x0 = t->trans_begin[g.first], n_trans = t->trans_begin[g.first + g.count] - x0;
+    if (n_trans) {
+      (rev ? trans_reverse : trans_forward).push_back(TransSeg{t->d_trans + x0, n_trans, 0});
+      if (t->trans_lds > trans_lds) trans_lds = t->trans_lds;
+    }
+    const Seg2D r = tile_range(t, g.first, g.count, rev);
+    if (r.n_tiles) (rev ? reverse : forward).push_back(r);
+    const Seg2D gr = gather_range(t, g.first, g.count, rev);
+    if (gr.n_tiles) gathered.push_back(gr);
+  }
+  plan_trans_group(trans_forward, false, trans_lds, flags, out);
+  plan_trans_group(trans_reverse, true, trans_lds, flags, out);
+  plan_group(forward, false, flags, out);
+  plan_group(reverse, true, flags, out);
+  plan_neighbours(
+      gathered, kJoinMaxIdleTiles, [](const Seg2D& x) { return (uint64_t)x.n_tiles; },
+      [&](size_t i, size_t j, uint32_t top, uint32_t fl) { plan_gather(&gathered[i], (uint32_t)(j - i), top, fl, out); }, flags);
+}
+
+// launches of the calling thread's current entry-point call; kept between calls so that a transfer's launch calls
+// do not allocate once the list has reached its size
+LaunchList& scratch_launches() {
+  thread_local LaunchList list;
+  list.clear();
+  return list;
+}
+
+int launch_single(const EthaTable* t, uint32_t kind, uint32_t first, uint32_t count, void* stream, uint32_t flags) {
+  return guarded("launch", [&]() -> int {
+    LaunchList& list = scratch_launches();
+    plan_single(EthaSegment{t, kind, first, count, 0}, flags, list);
+    return issue_all(list.data(), list.size(), stream);
+  });
+}
+
 }  // namespace
+
+// A recorded sequence of launch calls, planned once: see etha_schedule_create.
+struct EthaSchedule {
+  LaunchList launches;
+  struct Dep {
+    const EthaTable* table;
+    uint64_t serial;
+    uint32_t version;
+  };
+  std::vector<Dep> deps;
+  uint32_t n_calls = 0;
+};
 
 extern "C" {
 
@@ -1957,84 +2182,85 @@ uint64_t etha_kernel_launches(void) { return g_kernel_launches.load(std::memory_
 // the marker lets a build script find the digest in the file without loading the library
 static const char kSourceDigest[] = "etha-source-digest:" ETHA_SOURCE_HASH;
 const char* etha_source_hash(void) { return kSourceDigest + sizeof("etha-source-digest:") - 1; }
-const char* etha_last_error(void) { return g_err.c_str(); }
+const char* etha_last_error(void) { return g_err; }
 
 int etha_table_create(const EthaChunkDesc* descs, uint32_t n_chunks, const uint64_t* partial_ptrs,
                       uint32_t n_partial_ptrs, int upload, EthaTable** out) {
   if (!out) return fail(ETHA_ERR_INVALID, "null out");
   *out = nullptr;
   if (n_chunks && !descs) return fail(ETHA_ERR_INVALID, "null descriptor array");
-  Builder bld;
-  bld.run_begin.reserve(n_chunks + 1);
-  bld.row_begin.reserve(n_chunks + 1);
-  bld.is_reduce.assign(n_chunks, 0);
-  for (uint32_t i = 0; i < n_chunks; i++) {
-    const EthaChunkDesc& d = descs[i];
+  return guarded("etha_table_create", [&]() -> int {
+    Builder bld;
+    bld.run_begin.reserve(n_chunks + 1);
+    bld.row_begin.reserve(n_chunks + 1);
+    bld.is_reduce.assign(n_chunks, 0);
+    for (uint32_t i = 0; i < n_chunks; i++) {
+      const EthaChunkDesc& d = descs[i];
+      bld.run_begin.push_back((uint32_t)bld.run.size());
+      bld.row_begin.push_back((uint32_t)bld.row.size());
+      bld.trans_begin.push_back((uint32_t)bld.trans.size());
+      const int esw = dtype_size(d.wire_dtype);
+      if (esw == 0) return fail(ETHA_ERR_INVALID, "chunk %u: unknown wire_dtype %u", i, d.wire_dtype);
+      ReduceSpec red;
+      std::vector<uint64_t> peer_bases;
+      Region A;
+      if (d.n_partials) {
+        { const int rc_op = check_reduce_op(d.reduce_op, d.n_partials, i); if (rc_op != ETHA_OK) return rc_op; }
+        if (!partial_ptrs || (uint64_t)d.partial_first + d.n_partials > n_partial_ptrs)
+          return fail(ETHA_ERR_INVALID, "chunk %u: partial pointer range outside partial_ptrs", i);
+        // every peer shares the chunk geometry; validate each peer's range with its own base
+        for (uint32_t p = 0; p < d.n_partials; p++) {
+          Region tmp;
+          EthaChunkDesc dp = d;
+          dp.tensor_lo = dp.tensor_hi = 0;  // the single lo/hi pair cannot describe several peers
+          const int rc = tensor_region(dp, i, partial_ptrs[d.partial_first + p], false, &tmp);
+          if (rc != ETHA_OK) return rc;
+          peer_bases.push_back(partial_ptrs[d.partial_first + p]);
+        }
+        EthaChunkDesc dz = d;
+        dz.tensor_lo = dz.tensor_hi = 0;
+        const int rc = tensor_region(dz, i, 0, true, &A);  // offsets relative to a peer base
+        if (rc != ETHA_OK) return rc;
+        red.n_peers = d.n_partials;
+        red.peer_first = d.partial_first;
+        red.op = d.reduce_op;
+        bld.is_reduce[i] = 1;
+      } else {
+        const int rc = tensor_region(d, i, d.tensor_ptr, false, &A);
+        if (rc != ETHA_OK) return rc;
+      }
+      // bucket side: contiguous, row-major, wire dtype
+      Region B;
+      B.nd = A.nd;
+      B.base = d.bucket_ptr;
+      int64_t acc = esw;
+      for (int j = A.nd - 1; j >= 0; j--) {
+        B.shape[j] = A.shape[j];
+        B.stride[j] = acc;
+        acc *= A.shape[j];
+      }
+      const uint64_t nbytes = region_numel(A) * (uint64_t)esw;
+      if (nbytes) {
+        if (d.bucket_ptr == 0) return fail(ETHA_ERR_INVALID, "chunk %u: null bucket pointer", i);
+        if ((d.bucket_lo || d.bucket_hi) &&
+            (d.bucket_ptr < d.bucket_lo || d.bucket_ptr + nbytes > d.bucket_hi || d.bucket_ptr + nbytes < d.bucket_ptr))
+          return fail(ETHA_ERR_INVALID, "chunk %u: bucket bytes [%llx,%llx) leave the bucket buffer [%llx,%llx)", i,
+                      (unsigned long long)d.bucket_ptr, (unsigned long long)(d.bucket_ptr + nbytes),
+                      (unsigned long long)d.bucket_lo, (unsigned long long)d.bucket_hi);
+      }
+      bld.payload_bytes += nbytes;
+      const int rc = compile_pair(bld, i, A, B, d.tensor_dtype, d.wire_dtype, red, peer_bases);
+      if (rc != ETHA_OK) return rc;
+    }
     bld.run_begin.push_back((uint32_t)bld.run.size());
     bld.row_begin.push_back((uint32_t)bld.row.size());
     bld.trans_begin.push_back((uint32_t)bld.trans.size());
-    const int esw = dtype_size(d.wire_dtype);
-    if (esw == 0) return fail(ETHA_ERR_INVALID, "chunk %u: unknown wire_dtype %u", i, d.wire_dtype);
-    ReduceSpec red;
-    std::vector<uint64_t> peer_bases;
-    Region A;
-    if (d.n_partials) {
-      { const int rc_op = check_reduce_op(d.reduce_op, d.n_partials, i); if (rc_op != ETHA_OK) return rc_op; }
-      if (!partial_ptrs || (uint64_t)d.partial_first + d.n_partials > n_partial_ptrs)
-        return fail(ETHA_ERR_INVALID, "chunk %u: partial pointer range outside partial_ptrs", i);
-      // every peer shares the chunk geometry; validate each peer's range with its own base
-      for (uint32_t p = 0; p < d.n_partials; p++) {
-        Region tmp;
-        EthaChunkDesc dp = d;
-        dp.tensor_lo = dp.tensor_hi = 0;  // the single lo/hi pair cannot describe several peers
-        const int rc = tensor_region(dp, i, partial_ptrs[d.partial_first + p], false, &tmp);
-        if (rc != ETHA_OK) return rc;
-        peer_bases.push_back(partial_ptrs[d.partial_first + p]);
-      }
-      EthaChunkDesc dz = d;
-      dz.tensor_lo = dz.tensor_hi = 0;
-      const int rc = tensor_region(dz, i, 0, true, &A);  // offsets relative to a peer base
-      if (rc != ETHA_OK) return rc;
-      red.n_peers = d.n_partials;
-      red.peer_first = d.partial_first;
-      red.op = d.reduce_op;
-      bld.is_reduce[i] = 1;
-    } else {
-      const int rc = tensor_region(d, i, d.tensor_ptr, false, &A);
-      if (rc != ETHA_OK) return rc;
-    }
-    // bucket side: contiguous, row-major, wire dtype
-    Region B;
-    B.nd = A.nd;
-    B.base = d.bucket_ptr;
-    int64_t acc = esw;
-    for (int j = A.nd - 1; j >= 0; j--) {
-      B.shape[j] = A.shape[j];
-      B.stride[j] = acc;
-      acc *= A.shape[j];
-    }
-    const uint64_t nbytes = region_numel(A) * (uint64_t)esw;
-    if (nbytes) {
-      if (d.bucket_ptr == 0) return fail(ETHA_ERR_INVALID, "chunk %u: null bucket pointer", i);
-      if ((d.bucket_lo || d.bucket_hi) &&
-          (d.bucket_ptr < d.bucket_lo || d.bucket_ptr + nbytes > d.bucket_hi || d.bucket_ptr + nbytes < d.bucket_ptr))
-        return fail(ETHA_ERR_INVALID, "chunk %u: bucket bytes [%llx,%llx) leave the bucket buffer [%llx,%llx)", i,
-                    (unsigned long long)d.bucket_ptr, (unsigned long long)(d.bucket_ptr + nbytes),
-                    (unsigned long long)d.bucket_lo, (unsigned long long)d.bucket_hi);
-    }
-    bld.payload_bytes += nbytes;
-    const int rc = compile_pair(bld, i, A, B, d.tensor_dtype, d.wire_dtype, red, peer_bases);
-    if (rc != ETHA_OK) return rc;
-  }
-  bld.run_begin.push_back((uint32_t)bld.run.size());
-  bld.row_begin.push_back((uint32_t)bld.row.size());
-  bld.trans_begin.push_back((uint32_t)bld.trans.size());
-  EthaTable* t = new (std::nothrow) EthaTable();
-  if (!t) return fail(ETHA_ERR_NOMEM, "out of host memory");
-  t->kind = 0;
-  t->n_chunks = n_chunks;
-  if (partial_ptrs && n_partial_ptrs) t->h_peers.assign(partial_ptrs, partial_ptrs + n_partial_ptrs);
-  return finish_table(bld, t, upload, out);
+    EthaTable* t = new (std::nothrow) EthaTable();
+    if (!t) return fail(ETHA_ERR_NOMEM, "out of host memory");
+    t->kind = 0;
+    t->n_chunks = n_chunks;
+    return finish_table(bld, t, partial_ptrs, n_partial_ptrs, upload, out);
+  });
 }
 
 int etha_direct_table_create(const EthaChunkDesc* src, const EthaChunkDesc* dst, uint32_t n_chunks,
@@ -2042,62 +2268,63 @@ int etha_direct_table_create(const EthaChunkDesc* src, const EthaChunkDesc* dst,
   if (!out) return fail(ETHA_ERR_INVALID, "null out");
   *out = nullptr;
   if (n_chunks && (!src || !dst)) return fail(ETHA_ERR_INVALID, "null descriptor array");
-  Builder bld;
-  bld.is_reduce.assign(n_chunks, 0);
-  for (uint32_t i = 0; i < n_chunks; i++) {
+  return guarded("etha_direct_table_create", [&]() -> int {
+    Builder bld;
+    bld.is_reduce.assign(n_chunks, 0);
+    for (uint32_t i = 0; i < n_chunks; i++) {
+      bld.run_begin.push_back((uint32_t)bld.run.size());
+      bld.row_begin.push_back((uint32_t)bld.row.size());
+      bld.trans_begin.push_back((uint32_t)bld.trans.size());
+      if (dst[i].n_partials) return fail(ETHA_ERR_INVALID, "chunk %u: a destination cannot be Partial", i);
+      Region A, B;
+      ReduceSpec red;
+      std::vector<uint64_t> peer_bases;
+      const EthaChunkDesc& d = src[i];
+      int rc;
+      if (d.n_partials) {
+        { const int rc_op = check_reduce_op(d.reduce_op, d.n_partials, i); if (rc_op != ETHA_OK) return rc_op; }
+        if (!partial_ptrs || (uint64_t)d.partial_first + d.n_partials > n_partial_ptrs)
+          return fail(ETHA_ERR_INVALID, "chunk %u: partial pointer range outside partial_ptrs", i);
+        if (dtype_size(d.wire_dtype) == 0) return fail(ETHA_ERR_INVALID, "chunk %u: unknown wire_dtype %u", i, d.wire_dtype);
+        EthaChunkDesc dz = d;
+        dz.tensor_lo = dz.tensor_hi = 0;  // the single lo/hi pair cannot describe several peers
+        for (uint32_t p = 0; p < d.n_partials; p++) {
+          Region tmp;
+          rc = tensor_region(dz, i, partial_ptrs[d.partial_first + p], false, &tmp);
+          if (rc != ETHA_OK) return rc;
+          peer_bases.push_back(partial_ptrs[d.partial_first + p]);
+        }
+        rc = tensor_region(dz, i, 0, true, &A);  // offsets relative to a peer base
+        if (rc != ETHA_OK) return rc;
+        red.n_peers = d.n_partials;
+        red.peer_first = d.partial_first;
+        red.op = d.reduce_op;
+        // the bucket path rounds the accumulator to the wire dtype first; keep that rounding when it is not the last one
+        if (d.wire_dtype != dst[i].tensor_dtype) {
+          if (!is_float(d.wire_dtype))
+            return fail(ETHA_ERR_UNSUPPORTED, "chunk %u: Partial reduce needs a floating wire dtype", i);
+          red.via = 1 + d.wire_dtype;
+        }
+        bld.is_reduce[i] = 1;
+      } else {
+        rc = tensor_region(d, i, d.tensor_ptr, false, &A);
+        if (rc != ETHA_OK) return rc;
+      }
+      rc = tensor_region(dst[i], i, dst[i].tensor_ptr, false, &B);
+      if (rc != ETHA_OK) return rc;
+      bld.payload_bytes += region_numel(A) * (uint64_t)dtype_size(dst[i].tensor_dtype);
+      rc = compile_pair(bld, i, A, B, d.tensor_dtype, dst[i].tensor_dtype, red, peer_bases);
+      if (rc != ETHA_OK) return rc;
+    }
     bld.run_begin.push_back((uint32_t)bld.run.size());
     bld.row_begin.push_back((uint32_t)bld.row.size());
     bld.trans_begin.push_back((uint32_t)bld.trans.size());
-    if (dst[i].n_partials) return fail(ETHA_ERR_INVALID, "chunk %u: a destination cannot be Partial", i);
-    Region A, B;
-    ReduceSpec red;
-    std::vector<uint64_t> peer_bases;
-    const EthaChunkDesc& d = src[i];
-    int rc;
-    if (d.n_partials) {
-      { const int rc_op = check_reduce_op(d.reduce_op, d.n_partials, i); if (rc_op != ETHA_OK) return rc_op; }
-      if (!partial_ptrs || (uint64_t)d.partial_first + d.n_partials > n_partial_ptrs)
-        return fail(ETHA_ERR_INVALID, "chunk %u: partial pointer range outside partial_ptrs", i);
-      if (dtype_size(d.wire_dtype) == 0) return fail(ETHA_ERR_INVALID, "chunk %u: unknown wire_dtype %u", i, d.wire_dtype);
-      EthaChunkDesc dz = d;
-      dz.tensor_lo = dz.tensor_hi = 0;  // the single lo/hi pair cannot describe several peers
-      for (uint32_t p = 0; p < d.n_partials; p++) {
-        Region tmp;
-        rc = tensor_region(dz, i, partial_ptrs[d.partial_first + p], false, &tmp);
-        if (rc != ETHA_OK) return rc;
-        peer_bases.push_back(partial_ptrs[d.partial_first + p]);
-      }
-      rc = tensor_region(dz, i, 0, true, &A);  // offsets relative to a peer base
-      if (rc != ETHA_OK) return rc;
-      red.n_peers = d.n_partials;
-      red.peer_first = d.partial_first;
-      red.op = d.reduce_op;
-      // the bucket path rounds the accumulator to the wire dtype first; keep that rounding when it is not the last one
-      if (d.wire_dtype != dst[i].tensor_dtype) {
-        if (!is_float(d.wire_dtype))
-          return fail(ETHA_ERR_UNSUPPORTED, "chunk %u: Partial reduce needs a floating wire dtype", i);
-        red.via = 1 + d.wire_dtype;
-      }
-      bld.is_reduce[i] = 1;
-    } else {
-      rc = tensor_region(d, i, d.tensor_ptr, false, &A);
-      if (rc != ETHA_OK) return rc;
-    }
-    rc = tensor_region(dst[i], i, dst[i].tensor_ptr, false, &B);
-    if (rc != ETHA_OK) return rc;
-    bld.payload_bytes += region_numel(A) * (uint64_t)dtype_size(dst[i].tensor_dtype);
-    rc = compile_pair(bld, i, A, B, d.tensor_dtype, dst[i].tensor_dtype, red, peer_bases);
-    if (rc != ETHA_OK) return rc;
-  }
-  bld.run_begin.push_back((uint32_t)bld.run.size());
-  bld.row_begin.push_back((uint32_t)bld.row.size());
-  bld.trans_begin.push_back((uint32_t)bld.trans.size());
-  EthaTable* t = new (std::nothrow) EthaTable();
-  if (!t) return fail(ETHA_ERR_NOMEM, "out of host memory");
-  t->kind = 1;
-  t->n_chunks = n_chunks;
-  if (partial_ptrs && n_partial_ptrs) t->h_peers.assign(partial_ptrs, partial_ptrs + n_partial_ptrs);
-  return finish_table(bld, t, upload, out);
+    EthaTable* t = new (std::nothrow) EthaTable();
+    if (!t) return fail(ETHA_ERR_NOMEM, "out of host memory");
+    t->kind = 1;
+    t->n_chunks = n_chunks;
+    return finish_table(bld, t, partial_ptrs, n_partial_ptrs, upload, out);
+  });
 }
 
 int etha_selfcopy_table_create(const EthaChunkDesc* src, const EthaChunkDesc* dst, uint32_t n_chunks, int upload,
@@ -2162,46 +2389,49 @@ int etha_table_optimize_range(EthaTable* t, uint32_t first, uint32_t count) {
   if (!t) return fail(ETHA_ERR_INVALID, "null table");
   if ((uint64_t)first + count > t->n_chunks)
     return fail(ETHA_ERR_INVALID, "chunk range [%u,%u) exceeds table of %u chunks", first, first + count, t->n_chunks);
-  if (t->reduce_prefix[first + count] != t->reduce_prefix[first]) return ETHA_OK;  // reduce-pack writes buckets: already ordered
-  const auto key = std::make_pair(first, count);
-  if (t->ordered.count(key)) return ETHA_OK;
-  EthaTable::Ordered o;
-  const bool by_a = t->kind == 0;  // unpack writes the tensor (a) side; a self-copy writes its b side
-  std::vector<RowTile> gather_tiles;
-  std::vector<char> replaced(count, 0);
-  if (by_a) gather_sibling_chunks(t, first, count, gather_tiles, o.h_gather, replaced);
-  o.h_run.assign(t->h_run.begin() + t->run_begin[first], t->h_run.begin() + t->run_begin[first + count]);
-  for (uint32_t c = first; c < first + count; c++)
-    if (!replaced[c - first]) o.h_row.insert(o.h_row.end(), t->h_row.begin() + t->row_begin[c], t->h_row.begin() + t->row_begin[c + 1]);
-  const auto unit = [](uint32_t meta, bool a_side) { return 1ull << ((meta >> (a_side ? kMetaUaShift : kMetaUbShift)) & 15u); };
-  std::stable_sort(o.h_run.begin(), o.h_run.end(),
-                   [by_a](const RunTile& x, const RunTile& y) { return by_a ? x.a < y.a : x.b < y.b; });
-  std::stable_sort(o.h_row.begin(), o.h_row.end(), [by_a, unit](const RowTile& x, const RowTile& y) {
-    const uint64_t px = (by_a ? x.a : x.b) + x.c0 * unit(x.meta, by_a), py = (by_a ? y.a : y.b) + y.c0 * unit(y.meta, by_a);
-    return px < py;
-  });
-  o.n_plain_rows = (uint32_t)o.h_row.size();
-  o.h_row.insert(o.h_row.end(), gather_tiles.begin(), gather_tiles.end());  // in address order already
-  if (t->uploaded) {
-    const size_t run_bytes = o.h_run.size() * sizeof(RunTile), row_bytes = o.h_row.size() * sizeof(RowTile);
-    const size_t gather_bytes = o.h_gather.size() * sizeof(uint64_t);
-    hipError_t e = hipSuccess;
-    if (run_bytes) e = hipMalloc(&o.d_run, run_bytes);
-    if (e == hipSuccess && run_bytes) e = hipMemcpy(o.d_run, o.h_run.data(), run_bytes, hipMemcpyHostToDevice);
-    if (e == hipSuccess && row_bytes) e = hipMalloc(&o.d_row, row_bytes);
-    if (e == hipSuccess && row_bytes) e = hipMemcpy(o.d_row, o.h_row.data(), row_bytes, hipMemcpyHostToDevice);
-    if (e == hipSuccess && gather_bytes) e = hipMalloc(&o.d_gather, gather_bytes);
-    if (e == hipSuccess && gather_bytes) e = hipMemcpy(o.d_gather, o.h_gather.data(), gather_bytes, hipMemcpyHostToDevice);
-    if (e != hipSuccess) {
-      if (o.d_run) (void)hipFree(o.d_run);
-      if (o.d_row) (void)hipFree(o.d_row);
-      if (o.d_gather) (void)hipFree(o.d_gather);
-      return fail(ETHA_ERR_HIP, "uploading the ordered range: %s", hipGetErrorString(e));
+  return guarded("etha_table_optimize_range", [&]() -> int {
+    if (t->reduce_prefix[first + count] != t->reduce_prefix[first]) return ETHA_OK;  // reduce-pack writes buckets: already ordered
+    const auto key = std::make_pair(first, count);
+    if (t->ordered.count(key)) return ETHA_OK;
+    EthaTable::Ordered o;
+    const bool by_a = t->kind == 0;  // unpack writes the tensor (a) side; a self-copy writes its b side
+    std::vector<RowTile> gather_tiles;
+    std::vector<char> replaced(count, 0);
+    if (by_a) gather_sibling_chunks(t, first, count, gather_tiles, o.h_gather, replaced);
+    o.h_run.assign(t->h_run.begin() + t->run_begin[first], t->h_run.begin() + t->run_begin[first + count]);
+    for (uint32_t c = first; c < first + count; c++)
+      if (!replaced[c - first]) o.h_row.insert(o.h_row.end(), t->h_row.begin() + t->row_begin[c], t->h_row.begin() + t->row_begin[c + 1]);
+    const auto unit = [](uint32_t meta, bool a_side) { return 1ull << ((meta >> (a_side ? kMetaUaShift : kMetaUbShift)) & 15u); };
+    std::stable_sort(o.h_run.begin(), o.h_run.end(),
+                     [by_a](const RunTile& x, const RunTile& y) { return by_a ? x.a < y.a : x.b < y.b; });
+    std::stable_sort(o.h_row.begin(), o.h_row.end(), [by_a, unit](const RowTile& x, const RowTile& y) {
+      const uint64_t px = (by_a ? x.a : x.b) + x.c0 * unit(x.meta, by_a), py = (by_a ? y.a : y.b) + y.c0 * unit(y.meta, by_a);
+      return px < py;
+    });
+    o.n_plain_rows = (uint32_t)o.h_row.size();
+    o.h_row.insert(o.h_row.end(), gather_tiles.begin(), gather_tiles.end());  // in address order already
+    if (t->uploaded) {
+      const size_t run_bytes = o.h_run.size() * sizeof(RunTile), row_bytes = o.h_row.size() * sizeof(RowTile);
+      const size_t gather_bytes = o.h_gather.size() * sizeof(uint64_t);
+      hipError_t e = hipSuccess;
+      if (run_bytes) e = hipMalloc(&o.d_run, run_bytes);
+      if (e == hipSuccess && run_bytes) e = hipMemcpy(o.d_run, o.h_run.data(), run_bytes, hipMemcpyHostToDevice);
+      if (e == hipSuccess && row_bytes) e = hipMalloc(&o.d_row, row_bytes);
+      if (e == hipSuccess && row_bytes) e = hipMemcpy(o.d_row, o.h_row.data(), row_bytes, hipMemcpyHostToDevice);
+      if (e == hipSuccess && gather_bytes) e = hipMalloc(&o.d_gather, gather_bytes);
+      if (e == hipSuccess && gather_bytes) e = hipMemcpy(o.d_gather, o.h_gather.data(), gather_bytes, hipMemcpyHostToDevice);
+      if (e != hipSuccess) {
+        if (o.d_run) (void)hipFree(o.d_run);
+        if (o.d_row) (void)hipFree(o.d_row);
+        if (o.d_gather) (void)hipFree(o.d_gather);
+        return fail(ETHA_ERR_HIP, "uploading the ordered range: %s", hipGetErrorString(e));
+      }
+      t->device_bytes += run_bytes + row_bytes + gather_bytes;
     }
-    t->device_bytes += run_bytes + row_bytes + gather_bytes;
-  }
-  t->ordered.emplace(key, std::move(o));
-  return ETHA_OK;
+    t->ordered.emplace(key, std::move(o));
+    t->version++;  // launches of this range planned earlier (schedules) no longer describe what a launch does now
+    return ETHA_OK;
+  });
 }
 
 int etha_table_read_ordered(const EthaTable* t, uint32_t first, uint32_t count, int which, void* out, uint64_t cap_bytes,
@@ -2227,7 +2457,7 @@ int etha_pack_bucket(const EthaTable* t, uint32_t first, uint32_t count, void* s
   if (rc != ETHA_OK) return rc;
   if (t->reduce_prefix[first + count] != t->reduce_prefix[first])
     return fail(ETHA_ERR_INVALID, "range holds Partial chunks; use etha_reduce_pack_bucket");
-  return launch_tiles<false>(t, first, count, stream, flags);
+  return launch_single(t, ETHA_SEG_PACK, first, count, stream, flags);
 }
 
 int etha_unpack_bucket(const EthaTable* t, uint32_t first, uint32_t count, void* stream, uint32_t flags) {
@@ -2236,7 +2466,7 @@ int etha_unpack_bucket(const EthaTable* t, uint32_t first, uint32_t count, void*
   if (rc != ETHA_OK) return rc;
   if (t->reduce_prefix[first + count] != t->reduce_prefix[first])
     return fail(ETHA_ERR_INVALID, "range holds Partial chunks; a Partial placement cannot be a target");
-  return launch_tiles<true>(t, first, count, stream, flags);
+  return launch_single(t, ETHA_SEG_UNPACK, first, count, stream, flags);
 }
 
 int etha_reduce_pack_bucket(const EthaTable* t, uint32_t first, uint32_t count, void* stream, uint32_t flags) {
@@ -2245,7 +2475,7 @@ int etha_reduce_pack_bucket(const EthaTable* t, uint32_t first, uint32_t count, 
   if (rc != ETHA_OK) return rc;
   if (t->reduce_prefix[first + count] - t->reduce_prefix[first] != count)
     return fail(ETHA_ERR_INVALID, "range holds chunks that are not Partial chunks");
-  return launch_reduce(t, first, count, stream, flags);
+  return launch_single(t, ETHA_SEG_REDUCE_PACK, first, count, stream, flags);
 }
 
 int etha_selfcopy_bucket(const EthaTable* t, uint32_t first, uint32_t count, void* stream, uint32_t flags) {
@@ -2253,9 +2483,8 @@ int etha_selfcopy_bucket(const EthaTable* t, uint32_t first, uint32_t count, voi
   if (rc == ETHA_OK) rc = check_flags(flags);
   if (rc != ETHA_OK) return rc;
   const uint32_t n_reduce = t->reduce_prefix[first + count] - t->reduce_prefix[first];
-  if (n_reduce == 0) return launch_tiles<false>(t, first, count, stream, flags);
-  if (n_reduce != count) return fail(ETHA_ERR_INVALID, "range mixes Partial and plain chunks; launch them separately");
-  return launch_reduce(t, first, count, stream, flags);
+  if (n_reduce && n_reduce != count) return fail(ETHA_ERR_INVALID, "range mixes Partial and plain chunks; launch them separately");
+  return launch_single(t, ETHA_SEG_SELFCOPY, first, count, stream, flags);
 }
 
 int etha_launch_segments(const EthaSegment* segs, uint32_t n_segments, void* stream, uint32_t flags) {
@@ -2264,52 +2493,77 @@ int etha_launch_segments(const EthaSegment* segs, uint32_t n_segments, void* str
   if (n_segments == 0) return ETHA_OK;
   if (!segs) return fail(ETHA_ERR_INVALID, "null segment list");
   for (uint32_t i = 0; i < n_segments; i++) {  // validate everything before the first launch
-    const EthaSegment& g = segs[i];
-    if (g.kind > ETHA_SEG_SELFCOPY) return fail(ETHA_ERR_INVALID, "segment %u: unknown kind %u", i, g.kind);
-    rc = check_range(g.table, g.first, g.count, g.kind == ETHA_SEG_SELFCOPY ? 1 : 0);
+    rc = check_segment(segs[i], i);
     if (rc != ETHA_OK) return rc;
-    const uint32_t n_reduce = g.table->reduce_prefix[g.first + g.count] - g.table->reduce_prefix[g.first];
-    if ((g.kind == ETHA_SEG_PACK || g.kind == ETHA_SEG_UNPACK) && n_reduce)
-      return fail(ETHA_ERR_INVALID, "segment %u: range holds Partial chunks", i);
-    if (g.kind == ETHA_SEG_REDUCE_PACK && n_reduce != g.count)
-      return fail(ETHA_ERR_INVALID, "segment %u: range holds chunks that are not Partial chunks", i);
-    if (g.kind == ETHA_SEG_SELFCOPY && n_reduce && n_reduce != g.count)
-      return fail(ETHA_ERR_INVALID, "segment %u: range mixes Partial and plain chunks; launch them separately", i);
   }
-  std::vector<Seg2D> forward, reverse, gathered;
-  std::vector<TransSeg> trans_forward, trans_reverse;
-  uint32_t trans_lds = 0;
-  for (uint32_t i = 0; i < n_segments; i++) {
-    const EthaSegment& g = segs[i];
-    const EthaTable* t = g.table;
-    if (t->reduce_prefix[g.first + g.count] != t->reduce_prefix[g.first]) {
-      const uint32_t w0 = t->row_begin[g.first], w1 = t->row_begin[g.first + g.count];
-      if (w1 != w0) {
-        launch_kernel(etha_reduce_kernel, dim3((w1 - w0) * kBlocksPerTile), dim3(kBlockThreads), 0, stream, flags,
-                      (const RowTile*)(t->d_row + w0), (const uint64_t*)t->d_peers);
-        flags |= ETHA_LAUNCH_UNORDERED;
+  return guarded("etha_launch_segments", [&]() -> int {
+    LaunchList& list = scratch_launches();
+    plan_segments(segs, n_segments, flags, list);
+    return issue_all(list.data(), list.size(), stream);
+  });
+}
+
+int etha_schedule_create(const EthaSegment* segments, uint32_t n_segments, const EthaScheduleCall* calls, uint32_t n_calls,
+                         EthaSchedule** out) {
+  if (!out) return fail(ETHA_ERR_INVALID, "null out");
+  *out = nullptr;
+  if ((n_segments && !segments) || (n_calls && !calls)) return fail(ETHA_ERR_INVALID, "null argument");
+  return guarded("etha_schedule_create", [&]() -> int {
+    std::unique_ptr<EthaSchedule> s(new EthaSchedule());
+    std::map<const EthaTable*, int> seen;
+    for (uint32_t c = 0; c < n_calls; c++) {
+      const EthaScheduleCall& call = calls[c];
+      int rc = check_flags(call.flags);
+      if (rc != ETHA_OK) return rc;
+      if ((uint64_t)call.first_segment + call.n_segments > n_segments)
+        return fail(ETHA_ERR_INVALID, "call %u: segments [%u,+%u) outside the segment array of %u", c, call.first_segment,
+                    call.n_segments, n_segments);
+      if (call.single > 1 || (call.single && call.n_segments != 1))
+        return fail(ETHA_ERR_INVALID, "call %u: a single-range call names exactly one segment", c);
+      const EthaSegment* segs = segments + call.first_segment;
+      for (uint32_t i = 0; i < call.n_segments; i++) {
+        rc = check_segment(segs[i], call.first_segment + i);
+        if (rc != ETHA_OK) return rc;
+        if (seen.emplace(segs[i].table, 1).second) s->deps.push_back(EthaSchedule::Dep{segs[i].table, segs[i].table->serial, segs[i].table->version});
       }
-      continue;
+      if (call.single)
+        plan_single(segs[0], call.flags, s->launches);
+      else if (call.n_segments)
+        plan_segments(segs, call.n_segments, call.flags, s->launches);
     }
-    const bool rev = g.kind == ETHA_SEG_UNPACK;
-    const uint32_t x0 = t->trans_begin[g.first], n_trans = t->trans_begin[g.first + g.count] - x0;
-    if (n_trans) {
-      (rev ? trans_reverse : trans_forward).push_back(TransSeg{t->d_trans + x0, n_trans, 0});
-      if (t->trans_lds > trans_lds) trans_lds = t->trans_lds;
+    s->n_calls = n_calls;
+    *out = s.release();
+    return ETHA_OK;
+  });
+}
+
+int etha_schedule_launch(const EthaSchedule* s, void* stream) {
+  if (!s) return fail(ETHA_ERR_INVALID, "null schedule");
+  {
+    // the launches hold device addresses of the tables' tile programs: every table must still exist, unchanged
+    std::lock_guard<std::mutex> lock(g_tables_mutex);
+    for (const EthaSchedule::Dep& d : s->deps) {
+      auto it = g_live_tables.find(d.table);
+      if (it == g_live_tables.end() || it->second != d.serial)
+        return fail(ETHA_ERR_INVALID, "stale schedule: a table it launches has been destroyed");
+      if (d.table->version != d.version)
+        return fail(ETHA_ERR_INVALID, "stale schedule: a table it launches has changed since the schedule was created");
     }
-    const Seg2D r = tile_range(t, g.first, g.count, rev);
-    if (r.n_tiles) (rev ? reverse : forward).push_back(r);
-    const Seg2D gr = gather_range(t, g.first, g.count, rev);
-    if (gr.n_tiles) gathered.push_back(gr);
   }
-  launch_trans_group(trans_forward, false, trans_lds, stream, flags);
-  launch_trans_group(trans_reverse, true, trans_lds, stream, flags);
-  launch_group(forward, false, stream, flags);
-  launch_group(reverse, true, stream, flags);
-  launch_neighbours(
-      gathered, kJoinMaxIdleTiles, [](const Seg2D& x) { return (uint64_t)x.n_tiles; },
-      [&](size_t i, size_t j, uint32_t top, uint32_t fl) { launch_gather(&gathered[i], (uint32_t)(j - i), top, stream, fl); }, flags);
-  HIP_TRY(hipGetLastError());
+  return issue_all(s->launches.data(), s->launches.size(), stream);
+}
+
+int etha_schedule_info(const EthaSchedule* s, EthaScheduleInfo* out) {
+  if (!s || !out) return fail(ETHA_ERR_INVALID, "null argument");
+  out->n_calls = s->n_calls;
+  out->n_kernel_launches = (uint32_t)s->launches.size();
+  out->n_tables = (uint32_t)s->deps.size();
+  out->reserved = 0;
+  return ETHA_OK;
+}
+
+int etha_schedule_destroy(EthaSchedule* s) {
+  delete s;
   return ETHA_OK;
 }
 
@@ -2335,6 +2589,9 @@ int copy_regions_compile(const EthaChunkDesc* src, const EthaChunkDesc* dst, uin
   bld.row.clear();
   bld.trans.clear();
   bld.payload_bytes = 0;
+  // the compiled program must fit the array (the three tile lists start on 64-byte boundaries): compilation stops
+  // as soon as it cannot, before the host vectors grow past it
+  bld.max_bytes = ETHA_NOALLOC_SCRATCH_BYTES - 128;
   const ReduceSpec none;
   static const std::vector<uint64_t> no_peers;
   for (uint32_t i = 0; i < n_chunks; i++) {
@@ -2377,47 +2634,68 @@ int etha_copy_regions_noalloc(const EthaChunkDesc* src, const EthaChunkDesc* dst
   if (n_chunks && (!src || !dst)) return fail(ETHA_ERR_INVALID, "null descriptor array");
   int dev = 0;
   HIP_TRY(hipGetDevice(&dev));
-  if (dev < 0 || dev >= kMaxDevices || !g_noalloc[dev].scratch_ptr)
-    return fail(ETHA_ERR_INVALID, "call etha_noalloc_setup() with this device current first");
-  NoAllocState& st = g_noalloc[dev];
-  // host-side compilation reuses this thread's vectors: no heap growth once they have reached their size
-  thread_local Builder bld;
-  const int rc = copy_regions_compile(src, dst, n_chunks, bld);
-  if (rc != ETHA_OK) return rc;
-  const size_t run_bytes = bld.run.size() * sizeof(RunTile);
-  const size_t row_off = (run_bytes + 63) & ~(size_t)63, row_bytes = bld.row.size() * sizeof(RowTile);
-  const size_t trans_off = (row_off + row_bytes + 63) & ~(size_t)63, trans_bytes = bld.trans.size() * sizeof(TransTile);
-  const size_t total = trans_off + trans_bytes;
-  if (total > (size_t)ETHA_NOALLOC_SCRATCH_BYTES)
-    return fail(ETHA_ERR_UNSUPPORTED,
-                "these regions need a tile program of %llu bytes; etha_copy_regions_noalloc holds at most %llu "
-                "(use etha_selfcopy_table_create for larger copies)",
-                (unsigned long long)total, (unsigned long long)ETHA_NOALLOC_SCRATCH_BYTES);
-  if (run_bytes + row_bytes + trans_bytes == 0) return ETHA_OK;
-  if (st.copy_pending) HIP_TRY(hipEventSynchronize(st.copied));  // the previous call's upload still reads the staging buffer
-  uint8_t* stage = static_cast<uint8_t*>(st.staging);
-  if (run_bytes) memcpy(stage, bld.run.data(), run_bytes);
-  if (row_bytes) memcpy(stage + row_off, bld.row.data(), row_bytes);
-  if (trans_bytes) memcpy(stage + trans_off, bld.trans.data(), trans_bytes);
-  uint8_t* base = static_cast<uint8_t*>(st.scratch_ptr);  // the array's memory on this device: never the symbol's name
-  HIP_TRY(hipMemcpyAsync(base, stage, total, hipMemcpyHostToDevice, (hipStream_t)stream));
-  HIP_TRY(hipEventRecord(st.copied, (hipStream_t)stream));
-  st.copy_pending = true;
-  uint32_t lds = 0;
-  for (const TransTile& tt : bld.trans)
-    if (trans_lds_bytes(1u << tt.es_log2) > lds) lds = trans_lds_bytes(1u << tt.es_log2);
-  if (!bld.trans.empty()) {
-    launch_kernel(etha_transpose_kernel<false>, dim3((uint32_t)bld.trans.size()), dim3(kTransThreads), lds, stream, 0,
-                  (const TransTile*)(base + trans_off));
-    HIP_TRY(hipGetLastError());
-  }
-  const uint32_t n_run = (uint32_t)bld.run.size(), n_row = (uint32_t)bld.row.size();
-  if (n_run + n_row) {
-    launch_kernel(etha_tile_kernel<false>, dim3((n_run + n_row) * kBlocksPerTile), dim3(kBlockThreads), 0, stream, 0,
-                  (const RunTile*)base, n_run, (const RowTile*)(base + row_off), (const uint64_t*)nullptr);
-    HIP_TRY(hipGetLastError());
-  }
-  return ETHA_OK;
+  if (dev < 0 || dev >= kMaxDevices) return fail(ETHA_ERR_INVALID, "call etha_noalloc_setup() with this device current first");
+  // Not for a stream under capture: the upload of the tile program would become a graph node that reads the
+  // shared staging buffer at every replay, after later calls have overwritten it.
+  hipStreamCaptureStatus capture = hipStreamCaptureStatusNone;
+  HIP_TRY(hipStreamIsCapturing((hipStream_t)stream, &capture));
+  if (capture != hipStreamCaptureStatusNone)
+    return fail(ETHA_ERR_UNSUPPORTED, "etha_copy_regions_noalloc cannot be recorded into a graph: the stream is capturing");
+  return guarded("etha_copy_regions_noalloc", [&]() -> int {
+    // host-side compilation reuses this thread's vectors: they grow to at most the array's size
+    thread_local Builder bld;
+    const int rc = copy_regions_compile(src, dst, n_chunks, bld);
+    if (rc != ETHA_OK) {
+      if (bld.run.capacity() * sizeof(RunTile) + bld.row.capacity() * sizeof(RowTile) + bld.trans.capacity() * sizeof(TransTile) >
+          2ull * ETHA_NOALLOC_SCRATCH_BYTES) {  // a refused request does not leave its memory with the thread
+        std::vector<RunTile>().swap(bld.run);
+        std::vector<RowTile>().swap(bld.row);
+        std::vector<TransTile>().swap(bld.trans);
+      }
+      return rc;
+    }
+    const size_t run_bytes = bld.run.size() * sizeof(RunTile);
+    const size_t row_off = (run_bytes + 63) & ~(size_t)63, row_bytes = bld.row.size() * sizeof(RowTile);
+    const size_t trans_off = (row_off + row_bytes + 63) & ~(size_t)63, trans_bytes = bld.trans.size() * sizeof(TransTile);
+    const size_t total = trans_off + trans_bytes;
+    if (total > (size_t)ETHA_NOALLOC_SCRATCH_BYTES)
+      return fail(ETHA_ERR_UNSUPPORTED,
+                  "these regions need a tile program of %llu bytes; etha_copy_regions_noalloc holds at most %llu "
+                  "(use etha_selfcopy_table_create for larger copies)",
+                  (unsigned long long)total, (unsigned long long)ETHA_NOALLOC_SCRATCH_BYTES);
+    if (run_bytes + row_bytes + trans_bytes == 0) return ETHA_OK;
+    // one call at a time per process from here on: the staging buffer and the array are shared
+    std::lock_guard<std::mutex> lock(g_noalloc_mutex);
+    NoAllocState& st = g_noalloc[dev];
+    if (!st.scratch_ptr) return fail(ETHA_ERR_INVALID, "call etha_noalloc_setup() with this device current first");
+    if (st.copy_pending) HIP_TRY(hipEventSynchronize(st.copied));  // the previous call's upload still reads the staging buffer
+    uint8_t* stage = static_cast<uint8_t*>(st.staging);
+    if (run_bytes) memcpy(stage, bld.run.data(), run_bytes);
+    if (row_bytes) memcpy(stage + row_off, bld.row.data(), row_bytes);
+    if (trans_bytes) memcpy(stage + trans_off, bld.trans.data(), trans_bytes);
+    uint8_t* base = static_cast<uint8_t*>(st.scratch_ptr);  // the array's memory on this device: never the symbol's name
+    HIP_TRY(hipMemcpyAsync(base, stage, total, hipMemcpyHostToDevice, (hipStream_t)stream));
+    HIP_TRY(hipEventRecord(st.copied, (hipStream_t)stream));
+    st.copy_pending = true;
+    uint32_t lds = 0;
+    for (const TransTile& tt : bld.trans)
+      if (trans_lds_bytes(1u << tt.es_log2) > lds) lds = trans_lds_bytes(1u << tt.es_log2);
+    PreparedLaunch launches[2];
+    size_t n_launches = 0;
+    if (!bld.trans.empty()) {
+      launches[n_launches] = new_launch(kKernelTrans, false, 0, (uint32_t)bld.trans.size(), 1, kTransThreads, lds);
+      launches[n_launches++].u.trans.tiles = (const TransTile*)(base + trans_off);
+    }
+    const uint32_t n_run = (uint32_t)bld.run.size(), n_row = (uint32_t)bld.row.size();
+    if (n_run + n_row) {
+      PreparedLaunch& p = launches[n_launches++];
+      p = new_launch(kKernelTile, false, 0, (n_run + n_row) * kBlocksPerTile, 1, kBlockThreads, 0);
+      p.u.tile.run = (const RunTile*)base;
+      p.u.tile.n_run = n_run;
+      p.u.tile.row = (const RowTile*)(base + row_off);
+    }
+    return issue_all(launches, n_launches, stream);
+  });
 }
 
 int etha_arena_create(uint64_t nbytes, void** out_ptr) {
@@ -2449,50 +2727,54 @@ int etha_ipc_export(const void* dev_ptr, EthaIpcHandle* out) {
 int etha_ipc_open(const EthaIpcHandle* handle, void** out_ptr) {
   if (!handle || !out_ptr) return fail(ETHA_ERR_INVALID, "null argument");
   *out_ptr = nullptr;
-  // shared allocations of 2 GiB and more have not opened reliably on this platform
-  if (handle->size >= (2ull << 30))
-    return fail(ETHA_ERR_UNSUPPORTED, "IPC allocation of %llu bytes: keep shared allocations under 2 GiB",
-                (unsigned long long)handle->size);
-  IpcKey key;
-  memcpy(key.data(), handle->handle, 64);
-  std::lock_guard<std::mutex> lock(g_ipc_mutex);
-  IpcMapping& m = g_ipc_open[key];
-  if (m.refs == 0) {
-    hipIpcMemHandle_t h;
-    memcpy(&h, handle->handle, 64);
-    void* base = nullptr;
-    hipError_t e = hipIpcOpenMemHandle(&base, h, hipIpcMemLazyEnablePeerAccess);
-    if (e != hipSuccess) {
-      g_ipc_open.erase(key);
-      return fail(ETHA_ERR_HIP, "hipIpcOpenMemHandle: %s", hipGetErrorString(e));
+  return guarded("etha_ipc_open", [&]() -> int {
+    // shared allocations of 2 GiB and more have not opened reliably on this platform
+    if (handle->size >= (2ull << 30))
+      return fail(ETHA_ERR_UNSUPPORTED, "IPC allocation of %llu bytes: keep shared allocations under 2 GiB",
+                  (unsigned long long)handle->size);
+    IpcKey key;
+    memcpy(key.data(), handle->handle, 64);
+    std::lock_guard<std::mutex> lock(g_ipc_mutex);
+    IpcMapping& m = g_ipc_open[key];
+    if (m.refs == 0) {
+      hipIpcMemHandle_t h;
+      memcpy(&h, handle->handle, 64);
+      void* base = nullptr;
+      hipError_t e = hipIpcOpenMemHandle(&base, h, hipIpcMemLazyEnablePeerAccess);
+      if (e != hipSuccess) {
+        g_ipc_open.erase(key);
+        return fail(ETHA_ERR_HIP, "hipIpcOpenMemHandle: %s", hipGetErrorString(e));
+      }
+      m.base = base;
     }
-    m.base = base;
-  }
-  m.refs++;
-  void* p = (char*)m.base + handle->offset;
-  g_ipc_ptrs[p] = key;
-  g_ipc_ptr_refs[p]++;
-  *out_ptr = p;
-  return ETHA_OK;
+    m.refs++;
+    void* p = (char*)m.base + handle->offset;
+    g_ipc_ptrs[p] = key;
+    g_ipc_ptr_refs[p]++;
+    *out_ptr = p;
+    return ETHA_OK;
+  });
 }
 
 int etha_ipc_close(void* opened_ptr) {
   if (!opened_ptr) return ETHA_OK;
-  std::lock_guard<std::mutex> lock(g_ipc_mutex);
-  auto it = g_ipc_ptrs.find(opened_ptr);
-  if (it == g_ipc_ptrs.end()) return fail(ETHA_ERR_INVALID, "pointer was not returned by etha_ipc_open");
-  const IpcKey key = it->second;
-  if (--g_ipc_ptr_refs[opened_ptr] == 0) {
-    g_ipc_ptr_refs.erase(opened_ptr);
-    g_ipc_ptrs.erase(it);
-  }
-  IpcMapping& m = g_ipc_open[key];
-  if (--m.refs == 0) {
-    void* base = m.base;
-    g_ipc_open.erase(key);
-    HIP_TRY(hipIpcCloseMemHandle(base));
-  }
-  return ETHA_OK;
+  return guarded("etha_ipc_close", [&]() -> int {
+    std::lock_guard<std::mutex> lock(g_ipc_mutex);
+    auto it = g_ipc_ptrs.find(opened_ptr);
+    if (it == g_ipc_ptrs.end()) return fail(ETHA_ERR_INVALID, "pointer was not returned by etha_ipc_open");
+    const IpcKey key = it->second;
+    if (--g_ipc_ptr_refs[opened_ptr] == 0) {
+      g_ipc_ptr_refs.erase(opened_ptr);
+      g_ipc_ptrs.erase(it);
+    }
+    IpcMapping& m = g_ipc_open[key];
+    if (--m.refs == 0) {
+      void* base = m.base;
+      g_ipc_open.erase(key);
+      HIP_TRY(hipIpcCloseMemHandle(base));
+    }
+    return ETHA_OK;
+  });
 }
 
 }  // extern "C"

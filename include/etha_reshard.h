@@ -32,7 +32,7 @@
 extern "C" {
 #endif
 
-#define ETHA_ABI_VERSION 5
+#define ETHA_ABI_VERSION 6
 #define ETHA_MAX_NDIM 8
 
 /* status codes */
@@ -259,16 +259,48 @@ typedef struct EthaSegment {
 int etha_launch_segments(const EthaSegment* segments, uint32_t n_segments, void* stream, uint32_t flags);
 
 /*
- * Region copies for callers that cannot allocate device memory (code under HIP graph capture, tight serving
- * loops, harnesses that forbid hipMalloc).  No counterpart in the reference.
+ * A transfer as one call.  The reference plans once and transfers N times (tensor_bus/batch_state.py:38-40), and
+ * every transfer of a planned batch walks the same buckets in the same order through bucket_comm's loop
+ * (comm_methods.py:81-117).  A schedule is that walk recorded: the launch calls one transfer made, in order -
+ * each an etha_launch_segments call (segments [first_segment, +n_segments) of the segment array with its flags)
+ * or, with single = 1, one chunk range run as etha_pack_bucket / etha_unpack_bucket / etha_reduce_pack_bucket /
+ * etha_selfcopy_bucket would run it.  etha_schedule_create validates the calls and resolves them into ready-made
+ * kernel launches; etha_schedule_launch re-issues them on a stream with no planning left on the host.  The caller
+ * owns the claim that the recorded order is still right (same buckets, same readiness order).  The library checks
+ * what it can: a schedule whose tables have been destroyed, or changed by etha_table_optimize_range since it was
+ * created, refuses to launch with ETHA_ERR_INVALID ("stale schedule") - create a new one.
+ */
+typedef struct EthaSchedule EthaSchedule;
+typedef struct EthaScheduleCall {
+  uint32_t first_segment, n_segments; /* range of the segment array */
+  uint32_t flags;                     /* launch flags of the call */
+  uint32_t single;                    /* 1: n_segments == 1, run as the single-range entry point of its kind */
+} EthaScheduleCall;
+typedef struct EthaScheduleInfo {
+  uint32_t n_calls;
+  uint32_t n_kernel_launches; /* kernels one etha_schedule_launch issues */
+  uint32_t n_tables;
+  uint32_t reserved;
+} EthaScheduleInfo;
+int etha_schedule_create(const EthaSegment* segments, uint32_t n_segments, const EthaScheduleCall* calls, uint32_t n_calls,
+                         EthaSchedule** out);
+int etha_schedule_launch(const EthaSchedule* schedule, void* stream);
+int etha_schedule_info(const EthaSchedule* schedule, EthaScheduleInfo* out);
+int etha_schedule_destroy(EthaSchedule* schedule);
+
+/*
+ * Region copies for callers that cannot allocate device memory (tight serving loops, harnesses that forbid
+ * hipMalloc).  No counterpart in the reference.
  * etha_copy_regions_noalloc does what etha_selfcopy_table_create + etha_selfcopy_bucket + etha_table_destroy
  * do - copy src region i into dst region i, converting between their dtypes; no Partial sources - but keeps
  * the compiled tile program in a fixed array inside the library instead of in memory from hipMalloc, and calls
  * no hipMalloc / hipFree.  The program of one call may take at most ETHA_NOALLOC_SCRATCH_BYTES (24 bytes per
  * 16 KiB of contiguous payload, 64 bytes per 16 KiB of short-row payload: roughly 1-2.8 GB per call); larger
- * requests are refused with ETHA_ERR_UNSUPPORTED.  Every call on a GPU shares that GPU's array and upload
- * buffer: calls must be issued on one stream, or otherwise ordered so that one call's launches have finished
- * before the next call is made - calls that overlap on one GPU race.
+ * requests are refused with ETHA_ERR_UNSUPPORTED before anything is launched.  Every call on a GPU shares that
+ * GPU's array and upload buffer.  Calls from several host threads are serialised by the library; on the device,
+ * calls must be issued on one stream, or otherwise ordered so that one call's launches have finished before the
+ * next call's begin - calls that overlap on one GPU race.  A stream under HIP graph capture is refused
+ * (ETHA_ERR_UNSUPPORTED): the upload would be replayed from a buffer that later calls overwrite.
  * etha_noalloc_setup must have been called once with the device current (it looks up the array's device
  * address and allocates the pinned upload buffer; it is the only part that allocates).
  */

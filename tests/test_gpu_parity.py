@@ -738,8 +738,6 @@ def test_hip_graph_replay_matches_eager(gpu_device, pool):
     job = ReshardJob(specs, device=gpu_device, bucket_size=64 * 1024, target_ranks=targets, pool=pool)
     job.run(merge_launches=True)  # plans, uploads
     graph = job.capture(merge_launches=True)
-    from etha_amd.layout import local_shard
-
     for round_ in range(3):
         for i, d in enumerate(job.source_locals):
             for r, t in d.items():

@@ -148,3 +148,42 @@ def test_library_reports_the_sources_it_was_built_from():
     assert build.library_hash(build.LIB_PATH) == build.source_hash()
     assert nat.lib().etha_source_hash().decode() == build.source_hash()
     assert build.library_hash(os.path.join(ROOT, "README.md")) is None  # a file without the marker counts as stale
+
+
+def test_exceptions_stay_inside_the_library(tmp_path):
+    """The ABI is plain C: a C++ exception raised while a tile program is being compiled (a host allocation that
+    fails) comes back as ETHA_ERR_NOMEM with a message, never as an exception.  A test build of the library
+    raises std::bad_alloc once a program passes 40 tiles."""
+    import subprocess
+    import sys
+
+    from etha_amd import build
+
+    lib_path = str(tmp_path / "libetha_throwing.so")
+    build.build_library(defines=("ETHA_TEST_THROW_AT_TILE=40",), out_path=lib_path)
+    code = (
+        "import numpy as np\n"
+        "from etha_amd import _native as nat\n"
+        "def desc(rows):\n"
+        "    d = np.zeros(1, dtype=nat.CHUNK_DESC)\n"
+        "    d['tensor_ptr'], d['bucket_ptr'], d['ndim'] = 0x10000, 0x9000000, 2\n"
+        "    d['shape'][0][:2] = [rows, 4096]\n"
+        "    d['stride'][0][:2] = [4096, 1]\n"
+        "    d['tensor_dtype'] = d['wire_dtype'] = nat.F32\n"
+        "    return d\n"
+        "small = nat.Table.create(desc(8), upload=False)\n"  # 8 tiles: below the limit
+        "assert small.info().n_run_tiles == 8\n"
+        "for make in (lambda: nat.Table.create(desc(64), upload=False),\n"
+        "             lambda: nat.Table.create_selfcopy(desc(64), desc(64), upload=False)):\n"
+        "    try:\n"
+        "        make()\n"
+        "    except nat.EthaNativeError as e:\n"
+        "        assert e.code == nat.ERR_NOMEM and 'out of host memory' in str(e), str(e)\n"
+        "    else:\n"
+        "        raise SystemExit('the oversized program was accepted')\n"
+        "assert nat.Table.create(desc(8), upload=False).info().n_run_tiles == 8\n"  # the library still works
+        "print('contained')\n"
+    )
+    env = dict(os.environ, ETHA_AMD_LIB=lib_path, PYTHONPATH=ROOT)
+    proc = subprocess.run([sys.executable, "-c", code], capture_output=True, text=True, env=env, timeout=180)
+    assert proc.returncode == 0 and "contained" in proc.stdout, proc.stderr[-2000:]

@@ -285,3 +285,115 @@ def test_random_batches(seed, spec_fn=None):
                 assert_bit_equal(t, src_before[i][r], f"seed {seed} {spec.name} source rank {r} mutated")
     with pytest.raises(RuntimeError, match="no CPU path"):
         job.run()
+
+
+def _mutate_sources(job, ref, k):
+    """New source values on both jobs (so that a replay that moved stale bytes would show), targets poisoned."""
+    for a, b in zip(job.source_locals, ref.source_locals):
+        for r, t in a.items():
+            if any(t is x for d in job.target_locals for x in d.values()):
+                continue
+            if t.dtype.is_floating_point and t.dtype not in (torch.float8_e4m3fn, torch.float8_e5m2):
+                t.copy_((t.double() * -0.5 + k).to(t.dtype))
+            elif t.dtype == torch.bool:
+                t.copy_(~t)
+            elif t.dtype in (torch.float8_e4m3fn, torch.float8_e5m2):
+                t.copy_(t.float().roll(1, -1 if t.dim() else 0).to(t.dtype) if t.dim() else t)
+            else:
+                t.copy_(t.roll(1, -1) if t.dim() else t)
+            b[r].copy_(t)
+
+
+@pytest.mark.parametrize("staged", [False, True], ids=["one_drive", "send_then_recv"])
+@pytest.mark.parametrize("seed", range(40))
+def test_recorded_transfers_replay_what_the_pipelines_issue(seed, staged):
+    """A transfer that repeats is served from the sets its first run recorded, not by stepping the pipelines again.
+    The replayed sets go through the same byte-level hazard check and must give the oracle's result on new source
+    values; a transfer whose calls arrive in another order falls back to the pipelines and is recorded as well."""
+    rng = np.random.default_rng(7000 + seed)
+    wire_size = int(rng.choice([2, 2, 4, 8]))
+    specs = [_random_spec(rng, i, wire_size) for i in range(int(rng.integers(1, 5)))]
+    bucket_size = [64, 4096, 1 << 20][int(rng.integers(3))]
+    depth = int(rng.integers(1, 4))
+    merged = bool(rng.integers(2))
+    mode = ["buckets", "buckets", "zero_copy", "direct"][int(rng.integers(4))]
+    wire = LoopbackWire("cpu", segment_bytes=1 << 22, host_inspection=True, pool="ring", max_in_flight=depth)
+    job = ReshardJob(specs, device="cpu", bucket_size=bucket_size, keep_globals=True, fill=cpu_fill, wire=wire,
+                     direct=mode == "direct", zero_copy=mode == "zero_copy", max_in_flight=depth)
+    ref = ReshardJob(specs, device="cpu", bucket_size=bucket_size, keep_globals=True, fill=cpu_fill)
+    for a, b in zip(job.source_locals, ref.source_locals):
+        for r in a:
+            b[r].copy_(a[r])
+    ranges = []
+    for d in job.source_locals + job.target_locals:
+        for t in d.values():
+            st = t.untyped_storage()
+            if st.nbytes():
+                ranges.append((st.data_ptr(), st.data_ptr() + st.nbytes()))
+    for p in [wire.plan(b) for b in list(job.send_buckets.values()) + list(job.recv_buckets.values())]:
+        del p  # planning allocates the pool
+    if wire.pool is not None:
+        ranges += [(s.data_ptr(), s.data_ptr() + s.numel()) for s in wire.pool.segments]
+    if not ranges:
+        return
+    mem = AbsoluteMemory(min(r[0] for r in ranges), max(r[1] for r in ranges))
+    check = _HazardCheck()
+    issued: list = []
+
+    def on_set(members, flags):
+        issued.append((tuple((id(p), k, f, c) for p, k, f, c in members), flags))
+        if not flags & 1:
+            check.launch({}, 0)
+        for p, kind, first, count in reversed(members):
+            touched = {}
+            _run_step(mem, p, kind, first, count, ordered=(kind, first, count) in p._ordered_ranges, touched=touched)
+            check.launch(touched, 1)
+
+    def transfer(order=1):
+        issued.clear()
+        if staged:  # the senders' calls come first and fill their rings; the receivers' calls bring the rest
+            job.run_send(merged, drive=True)
+            recv = list(job.recv_buckets.values())[::order]
+            from etha_amd.comm import bucket_comm
+            for b in recv:
+                bucket_comm(b, depth, wire=wire, merge_launches=merged, synchronize=False)
+        else:
+            job.run(merge_launches=merged)
+        assert wire.idle()
+        return list(issued)
+
+    def verify(what):
+        run_oracle(ref)
+        for i, spec in enumerate(specs):
+            for r, t in job.target_locals[i].items():
+                assert_bit_equal(t, ref.target_locals[i][r], f"seed {seed} {what}: {spec.name} rank {r} vs oracle")
+
+    wire.on_set = on_set
+    try:
+        first = transfer()
+        verify("recording")
+        for k in (1, 2):
+            _mutate_sources(job, ref, k)
+            before = wire.replays
+            again = transfer()
+            if first:
+                assert wire.replays > before, "the repeated transfer was not served from the recording"
+            assert again == first, "a replay issues exactly the recorded sets"
+            verify(f"replay {k}")
+        if staged and len(job.recv_buckets) > 1:
+            _mutate_sources(job, ref, 3)
+            transfer(order=-1)  # another arrival order: not a recorded sequence from some point on
+            verify("other order")
+            _mutate_sources(job, ref, 4)
+            before = wire.replays
+            transfer(order=-1)
+            assert wire.replays > before
+            verify("other order, replayed")
+        # switched off: the pipelines run again and give the same launches
+        wire.replay_schedules = False
+        _mutate_sources(job, ref, 5)
+        before = wire.replays
+        assert transfer() == first and wire.replays == before
+        verify("pipelines")
+    finally:
+        wire.on_set = None

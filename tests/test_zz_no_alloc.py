@@ -79,10 +79,16 @@ def test_noalloc_region_copy_matches_the_table_path(gpu_device):
         torch.cuda.synchronize()
         for k, (a, b) in enumerate(zip(t1, t2)):
             assert torch.equal(_bits(a), _bits(b)), f"call with seed {seed}: target {k} differs from the table path"
-        # and the table path's own meaning, for one pair: the converted slice landed, the rest is untouched
-        s, ss, d, ds = p2[0]
-        assert torch.equal(_bits(d[ds]), _bits(s[ss].to(torch.bfloat16)))
-        assert float(d[0, 0]) == -1.0
+    # and what either path means, for every pair of every call: the slice, converted by torch, landed; bytes outside
+    # the destination slice kept their fill value
+    for p2, t1, t2, seed in kept:
+        fills = (-1.0, 7, 3.0, 2.0)
+        for k, ((s, ss, d, ds), first, fill) in enumerate(zip(p2, t1, fills)):
+            want = s[ss].to(d.dtype)
+            assert torch.equal(_bits(first[ds]), _bits(want)), f"call with seed {seed}: pair {k} is not torch's slice.to()"
+            outside = torch.ones_like(first, dtype=torch.bool)
+            outside[ds] = False
+            assert bool((first[outside] == fill).all()), f"call with seed {seed}: pair {k} wrote outside its region"
 
 
 def test_noalloc_refuses_what_does_not_fit_and_what_it_cannot_do(gpu_device):
@@ -106,3 +112,27 @@ def test_noalloc_refuses_what_does_not_fit_and_what_it_cannot_do(gpu_device):
     a["n_partials"] = 2
     with pytest.raises(nat.EthaNativeError, match="Partial"):
         nat.copy_regions_noalloc(a, b)
+
+
+def test_noalloc_refuses_a_capturing_stream(gpu_device):
+    """Recorded into a graph, the upload of the tile program would be replayed from a staging buffer that later
+    calls overwrite: the entry point refuses a stream under capture and launches nothing."""
+    torch.cuda.set_device(gpu_device)
+    nat.noalloc_setup()
+    src = torch.arange(4096, device=gpu_device, dtype=torch.float32)
+    dst = torch.zeros(4096, device=gpu_device, dtype=torch.float32)
+    a, b = _rows([(src, (slice(0, 4096),), dst, (slice(0, 4096),))])
+    graph = torch.cuda.CUDAGraph()
+    side = torch.cuda.Stream(device=gpu_device)
+    with torch.cuda.stream(side):
+        with torch.cuda.graph(graph, stream=side):
+            before = nat.kernel_launches()
+            with pytest.raises(nat.EthaNativeError, match="capturing") as e:
+                nat.copy_regions_noalloc(a, b, torch.cuda.current_stream(gpu_device).cuda_stream)
+            assert e.value.code == nat.ERR_UNSUPPORTED and nat.kernel_launches() == before
+            dst.add_(0)  # the capture itself stays valid: it records this and ends normally
+    torch.cuda.synchronize()
+    assert float(dst.abs().sum()) == 0.0
+    nat.copy_regions_noalloc(a, b, torch.cuda.current_stream(gpu_device).cuda_stream)  # eagerly it still works
+    torch.cuda.synchronize()
+    assert torch.equal(dst, src)
