@@ -55,7 +55,9 @@ def parse_args():
                          "configuration)")
     ap.add_argument("--cpu-layers", type=int, default=8,
                     help="decoder layers of the sample the CPU baseline falls back to when host memory is short")
-    ap.add_argument("--cpu-seconds", type=float, default=15.0, help="CPU work the baseline leg is bounded to")
+    ap.add_argument("--cpu-seconds", type=float, default=10.0, help="CPU work the baseline leg is bounded to")
+    ap.add_argument("--no-process-legs", action="store_true",
+                    help="skip the legs that start worker processes (the two-process wire and the tensor bus end to end)")
     ap.add_argument("--calibration-copy", action="store_true",
                     help="after the timed region run three plain 1 GiB torch copies (known traffic, for scaling "
                          "hardware counters collected with rocprofv3 --pmc)")
@@ -165,7 +167,8 @@ def cpu_baseline(workload: str, layers: int, seconds: float):
 
 def read_traffic(workload: str, mode: str):
     """HBM bytes per step of a workload from the committed counter summary (``profiles/hbm_traffic.txt``), with the
-    commit and command it was measured at.  Lines: ``workload | mode | fetch_bytes | write_bytes | launches | commit``."""
+    commit, command and library build it was measured at.
+    Lines: ``workload | mode | fetch_bytes | write_bytes | launches | commit | library digest``."""
     try:
         with open(TRAFFIC_FILE) as f:
             for line in f:
@@ -173,10 +176,22 @@ def read_traffic(workload: str, mode: str):
                 if len(parts) >= 6 and parts[0] == workload and parts[1] == mode:
                     return {"fetch_bytes_per_step": int(parts[2]), "write_bytes_per_step": int(parts[3]),
                             "launches_per_step": int(parts[4]), "measured_at_commit": parts[5],
+                            "library_digest": parts[6] if len(parts) > 6 else None,
                             "source": "profiles/hbm_traffic.txt"}
     except OSError:
         pass
     return None
+
+
+def with_library_check(traffic):
+    """The counters were read under rocprofv3 in a run of their own: say which build of the library that was, and
+    whether it is the one running now."""
+    if traffic is None:
+        return None
+    from etha_amd import _native
+
+    running = _native.lib().etha_source_hash().decode()
+    return {**traffic, "running_library_digest": running, "stale": traffic.get("library_digest") != running}
 
 
 def _numel(shape):
@@ -264,6 +279,94 @@ def launches_per_step(job, run):
     torch.cuda.synchronize()
     job.wire.launch_log = None
     return _native.kernel_launches() - before, len(log), sum(1 for entry in log if entry[3] & 1)
+
+
+OTHER_WORKLOADS = ("single_fp32_shard0_to_shard1", "many_small_2d_to_replicate", "partial4_to_shard2",
+                   "moe_experts_and_uneven_vocab", "llama3_8b_fsdp8_to_tp2_fp32_to_bf16", "transposed_parents")
+
+
+def measure_workload(name: str, dev, steps: int, warmup: int):
+    """One workload in the default form (ring of 2 slots per channel, independent steps share launches): device
+    time per step by HIP events, algorithmic bytes, launches."""
+    import torch
+
+    from etha_amd import workloads
+    from etha_amd.world import ReshardJob
+
+    specs, targets, bucket = workloads.WORKLOADS[name]()
+    job = ReshardJob(specs, device=dev, bucket_size=bucket, target_ranks=targets)
+    for _ in range(max(warmup, 3)):
+        job.run(merge_launches=True)
+    dev_ms, wall_ms = time_steps(job, max(steps, 20), lambda: job.run(merge_launches=True, synchronize=False))
+    host_ms = HOST_MS.get("issue")
+    n_launch, n_steps, _ = launches_per_step(job, lambda: job.run(merge_launches=True, synchronize=False))
+    pack_bytes, unpack_bytes, self_bytes, _, _ = algorithmic_bytes(job)
+    total = pack_bytes + unpack_bytes
+    S = job.payload_bytes()
+    traffic = read_traffic(name, "ring/sets")
+    out = {
+        "payload_bytes": S,
+        "device_ms_per_step": round(dev_ms, 4),
+        "ms_per_step": round(wall_ms, 4),
+        "host_issue_ms_per_step": round(host_ms, 4),
+        "algorithmic_bytes_per_step": total,
+        "pct_of_hbm_peak": round(100.0 * total / (dev_ms * 1e-3) / 1e9 / HBM_PEAK_GBS, 2),
+        "effective_GB/s": round(S / (dev_ms * 1e-3) / 1e9, 1),
+        "launches_per_step": n_launch,
+        "bucket_steps_per_step": n_steps,
+        "steps": max(steps, 20),
+        "warmup": max(warmup, 3),
+        "pool_reserved_bytes": job.wire.pool.reserved_bytes if job.wire.pool is not None else 0,
+        "hbm_GB/s": None if traffic is None else
+        round((traffic["fetch_bytes_per_step"] + traffic["write_bytes_per_step"]) / (dev_ms * 1e-3) / 1e9, 1),
+    }
+    del job
+    torch.cuda.empty_cache()
+    return out
+
+
+def copy_ceiling(dev, reps: int = 10):
+    """What a plain copy reaches on this device through the library's own pack kernel: one contiguous 4 GiB tensor
+    packed into one bucket (read 4 GiB, write 4 GiB), and the same tensor as fp32 packed into a bf16 bucket (read
+    4 GiB, write 2 GiB).  The workloads above are bounded by this, not by the published 8 TB/s."""
+    import torch
+    from torch.distributed.tensor.placement_types import Replicate
+
+    from etha_amd.world import ReshardJob, TensorSpec, transfer_dtype_rule
+
+    out = {}
+    stream = torch.cuda.current_stream(dev)
+    for label, n, sdt, tdt in (("bf16_to_bf16", 1 << 31, torch.bfloat16, None), ("fp32_to_bf16", 1 << 30, torch.float32, torch.bfloat16)):
+        spec = TensorSpec("c", (n,), [0], (Replicate(),), [1], (Replicate(),), sdt, tdt, seed=1)
+        job = ReshardJob([spec], device=dev, bucket_size=64 << 20, pool="resident")
+        for _ in range(3):
+            job.run()
+        ev = [torch.cuda.Event(enable_timing=True) for _ in range(reps + 1)]
+        ev[0].record(stream)
+        for k in range(reps):
+            job.run_send()
+            ev[k + 1].record(stream)
+        torch.cuda.synchronize()
+        ms = sorted(ev[k].elapsed_time(ev[k + 1]) for k in range(reps))
+        wire = transfer_dtype_rule(sdt, tdt or sdt).itemsize
+        nbytes = n * sdt.itemsize + n * wire
+        out[label] = {"bytes_read": n * sdt.itemsize, "bytes_written": n * wire, "median_ms": round(ms[len(ms) // 2], 4),
+                      "GB/s": round(nbytes / (ms[len(ms) // 2] * 1e-3) / 1e9, 1),
+                      "pct_of_hbm_peak": round(100.0 * nbytes / (ms[len(ms) // 2] * 1e-3) / 1e9 / HBM_PEAK_GBS, 2)}
+        del job
+        torch.cuda.empty_cache()
+    return out
+
+
+def process_leg(module: str, *flags, timeout: float = 180.0):
+    """A leg that needs worker processes of its own: run the module as a child and take the JSON line it prints."""
+    import subprocess
+
+    proc = subprocess.run([sys.executable, "-m", module, *flags], cwd=ROOT, capture_output=True, text=True, timeout=timeout)
+    lines = [l for l in proc.stdout.splitlines() if l.startswith("{")]
+    if proc.returncode != 0 or not lines:
+        raise RuntimeError(f"{module} exited with {proc.returncode}: {proc.stderr[-500:]}")
+    return json.loads(lines[-1])
 
 
 def main():
@@ -384,7 +487,10 @@ def main():
             # HBM bytes per launch from the committed rocprofv3 counter summary (null when this configuration has none)
             "traffic": None if traffic is None else
             (traffic["fetch_bytes_per_step"] + traffic["write_bytes_per_step"]) // max(traffic["launches_per_step"], 1),
-            "traffic_detail": traffic,
+            "traffic_detail": with_library_check(traffic),
+            # achieved HBM rate by the counters: (FETCH_SIZE + WRITE_SIZE bytes per step) / device time per step
+            "hbm_GB/s": None if traffic is None else
+            round((traffic["fetch_bytes_per_step"] + traffic["write_bytes_per_step"]) / (dev_ms * 1e-3) / 1e9, 1),
             "bytes_per_launch": total_bytes // max(n_launch, 1),
             # launches overlap their neighbours: the average is the timed region over the launches in it
             "avg_launch_ms": round(dev_ms / max(n_launch, 1), 5),
@@ -498,6 +604,41 @@ def main():
                 torch.cuda.empty_cache()
         except Exception as e:  # an optional leg must not take the measured line with it
             out["extra_legs_error"] = f"{type(e).__name__}: {e}"
+
+    if plain and args.pool == "ring" and args.workload == "llama3_8b_fsdp8_to_tp2":
+        # every other configuration in its default form, and what a plain copy reaches through the same kernels
+        job = None
+        torch.cuda.empty_cache()
+        out["workloads"] = {}
+        for name in OTHER_WORKLOADS:
+            try:
+                out["workloads"][name] = measure_workload(name, dev, args.steps, args.warmup)
+            except Exception as e:
+                out["workloads"][name] = {"error": f"{type(e).__name__}: {e}"}
+        try:
+            out["copy_ceiling"] = copy_ceiling(dev)
+        except Exception as e:
+            out["copy_ceiling"] = {"error": f"{type(e).__name__}: {e}"}
+        if not args.no_process_legs:
+            torch.cuda.empty_cache()
+            try:
+                d = process_leg("etha_amd.comm.bench_wire", "--workload", args.workload, "--steps", "10", "--warmup", "3")
+                out["two_process_wire"] = {"ms_per_transfer": round(d["ms_per_transfer"], 3), "min_ms": round(d["min_ms"], 3),
+                                           "effective_GB/s": round(d["value"], 1), "payload_bytes": d["payload_bytes"],
+                                           "steps": d["steps"], **d["config"],
+                                           "clock": "host wall clock: producer starts packing -> consumer's last unpack done",
+                                           "bit_equal_target_tensors": d["target_tensors_bit_equal_to_the_in_process_transfer"]}
+            except Exception as e:
+                out["two_process_wire"] = {"error": f"{type(e).__name__}: {e}"}
+            try:
+                d = process_leg("etha_amd.tensor_bus.bench_transfer", "--workload", args.workload, "--steps", "10", "--warmup", "3")
+                out["bus_end_to_end"] = {"ms_per_transfer": round(d["ms_per_transfer"], 3), "min_ms": round(d["min_ms"], 3),
+                                         "effective_GB/s": round(d["value"], 1), "payload_bytes": d["payload_bytes"],
+                                         "steps": d["steps"], **d["config"], "agent": d["agent"],
+                                         "clock": "host wall clock: first rank's transfer('send') -> last rank's blocking transfer('recv') returns",
+                                         "tensors_verified_by_checksum": d["tensors_verified_by_checksum"]}
+            except Exception as e:
+                out["bus_end_to_end"] = {"error": f"{type(e).__name__}: {e}"}
 
     if args.calibration_copy:
         a = torch.empty(1 << 30, dtype=torch.uint8, device=dev).fill_(1)

@@ -361,7 +361,7 @@ class TransferPlan:
                                            "(a real wire would block here)")
                     if info.tiles:
                         self.launch_step(kind, first, count, stream)
-                    mark_received(entry, info.bucket.rank)
+                    mark_received(entry, info.bucket.rank, self.wire)
                 elif info.tiles:
                     self.launch_step(kind, first, count, stream)
 
@@ -452,17 +452,21 @@ def mark_sent(wire, entry) -> None:
     entry.left = wire.consumers(entry)
     entry.slot.filled += 1
     entry.slot.holder = entry if entry.left else None
+    if wire.outbox is not None and entry.left:  # the consumers live in another process: tell them
+        wire.outbox.append(("packed", entry.key, entry.seq))
 
 
 def recv_may_start(entry, rank) -> bool:
     return entry.slot.holder is entry and rank in entry.left
 
 
-def mark_received(entry, rank) -> None:
+def mark_received(entry, rank, wire=None) -> None:
     entry.left.discard(rank)
     entry.slot.drained += 1
     if not entry.left:
         entry.slot.holder = None
+    if wire is not None and wire.outbox is not None and entry.remote:  # the producer lives in another process
+        wire.outbox.append(("unpacked", entry.key, entry.seq, rank))
 
 
 @dataclass
@@ -494,7 +498,7 @@ class Program:
         for b in buckets:
             for i in plan.steps_of.get(id(b), ()):
                 entry, kind = plan.info[i].entry, plan.steps[i][0]
-                if entry is not None and kind in (_UNPACK, _DIRECT, _DIRECT_REDUCE):
+                if entry is not None and kind in (_UNPACK, _DIRECT, _DIRECT_REDUCE) and not entry.remote:
                     if entry.submitted < entry.arrived.get(b.rank, 0) + 1:
                         raise RuntimeError(
                             f"{b}: recv bucket runs before its send bucket was ever sent (a real wire would block here)")
@@ -546,7 +550,7 @@ class Program:
                 return False  # nothing has arrived yet
         return True
 
-    def _finalize(self, bucket, todo: list) -> None:
+    def _finalize(self, bucket, todo: list, wire=None) -> None:
         steps = self._steps(bucket)
         if bucket.transport == Transport.LOCAL:
             todo.extend(i for i, _, _ in steps[1:])  # the unpack of a staged copy
@@ -554,7 +558,7 @@ class Program:
         for i, kind, info in steps:
             if kind in (_UNPACK, _DIRECT, _DIRECT_REDUCE):
                 todo.append(i)
-                mark_received(info.entry, bucket.rank)
+                mark_received(info.entry, bucket.rank, wire)
 
     def sweep(self, wire) -> bool:
         """One turn of the prepare / launch / complete phases over all channels; True if anything moved.
@@ -581,7 +585,7 @@ class Program:
             progress = False
             for ch in self.channels.values():
                 if ch.in_flight and self._is_complete(ch.in_flight[0]):
-                    self._finalize(ch.in_flight.popleft(), todo)
+                    self._finalize(ch.in_flight.popleft(), todo, wire)
                     progress = moved = True
         if todo:
             wire.emit(self.plan, todo, self.merge)

@@ -104,6 +104,7 @@ class WireEntry:
     packed: int = 0  # transfers packed into the slot so far
     arrived: dict = field(default_factory=dict)  # destination rank -> transfers it has asked for
     left: set = field(default_factory=set)  # consumers of the bytes now in the slot that have not unpacked yet
+    remote: bool = False  # a copy, in a consumer process, of an entry that a producer process owns
 
 
 class _no_context:
@@ -205,6 +206,11 @@ class LoopbackWire:
         self._tx_calls: list | None = None  # recording: what the drive under way has issued so far
         self._suppress = False  # rebuilding pipeline state: steps are walked, nothing is launched
         self.replays = 0  # drives served from a recorded schedule (statistics)
+        # Across processes (export_manifest / from_manifest with a ring pool): a list that collects what the peer
+        # process must be told - ("packed", key, seq) once a send bucket is in its slot, ("unpacked", key, seq, rank)
+        # once a destination has read it.  None: every rank of this wire lives in this process.
+        self.outbox: list | None = None
+        self.local_ranks: set | None = None  # consumer process: the destination ranks that live here
         self.pool: BucketPool | None = None
         # per wire key: sequence number -> (slot, chunk sizes) of every planned send bucket still alive
         self._sent: dict[tuple, dict[int, tuple[Slot, tuple[int, ...]]]] = defaultdict(dict)
@@ -290,6 +296,59 @@ class LoopbackWire:
     def consumers(self, entry: WireEntry) -> set:
         return {r for r in entry.dst_ranks if r not in self.absent_ranks}
 
+    # -- a ring whose two ends live in different processes ----------------------------------------
+    def take_outbox(self) -> list:
+        """What the peer process has to be told since the last call.  The caller synchronises the stream first (the
+        hand-over between processes is ordered by a host-side fence) and sends the list over its own channel."""
+        out, self.outbox = self.outbox or [], []
+        return out
+
+    def apply_remote(self, messages) -> None:
+        """The peer's notifications: a producer learns that destinations have unpacked (their slots become free), a
+        consumer that send buckets have been packed (they may now be unpacked).  The same hand-shake
+        ``mark_sent`` / ``mark_received`` keep inside one process."""
+        from .comm_methods import mark_received
+
+        for msg in messages:
+            what, key, seq = msg[0], tuple(msg[1]), msg[2]
+            key = (key[0], key[1], tuple(key[2]), key[3])
+            entry = self._sent.get(key, {}).get(seq)
+            if entry is None:
+                raise RuntimeError(f"the peer process names bucket #{seq} of {key}, which is not planned on this wire")
+            if what == "packed":
+                if entry.slot.holder is not None:
+                    raise RuntimeError(f"bucket #{seq} of {key} was packed into a slot that still holds unread bytes")
+                entry.packed += 1
+                entry.left = {r for r in self.consumers(entry) if self.local_ranks is None or r in self.local_ranks}
+                entry.slot.filled += 1
+                entry.slot.holder = entry if entry.left else None
+            elif what == "unpacked":
+                if entry.slot.holder is not entry or msg[3] not in entry.left:
+                    raise RuntimeError(f"rank {msg[3]} reports bucket #{seq} of {key} as unpacked, which it was not sent")
+                mark_received(entry, msg[3])
+            else:
+                raise ValueError(f"unknown wire notification {what!r}")
+
+    def exchange(self, conn, synchronize=None) -> None:
+        """Run the transfers queued on this wire to completion against the peer process at the other end of ``conn``
+        (a ``multiprocessing`` connection): step the pipelines, fence, send what the peer must know, wait for its
+        notifications, until nothing is pending here.  Both processes call this once per transfer."""
+        if self.outbox is None:
+            raise RuntimeError("this wire has no peer process (see export_manifest / from_manifest)")
+        sync = synchronize or (lambda: torch.cuda.current_stream(self.device).synchronize())
+        while True:
+            self.drive()
+            out = self.take_outbox()
+            if out:
+                sync()  # the peer may touch the slots as soon as it hears of them
+                conn.send(("wire", out))
+            if self.idle():
+                return
+            kind, messages = conn.recv()
+            if kind != "wire":
+                raise RuntimeError(f"unexpected message from the peer process: {kind!r}: {messages}")
+            self.apply_remote(messages)
+
     # -- across processes ----------------------------------------------------------------------
     def export_manifest(self) -> dict:
         """Describe every planned send slot so that another process on the same GPU can consume it.
@@ -300,16 +359,18 @@ class LoopbackWire:
         """
         from .. import _native as nat
 
-        if self.pool_mode != "resident":
-            raise NotImplementedError(
-                "a ring pool is recycled under a hand-shake that only exists inside one process; "
-                "export needs LoopbackWire(pool='resident')")
+        if self.pool_mode == "ring":
+            # slots are recycled: from now on the consumers' progress arrives as notifications (apply_remote)
+            self.outbox = []
+            self.forget_recorded_transfers()
         if self.pool is None:
-            return {"device": None, "segments": [], "slots": {}}
+            return {"device": None, "pool": self.pool_mode, "segments": [], "slots": {}}
         segments = []
-        with torch.cuda.device(self.pool.device):
+        host = self.pool.device.type != "cuda"  # host inspection: the "other process" is this one, addresses are shared
+        with torch.cuda.device(self.pool.device) if not host else _no_context():
             for seg in self.pool.segments:
-                segments.append({"ipc": nat.ipc_export(seg.data_ptr()), "nbytes": seg.numel()})
+                segments.append({"ptr": seg.data_ptr(), "nbytes": seg.numel()} if host else
+                                {"ipc": nat.ipc_export(seg.data_ptr()), "nbytes": seg.numel()})
         slots: dict = {}
         for key, entries in self._sent.items():
             out = []
@@ -318,8 +379,9 @@ class LoopbackWire:
                 if slot.sources is not None:
                     raise NotImplementedError("a direct wire has no bucket buffers to export; it works inside one process")
                 if slot.borrowed:  # lives in a source tensor: export that allocation, range = the slot itself
-                    with torch.cuda.device(self.pool.device):
-                        segments.append({"ipc": nat.ipc_export(slot.ptr), "nbytes": slot.nbytes})
+                    with torch.cuda.device(self.pool.device) if not host else _no_context():
+                        segments.append({"ptr": slot.ptr, "nbytes": slot.nbytes} if host else
+                                        {"ipc": nat.ipc_export(slot.ptr), "nbytes": slot.nbytes})
                     out.append({"seq": seq, "segment": len(segments) - 1, "offset": 0, "nbytes": slot.nbytes, "sizes": sizes})
                     continue
                 idx = next(i for i, seg in enumerate(self.pool.segments)
@@ -327,7 +389,7 @@ class LoopbackWire:
                 out.append({"seq": seq, "segment": idx, "offset": slot.ptr - self.pool.segments[idx].data_ptr(),
                             "nbytes": slot.nbytes, "sizes": sizes})
             slots[key] = out
-        return {"device": self.pool.device.index, "segments": segments, "slots": slots}
+        return {"device": None if host else self.pool.device.index, "pool": self.pool_mode, "segments": segments, "slots": slots}
 
     @classmethod
     def from_manifest(cls, manifest: dict, device: torch.device | str | None = None) -> "LoopbackWire":
@@ -335,20 +397,30 @@ class LoopbackWire:
         from .. import _native as nat
 
         dev = torch.device(device) if device is not None else torch.device("cuda", manifest["device"] or 0)
-        wire = cls(dev, pool="resident")
+        ring = manifest.get("pool", "resident") == "ring"
+        wire = cls(dev, pool="ring" if ring else "resident", host_inspection=dev.type != "cuda")
         wire._imported = []
         bases = []
-        with torch.cuda.device(dev):
+        with torch.cuda.device(dev) if dev.type == "cuda" else _no_context():
             for seg in manifest["segments"]:
+                if "ptr" in seg:  # exported by a host-inspection wire of this very process
+                    bases.append((seg["ptr"], seg["nbytes"]))
+                    continue
                 ptr = nat.ipc_open(seg["ipc"])
                 wire._imported.append(ptr)
                 bases.append((ptr, seg["nbytes"]))
+        slots: dict = {}  # buckets of one channel that share a ring slot share the Slot object here too
         for key, entries in manifest["slots"].items():
             for e in entries:
                 base, nbytes = bases[e["segment"]]
-                slot = Slot(ptr=base + e["offset"], nbytes=e["nbytes"], lo=base, hi=base + nbytes)
+                where = (e["segment"], e["offset"], e["nbytes"]) if ring else (key, e["seq"])
+                slot = slots.get(where)
+                if slot is None:
+                    slot = slots[where] = Slot(ptr=base + e["offset"], nbytes=e["nbytes"], lo=base, hi=base + nbytes)
                 wire._sent[key][e["seq"]] = WireEntry(key=key, seq=e["seq"], slot=slot, sizes=tuple(e["sizes"]),
-                                                      dst_ranks=tuple(key[2]))
+                                                      dst_ranks=tuple(key[2]), remote=True)
+        if ring:
+            wire.outbox = []
         return wire
 
     def mark_packed(self) -> None:
@@ -418,7 +490,7 @@ class LoopbackWire:
     # -- recorded transfers ----------------------------------------------------------------------
     def _tracing(self) -> bool:
         if not (self.replay_schedules and self.pool_mode == "ring" and self.on_launch is None and self.launch_log is None
-                and (self.on_set is not None or (self.device is not None and self.device.type == "cuda"))):
+                and self.outbox is None and (self.on_set is not None or (self.device is not None and self.device.type == "cuda"))):
             return False
         if self.absent_ranks != self._trace_absent:  # who unpacks decides when a slot is free again
             self.forget_recorded_transfers()

@@ -96,8 +96,14 @@ class TensorBusAgent:
 
     def __init__(self, world_size: int, path_naming_fn=None, device: str | torch.device = "cuda:0",
                  heartbeat_interval: float = 0.2, zero_copy_single_chunk: bool = False,
-                 direct_same_device: bool = False, pool: str = "ring", max_in_flight: int = 2):
+                 direct_same_device: bool = False, pool: str = "ring", max_in_flight: int = 2,
+                 gather_window: float = 0.001):
         self.world_size = world_size
+        # The ranks of a batch issue their transfer commands together (the reference brackets a transfer with a
+        # barrier over all of them, agent.py:457).  When the first one arrives the agent waits up to this long for
+        # the others, so that it can queue every rank's pipeline in rank order and step them in one go: the same
+        # sequence every transfer, which the wire then serves from its recording (LoopbackWire.replay_schedules).
+        self.gather_window = gather_window
         self.device = torch.device(device)
         self.path_naming_fn = path_naming_fn or default_path_naming
         self.heartbeat_interval = heartbeat_interval
@@ -121,6 +127,7 @@ class TensorBusAgent:
         self._last_core: dict | None = None
         self._moved = False  # set by a command that changed shared state without completing
         self._unsynced: list[tuple[dict, float, str]] = []  # (result, start time, label) of transfers enqueued, not yet synchronised
+        self._queued = False  # pipelines were queued on the wire in this pass and have not been stepped yet
         self.stats = {"ipc_tensors": 0, "in_process_tensors": 0, "transfers": 0}
         for rank in range(world_size):
             cmd_path, state_path = self.path_naming_fn(rank)
@@ -189,6 +196,15 @@ class TensorBusAgent:
                 self._pending.append(self._inbox.get_nowait())
             except queue.Empty:
                 break
+        deadline = time.perf_counter() + self.gather_window
+        while self._siblings_missing():
+            left = deadline - time.perf_counter()
+            if left <= 0:
+                break
+            try:
+                self._pending.append(self._inbox.get(timeout=left))
+            except queue.Empty:
+                break
         # Sweep until nothing moves.  Commands that complete are answered only after the sweep: the device
         # work of every transfer that became ready is enqueued first, then the stream is synchronised once
         # and the state files are written once, instead of once per rank.
@@ -196,7 +212,7 @@ class TensorBusAgent:
         progressed = True
         while progressed:
             progressed, self._moved = False, False
-            for entry in list(self._pending):
+            for entry in self._in_rank_order(self._pending):
                 try:
                     done, value = self._advance(entry)
                 except Exception as e:  # report to the worker, keep serving
@@ -209,6 +225,10 @@ class TensorBusAgent:
                     finished.append((entry, ("ok", value)))
                     self._pending.remove(entry)
                     progressed = True
+            if self._queued:  # every pipeline queued in this pass is stepped now, together
+                self._queued = False
+                self.wire.drive()
+                progressed = True
             # a command that changed shared state without completing (a send that lends its tensors and now
             # waits for its receivers) may have unblocked commands examined earlier in this pass
             progressed = progressed or self._moved
@@ -227,6 +247,33 @@ class TensorBusAgent:
             self._write_state(force=True)
             for entry, message in finished:
                 self._reply(entry, message)
+
+    @staticmethod
+    def _in_rank_order(pending: list) -> list:
+        """Commands in arrival order, except that the transfer commands among them are taken batch by batch, sends
+        before receives, ranks ascending - whichever order their threads happened to deliver them in."""
+        transfers = sorted((e for e in pending if isinstance(e.command, Transfer)),
+                           key=lambda e: (e.command.batch_id, e.command.transfer_type != "send", e.rank))
+        return [e for e in pending if not isinstance(e.command, Transfer)] + transfers
+
+    def _siblings_missing(self) -> bool:
+        """True while some rank of a batch has issued a transfer command that is not under way yet and another rank
+        with buckets in the same direction has not issued its command of that generation."""
+        waiting: dict = {}
+        for e in self._pending:
+            if isinstance(e.command, Transfer) and not e.started:
+                waiting.setdefault((e.command.batch_id, e.command.transfer_type), set()).add(e.rank)
+        for (batch_id, kind), ranks in waiting.items():
+            batch = self.batches.get(batch_id)
+            if batch is None:
+                continue
+            table = batch.send_buckets if kind == "send" else batch.recv_buckets
+            counts = batch.send_count if kind == "send" else batch.recv_count
+            gen = min((counts.get(r, 0) for r in ranks), default=0)
+            for r, buckets in table.items():
+                if buckets and r not in ranks and counts.get(r, 0) <= gen:
+                    return True
+        return False
 
     @staticmethod
     def _reply(entry: _Entry, message) -> None:
@@ -466,7 +513,8 @@ class TensorBusAgent:
                 batch.transfer_signal = True
                 entry.result = {"ms": 0.0}
                 self._unsynced.append((entry.result, time.perf_counter(), f"batch {cmd.batch_id} rank {rank} send #{gen}"))
-                bucket_comm(buckets, wire=self.wire, merge_launches=True, synchronize=False, scope=batch.batch_id)
+                bucket_comm(buckets, wire=self.wire, merge_launches=True, synchronize=False, scope=batch.batch_id, drive=False)
+                self._queued = True
                 batch.send_count[rank] = gen + 1
                 for d in self._peers(buckets, "dst"):
                     batch.owed[d] = max(batch.owed.get(d, 0), gen + 1)
@@ -497,7 +545,8 @@ class TensorBusAgent:
                     return False, None  # wait for the source's send of this generation
             result = {"ms": 0.0}
             self._unsynced.append((result, time.perf_counter(), f"batch {cmd.batch_id} rank {rank} recv #{gen}"))
-            bucket_comm(buckets, wire=self.wire, merge_launches=True, synchronize=False, scope=batch.batch_id)
+            bucket_comm(buckets, wire=self.wire, merge_launches=True, synchronize=False, scope=batch.batch_id, drive=False)
+            self._queued = True
             batch.recv_count[rank] = gen + 1
             if all(batch.recv_count.get(d, 0) >= n for d, n in batch.owed.items()):
                 batch.transfer_signal = False  # every destination of every send so far has received

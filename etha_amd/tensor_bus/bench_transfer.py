@@ -182,7 +182,7 @@ def main() -> None:
         for p in procs:
             if p.is_alive():
                 p.kill()
-        agent_stats = dict(agent.stats)
+        agent_stats = dict(agent.stats, drives_served_from_a_recording=agent.wire.replays)
         agent.close()
     # checksum of checksums: a same-dtype tensor's bits, summed over all target ranks, equal the sum over all
     # source ranks times the number of copies the target layout holds of each element (per copy the source holds)

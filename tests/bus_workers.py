@@ -167,15 +167,22 @@ def _pool_specs():
     from etha_amd.world import TensorSpec
 
     src, tgt = list(range(4)), [4, 5]
-    return [
+    specs = [
         TensorSpec("q", (512, 256), src, (Shard(0),), tgt, (Shard(0),), torch.bfloat16, seed=11, std=1.0),
         TensorSpec("o", (256, 512), src, (Shard(0),), tgt, (Shard(1),), torch.bfloat16, seed=12, std=1.0),
         TensorSpec("norm", (256,), src, (Shard(0),), tgt, (Replicate(),), torch.float32, torch.bfloat16, seed=13, std=1.0),
     ]
+    # several buckets per channel, so that a ring of one or two slots is recycled while a transfer runs
+    for i in range(3):
+        specs.append(TensorSpec(f"up{i}", (256, 320), src, (Shard(0),), tgt, (Shard(1),), torch.bfloat16, seed=20 + i, std=1.0))
+        specs.append(TensorSpec(f"n{i}", (512,), src, (Shard(0),), tgt, (Replicate(),), torch.bfloat16, seed=30 + i, std=1.0))
+    return specs
 
 
-def producer_process(device, conn, rounds, zero_copy=False):
-    """Owns the source shards and the bucket pool: plans, exports the pool, packs each round."""
+def producer_process(device, conn, rounds, zero_copy=False, pool="resident", depth=2):
+    """Owns the source shards and the bucket pool: plans, exports the pool, packs each round.  With a ring pool the
+    slots are recycled while the transfer runs: ``exchange`` trades "packed" / "unpacked" notifications with the
+    consumer process; with a resident pool one "packed" message per round is enough."""
     try:
         import torch
 
@@ -184,22 +191,40 @@ def producer_process(device, conn, rounds, zero_copy=False):
         from helpers import cpu_fill
 
         setup_ptrace()
-        # a pool that another process reads is resident: a ring is recycled under a hand-shake inside one process
         job = ReshardJob(_pool_specs(), device=device, bucket_size=32 * 1024, fill=cpu_fill, zero_copy=zero_copy,
-                         pool="resident")
+                         pool=pool, max_in_flight=depth)
         lent = 0
         for buckets in job.send_buckets.values():
             lent += len(job.wire.plan(buckets).lent)  # planning assigns the slots
         assert (lent > 0) == bool(zero_copy)
         conn.send(("manifest", job.wire.export_manifest()))
+        payload = job.payload_bytes()
+        reserved = job.wire.pool.reserved_bytes if job.wire.pool is not None else 0
+        if pool == "ring":  # the reference's bound: max_in_flight buckets per channel, not the payload
+            channels = {(b.src_rank, tuple(b.dst_ranks), b.transport.value) for bs in job.send_buckets.values() for b in bs
+                        if b.transport.value in ("p2p", "broadcast")}
+            largest = max(b.total_bytes for bs in job.send_buckets.values() for b in bs)
+            assert reserved <= len(channels) * depth * (-(-largest // 256) * 256), (reserved, len(channels), depth, largest)
+            per_channel = {}
+            for bs in job.send_buckets.values():
+                for b in bs:
+                    if b.transport.value in ("p2p", "broadcast"):
+                        k = (b.src_rank, tuple(b.dst_ranks), b.transport.value)
+                        per_channel[k] = per_channel.get(k, 0) + 1
+            assert zero_copy or max(per_channel.values()) > depth  # slots really are reused within one transfer
         for round_ in range(rounds):
             if round_ > 0:
                 for d in job.source_locals:
                     for t in d.values():
                         t.mul_(-2.0)
-            job.run_send(merge_launches=True)
-            torch.cuda.synchronize()  # cross-process ordering is a host-side fence
-            conn.send(("packed", round_))
+            if pool == "ring":
+                job.run_send(merge_launches=True, drive=False)
+                job.wire.exchange(conn)
+                assert job.wire.idle()
+            else:
+                job.run_send(merge_launches=True)
+                torch.cuda.synchronize()  # cross-process ordering is a host-side fence
+                conn.send(("packed", round_))
             assert conn.recv() == ("consumed", round_)
         conn.send(("done", None))
     except BaseException:
@@ -220,13 +245,19 @@ def consumer_process(device, conn, rounds, out_q):
         kind, manifest = conn.recv()
         assert kind == "manifest", manifest
         wire = LoopbackWire.from_manifest(manifest, device)
+        ring = wire.pool_mode == "ring"
         specs = _pool_specs()
         job = ReshardJob(specs, device=device, bucket_size=32 * 1024, fill=cpu_fill, keep_globals=True, wire=wire)
         bad = []
         for round_ in range(rounds):
-            assert conn.recv() == ("packed", round_)
-            wire.mark_packed()
-            job.run_recv(merge_launches=True)
+            if ring:
+                job.run_recv(merge_launches=True, drive=False)
+                wire.exchange(conn)
+                assert wire.idle()
+            else:
+                assert conn.recv() == ("packed", round_)
+                wire.mark_packed()
+                job.run_recv(merge_launches=True)
             torch.cuda.synchronize()
             for i, spec in enumerate(specs):
                 glob = job.globals_[i].cpu().float() * ((-2.0) ** round_)
@@ -235,6 +266,7 @@ def consumer_process(device, conn, rounds, out_q):
                     if not torch.equal(t.cpu().view(torch.uint8), want.contiguous().view(torch.uint8)):
                         bad.append((round_, spec.name, r))
             conn.send(("consumed", round_))
+        assert wire.pool is None or wire.pool.reserved_bytes == 0  # the consumer holds no bucket memory of its own
         wire.close_imported()
         out_q.put(("consumer", "ok" if not bad else "mismatch", bad))
     except BaseException:

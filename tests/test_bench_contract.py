@@ -43,3 +43,40 @@ def test_bench_line_has_the_contract_fields(gpu_device):
     cpu = d["cpu_baseline"]
     assert cpu["kind"] == "port" and cpu["unit"] == "GB/s" and cpu["cores"] >= 1 and cpu["value"] > 0 and cpu["sample"]
     assert "extra_legs_error" not in d
+
+
+@pytest.mark.gpu
+def test_default_line_carries_every_configuration(gpu_device):
+    """The default run (the one the driver makes): the headline on config 2 plus one entry per other configuration,
+    the copy ceiling, the counter-derived HBM rate and the two legs that run in worker processes."""
+    r = _bench("--steps", "20", "--warmup", "3", "--cpu-seconds", "2", timeout=600)
+    assert r.returncode == 0, r.stderr[-2000:]
+    lines = [l for l in r.stdout.splitlines() if l.strip()]
+    assert len(lines) == 1
+    d = json.loads(lines[0])
+    assert d["config"]["workload"] == "llama3_8b_fsdp8_to_tp2" and d["steps"] == 20 and d["warmup"] == 3
+    assert "extra_legs_error" not in d
+    wl = d["workloads"]
+    assert set(wl) == {"single_fp32_shard0_to_shard1", "many_small_2d_to_replicate", "partial4_to_shard2",
+                       "moe_experts_and_uneven_vocab", "llama3_8b_fsdp8_to_tp2_fp32_to_bf16", "transposed_parents"}
+    for name, w in wl.items():
+        assert "error" not in w, (name, w)
+        assert w["steps"] >= 20 and w["warmup"] >= 3
+        for key in ("device_ms_per_step", "algorithmic_bytes_per_step", "pct_of_hbm_peak", "effective_GB/s", "launches_per_step"):
+            assert w[key] > 0, (name, key)
+        assert abs(w["pct_of_hbm_peak"] - 100 * w["algorithmic_bytes_per_step"] / (w["device_ms_per_step"] * 1e-3) / 8e12) < 0.05
+        assert w["pct_of_hbm_peak"] < 100
+    assert wl["partial4_to_shard2"]["algorithmic_bytes_per_step"] == 7 * (1 << 30)  # 4 reads + 1 write, then unpack 1 + 1
+    for leg in ("bf16_to_bf16", "fp32_to_bf16"):
+        c = d["copy_ceiling"][leg]
+        assert 0 < c["pct_of_hbm_peak"] < 100 and c["bytes_read"] == 4 << 30
+    roof = d["roofline"]
+    detail = roof["traffic_detail"]
+    if detail is not None:
+        assert isinstance(detail["stale"], bool) and detail["running_library_digest"]
+        assert abs(roof["hbm_GB/s"] - (detail["fetch_bytes_per_step"] + detail["write_bytes_per_step"]) / (d["device_ms_per_step"] * 1e-3) / 1e9) < 1
+    for leg in ("two_process_wire", "bus_end_to_end"):
+        assert "error" not in d[leg], d[leg]
+        assert d[leg]["ms_per_transfer"] > 0 and d[leg]["effective_GB/s"] > 0
+    assert d["two_process_wire"]["pool"] == "ring" and d["two_process_wire"]["bit_equal_target_tensors"] == 290
+    assert d["two_process_wire"]["pool_reserved_bytes"] < d["config"]["payload_bytes"] // 4

@@ -231,5 +231,87 @@ def test_resident_pool_keeps_one_slot_per_bucket():
     run_oracle(ref)
     _compare(job, ref, specs)
     assert job.wire.pool.reserved_bytes >= job.payload_bytes()
-    with pytest.raises(NotImplementedError, match="resident"):
-        LoopbackWire("cpu", host_inspection=True).export_manifest()
+    empty = LoopbackWire("cpu", host_inspection=True).export_manifest()  # a ring can be exported too: nothing planned yet
+    assert empty["pool"] == "ring" and empty["slots"] == {}
+
+
+@pytest.mark.parametrize("depth", [1, 2, 3])
+@pytest.mark.parametrize("zero_copy", [False, True], ids=["packed", "lent"])
+def test_a_ring_whose_ends_live_in_different_processes(depth, zero_copy):
+    """Producer and consumer each hold their own wire and trade "packed" / "unpacked" notifications over a pipe
+    (LoopbackWire.exchange), as two processes on one GPU do; here the two ends are threads of this process and the
+    launches go to the tile interpreter.  Two transfers; the pool stays within max_in_flight slots per channel;
+    a notification that does not fit the hand-shake is refused."""
+    import multiprocessing as mp
+    import threading
+
+    from test_random_layouts_cpu import _run_step
+    from tile_interpreter import AbsoluteMemory
+
+    src, tgt = list(range(4)), [4, 5]
+    specs = [TensorSpec(f"w{i}", (128, 96 + 32 * i), src, (Shard(0),), tgt, (Shard(1),), torch.bfloat16, seed=i, std=1.0)
+             for i in range(5)]
+    specs.append(TensorSpec("n", (256,), src, (Shard(0),), tgt, (Replicate(),), torch.float32, torch.bfloat16, seed=9, std=1.0))
+    specs.append(TensorSpec("big", (256, 512), src, (Shard(0),), tgt, (Shard(0),), torch.bfloat16, seed=10, std=1.0))
+    producer, ref = _jobs(specs, 4096, depth, zero_copy=zero_copy)
+    for buckets in producer.send_buckets.values():
+        producer.wire.plan(buckets)
+    manifest = producer.wire.export_manifest()
+    assert manifest["pool"] == "ring"
+    wire = LoopbackWire.from_manifest(manifest, "cpu")
+    consumer = ReshardJob(specs, device="cpu", bucket_size=4096, keep_globals=True, fill=cpu_fill, wire=wire, max_in_flight=depth)
+    assert producer.wire.pool.reserved_bytes <= _ring_bound(producer, depth)
+    spans = []
+    for job in (producer, consumer):
+        for d in job.source_locals + job.target_locals:
+            for t in d.values():
+                st = t.untyped_storage()
+                if st.nbytes():
+                    spans.append((st.data_ptr(), st.data_ptr() + st.nbytes()))
+    spans += [(s.data_ptr(), s.data_ptr() + s.numel()) for s in producer.wire.pool.segments]
+    mem = AbsoluteMemory(min(s[0] for s in spans), max(s[1] for s in spans))
+    lock = threading.Lock()
+
+    def on_set(members, flags):
+        with lock:
+            for p, kind, first, count in members:
+                _run_step(mem, p, kind, first, count, ordered=(kind, first, count) in p._ordered_ranges)
+
+    producer.wire.on_set = consumer.wire.on_set = on_set
+    a, b = mp.Pipe()
+    errors = []
+
+    def consume():
+        try:
+            consumer.run_recv(True, drive=False)
+            consumer.wire.exchange(b, synchronize=lambda: None)
+        except BaseException as e:  # noqa: BLE001
+            errors.append(e)
+            a.close()
+
+    for round_ in range(2):
+        if round_:
+            for d, e in zip(producer.source_locals, ref.source_locals):
+                for r, t in d.items():
+                    t.mul_(-3.0)
+                    e[r].copy_(t)
+        th = threading.Thread(target=consume)
+        th.start()
+        producer.run_send(True, drive=False)
+        producer.wire.exchange(a, synchronize=lambda: None)
+        th.join(60)
+        assert not th.is_alive() and not errors, errors
+        assert producer.wire.idle() and consumer.wire.idle()
+        run_oracle(ref)
+        for i, spec in enumerate(specs):
+            for r, t in consumer.target_locals[i].items():
+                assert_bit_equal(t, ref.target_locals[i][r], f"round {round_} {spec.name} rank {r} vs oracle")
+    assert consumer.wire.pool is None  # the consumer allocated no bucket memory
+    # notifications that contradict the hand-shake are refused
+    key, entries = next(iter(producer.wire._sent.items()))
+    with pytest.raises(RuntimeError, match="was not sent"):
+        producer.wire.apply_remote([("unpacked", key, min(entries), 4)])
+    with pytest.raises(RuntimeError, match="not planned on this wire"):
+        consumer.wire.apply_remote([("packed", key, 10_000)])
+    with pytest.raises(ValueError, match="unknown wire notification"):
+        consumer.wire.apply_remote([("sent", key, min(entries))])

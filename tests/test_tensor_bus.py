@@ -228,16 +228,19 @@ def test_two_process_hipipc_handoff(gpu_device, tmp_path):
 
 
 @pytest.mark.gpu
+@pytest.mark.parametrize("pool,depth", [("resident", 2), ("ring", 1), ("ring", 2)], ids=["resident", "ring1", "ring2"])
 @pytest.mark.parametrize("zero_copy", [False, True], ids=["packed", "lent"])
-def test_bucket_pool_crosses_a_process_boundary(gpu_device, zero_copy):
+def test_bucket_pool_crosses_a_process_boundary(gpu_device, zero_copy, pool, depth):
     """The wire step as a same-GPU loopback between two processes: the producer packs into its pool, the
-    consumer maps the pool with hipIpcOpenMemHandle and unpacks from it; two rounds with new values."""
+    consumer maps the pool with hipIpcOpenMemHandle and unpacks from it; two rounds with new values.  With a
+    ring pool the producer owns max_in_flight slots per channel (asserted there) and the two processes trade
+    "packed" / "unpacked" notifications while the transfer runs, each behind a host-side fence."""
     from bus_workers import consumer_process, producer_process
 
     ctx = mp.get_context("spawn")
     a, b = ctx.Pipe()
     out_q = ctx.Queue()
-    procs = [ctx.Process(target=producer_process, args=(str(gpu_device), a, 2, zero_copy)),
+    procs = [ctx.Process(target=producer_process, args=(str(gpu_device), a, 2, zero_copy, pool, depth)),
              ctx.Process(target=consumer_process, args=(str(gpu_device), b, 2, out_q))]
     try:
         for p in procs:
