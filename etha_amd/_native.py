@@ -66,8 +66,10 @@ ROW_TILE = np.dtype(
     ]
 )
 TRANS_TILE = np.dtype([("a", "<u8"), ("b", "<u8"), ("a_pitch", "<i8"), ("b_pitch", "<i8"), ("nj", "<u4"), ("nk", "<u4"),
-                       ("es_log2", "<u4"), ("cvt", "<u4")])
-assert RUN_TILE.itemsize == 24 and ROW_TILE.itemsize == 64 and TRANS_TILE.itemsize == 48
+                       ("es_log2", "<u4"), ("cvt", "<u4"), ("peer_first", "<u4"), ("n_peers", "<u4"), ("reduce_op", "<u4"),
+                       ("via", "<u4")])
+TRANS_TYPED = 1 << 8  # TransTile.cvt: a block of the typed transposing kernel
+assert RUN_TILE.itemsize == 24 and ROW_TILE.itemsize == 64 and TRANS_TILE.itemsize == 64
 
 
 class Segment(ctypes.Structure):

@@ -126,7 +126,7 @@ class _TraceNode:
     """One point of a recorded transfer (see :attr:`LoopbackWire.replay_schedules`): reached from its parent by a
     ``submit`` or a ``drive`` event.  A node reached by a drive holds what that drive issued."""
 
-    __slots__ = ("children", "calls", "schedule", "pending", "recorded")
+    __slots__ = ("children", "calls", "schedule", "pending", "recorded", "outbox")
 
     def __init__(self):
         self.children: dict = {}
@@ -134,6 +134,7 @@ class _TraceNode:
         self.schedule = None  # the same as one native schedule (built on first replay on a GPU)
         self.pending: frozenset = frozenset()  # ids of the plans whose pipelines are still waiting after this drive
         self.recorded = False
+        self.outbox: tuple = ()  # what this drive left for the peer process (a wire with a remote end)
 
 
 def wire_key(bucket: Bucket) -> tuple:
@@ -202,6 +203,7 @@ class LoopbackWire:
         self._tx_events: list = []  # events of the transfer under way since the wire was last idle
         self._tx_node: _TraceNode | None = None  # trie node of those events; None: this transfer is not traced
         self._tx_replaying = False  # the transfer under way follows a recorded one: no pipelines exist for it
+        self._tx_dirty = False  # slots changed hands outside a transfer (a peer's early notification): do not trace the next one
         self._tx_pending: set = set()  # replaying: ids of plans submitted and not yet finished
         self._tx_calls: list | None = None  # recording: what the drive under way has issued so far
         self._suppress = False  # rebuilding pipeline state: steps are walked, nothing is launched
@@ -307,6 +309,24 @@ class LoopbackWire:
         """The peer's notifications: a producer learns that destinations have unpacked (their slots become free), a
         consumer that send buckets have been packed (they may now be unpacked).  The same hand-shake
         ``mark_sent`` / ``mark_received`` keep inside one process."""
+        messages = tuple((m[0], (m[1][0], m[1][1], tuple(m[1][2]), m[1][3]), *m[2:]) for m in messages)
+        event = ("r", messages)
+        if self._tx_replaying:
+            child = self._tx_node.children.get(event)
+            if child is not None:  # the peer follows the recorded transfer too: nothing to update, no pipelines exist
+                self._tx_node = child
+                self._tx_events.append(event)
+                return
+            self._rebuild_pipelines()
+        self._apply_remote(messages)
+        if self._programs or self._tx_events:
+            self._tx_events.append(event)
+            if self._tx_node is not None:
+                self._tx_node = self._child(self._tx_node, event)
+        else:  # between transfers: the next one does not start from the state every recording starts from
+            self._tx_dirty = True
+
+    def _apply_remote(self, messages) -> None:
         from .comm_methods import mark_received
 
         for msg in messages:
@@ -490,7 +510,7 @@ class LoopbackWire:
     # -- recorded transfers ----------------------------------------------------------------------
     def _tracing(self) -> bool:
         if not (self.replay_schedules and self.pool_mode == "ring" and self.on_launch is None and self.launch_log is None
-                and self.outbox is None and (self.on_set is not None or (self.device is not None and self.device.type == "cuda"))):
+                and (self.on_set is not None or (self.device is not None and self.device.type == "cuda"))):
             return False
         if self.absent_ranks != self._trace_absent:  # who unpacks decides when a slot is free again
             self.forget_recorded_transfers()
@@ -524,18 +544,25 @@ class LoopbackWire:
         self._tx_pending = set()
         self._suppress = True
         try:
+            outbox = self.outbox
+            if outbox is not None:
+                self.outbox = []  # what the walk leaves there has been handed out by the replayed drives already
             for ev in events:
                 if ev[0] == "s":
                     self._programs.append(Program(ev[1], ev[2], ev[3]))
+                elif ev[0] == "r":
+                    self._apply_remote(ev[1])
                 else:
                     self._drive_pipelines()
         finally:
             self._suppress = False
+            self.outbox = outbox
 
     def _end_of_drive(self, idle: bool) -> None:
         if idle:  # the transfer is over: the next submit starts a new one
             self._tx_events, self._tx_node, self._tx_replaying = [], None, False
             self._tx_pending = set()
+            self._tx_dirty = False
 
     # -- the bucket pipelines of every rank on this wire ---------------------------------------
     def submit(self, plan, max_in_flight: int, merge_launches: bool = False):
@@ -545,7 +572,7 @@ class LoopbackWire:
         event = ("s", id(plan), max_in_flight, merge_launches, self.unordered_launches, self.group_launches)
         if not self._programs and not self._tx_events:  # an idle wire: a new transfer begins
             self._tx_replaying = False
-            self._tx_node = self._trace_root if self._tracing() else None
+            self._tx_node = self._trace_root if self._tracing() and not self._tx_dirty else None
             if self._tx_node is not None and event in self._tx_node.children:
                 self._tx_replaying = True
         if self._tx_replaying:
@@ -579,6 +606,7 @@ class LoopbackWire:
         if record and self.on_set is None and torch.cuda.is_current_stream_capturing():
             record, self._tx_node = False, None  # what a capture leaves out (uploads) must not end up in a recorded transfer
         self._tx_calls = [] if record else None
+        outbox_before = len(self.outbox) if self.outbox is not None else 0
         try:
             self._drive_pipelines()
         except BaseException:
@@ -590,6 +618,7 @@ class LoopbackWire:
             node = self._tx_node = self._child(self._tx_node, _DRIVE)
             if node is not None and not node.recorded:
                 node.calls, node.pending, node.recorded = calls, frozenset(id(p.plan) for p in self._programs), True
+                node.outbox = tuple(self.outbox[outbox_before:]) if self.outbox is not None else ()
         self._end_of_drive(not self._programs)
 
     def _drive_recorded(self) -> bool:
@@ -624,6 +653,8 @@ class LoopbackWire:
                 self.forget_recorded_transfers()
                 return False
         self.replays += 1
+        if self.outbox is not None:
+            self.outbox.extend(node.outbox)
         self._tx_node = node
         self._tx_events.append(_DRIVE)
         self._tx_pending = set(node.pending)

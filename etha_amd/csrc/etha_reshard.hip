@@ -97,9 +97,21 @@ struct TransTile {   // a 2-D block whose contiguous dim differs between the two
   int64_t b_pitch;   // bytes between consecutive j on the b side
   uint32_t nj, nk;   // extent of the block: a wide block, a block of trans_dim_a x trans_dim_b elements, or less at an edge
   uint32_t es_log2;  // log2 of the element size in bytes (of the b side, when the block converts)
-  uint32_t cvt;      // 0: same element type on both sides; else (dtype of a << 4) | dtype of b: a holds f32, b f16 or bf16
+  uint32_t cvt;      // 0: same element type on both sides; else (dtype of a << 4) | dtype of b, plus kTransTyped for the
+                     // blocks of the typed kernel (without it: a holds f32, b f16 or bf16, converted by the plain kernel)
+  uint32_t peer_first;  // typed blocks of a Partial source: index of the first peer base (a is then an offset from each base)
+  uint32_t n_peers;     // 0 = not a reduction
+  uint32_t reduce_op;   // one ETHA_* op (nested levels keep their row tiles)
+  uint32_t via;         // as in RowTile
 };
-static_assert(sizeof(TransTile) == 48, "TransTile layout");
+static_assert(sizeof(TransTile) == 64, "TransTile layout");
+// Blocks of the typed transposing kernel: any pair of value types (converted element by element while the block is
+// parked in LDS) and Partial sources (the members' blocks are combined in registers first).  Full blocks are
+// trans_typed_dim x trans_typed_dim elements.
+constexpr uint32_t kTransTyped = 1u << 8;
+__host__ __device__ constexpr uint32_t trans_typed_dim(uint32_t esa, uint32_t esb) { return (esa == 8 || esb == 8) ? 64u : 128u; }
+// Full blocks of a Partial source whose members hold 2-byte elements (the straight-line reduce path): j x k elements.
+constexpr uint32_t kRedDimJ2 = 128, kRedDimK2 = 128;
 // A transposing block is D x D elements, handled by one workgroup of kTransThreads work-items.  D is chosen
 // per element size so that a row of the block is at least 128 bytes on both sides and a full block is a
 // few 16-byte vectors per work-item.  LDS rows are padded to an odd number of 32-bit words.
@@ -131,6 +143,12 @@ constexpr uint32_t kTransCvtWideJ = ETHA_TRANS_DIM_A, kTransCvtWideK = 2 * ETHA_
 __host__ __device__ constexpr uint32_t trans_pitch(uint32_t dim, uint32_t es) {  // LDS row pitch in elements: an odd number of words
   return dim + (es >= 4 ? 1u : 4u / es);
 }
+__host__ __device__ constexpr uint32_t trans_typed_lds_bytes(uint32_t esa, uint32_t esb) {  // rows of the destination's elements
+  const uint32_t d = trans_typed_dim(esa, esb), m = esa > esb ? esa : esb;
+  const uint32_t typed = d * (d + (m >= 4 ? 1u : 4u / m)) * m;
+  const uint32_t red = esa == 2 ? kRedDimK2 * (kRedDimJ2 + (esb >= 4 ? 1u : 4u / esb)) * esb : 0u;
+  return typed > red ? typed : red;
+}
 __host__ __device__ constexpr uint32_t trans_lds_bytes(uint32_t es) {  // either direction: rows of one side (one panel of a wide block), one row per element of the other
   const uint32_t w = trans_wide(es), p = trans_panels(es);
   const uint32_t fwd = w * trans_dim_b(es) * trans_pitch(w * trans_dim_a(es) / p, es) * es, rev = w * trans_dim_a(es) * trans_pitch(w * trans_dim_b(es) / p, es) * es;
@@ -152,6 +170,9 @@ constexpr uint32_t kMetaGeneric = 1u << 20;  // converting move with an integer,
 // units is n_peers pieces of `via` units each, piece p read at gather[peer_first + p] + row * b_pitch.  The a
 // side is addressed as in any row tile, so one wavefront writes whole destination lines.
 constexpr uint32_t kMetaGather = 1u << 21;
+// converting and reducing moves: log2 of the elements one unit holds (2 bits).  kMetaVec marks the full vector of a
+// dtype pair; a row's remainder moves in narrower vectors of 4 or 2 elements before single elements are used.
+constexpr uint32_t kMetaElemsShift = 22;
 constexpr uint32_t kGatherMaxPieces = 8;       // the kernel reads this many piece addresses per tile (the list is padded)
 
 // ---- typed vector access ----------------------------------------------------------------------
@@ -240,22 +261,29 @@ __device__ __forceinline__ void cvt_n(uint64_t src, uint64_t dst) {
   out.store(dst);
 }
 
+// nl = log2 of the elements in this unit (at most those of the pair's full vector)
 template <typename S, typename D>
-__device__ __forceinline__ void cvt_pair(bool vec, uint64_t src, uint64_t dst) {
+__device__ __forceinline__ void cvt_pair(uint32_t nl, uint64_t src, uint64_t dst) {
   constexpr int kN = cvt_elems_per_unit(sizeof(typename S::bits), sizeof(typename D::bits));
-  if (vec)
-    cvt_n<S, D, kN>(src, dst);
-  else
-    cvt_n<S, D, 1>(src, dst);
+  if constexpr (kN >= 8) {
+    if (nl == 3) return cvt_n<S, D, 8>(src, dst);
+  }
+  if constexpr (kN >= 4) {
+    if (nl == 2) return cvt_n<S, D, 4>(src, dst);
+  }
+  if constexpr (kN >= 2) {
+    if (nl == 1) return cvt_n<S, D, 2>(src, dst);
+  }
+  cvt_n<S, D, 1>(src, dst);
 }
 
 template <typename S>
-__device__ __forceinline__ void cvt_from(uint32_t dd, bool vec, uint64_t src, uint64_t dst) {
+__device__ __forceinline__ void cvt_from(uint32_t dd, uint32_t nl, uint64_t src, uint64_t dst) {
   switch (dd) {
-    case ETHA_F16: cvt_pair<S, TagF16>(vec, src, dst); break;
-    case ETHA_BF16: cvt_pair<S, TagBF16>(vec, src, dst); break;
-    case ETHA_F32: cvt_pair<S, TagF32>(vec, src, dst); break;
-    default: cvt_pair<S, TagF64>(vec, src, dst); break;
+    case ETHA_F16: cvt_pair<S, TagF16>(nl, src, dst); break;
+    case ETHA_BF16: cvt_pair<S, TagBF16>(nl, src, dst); break;
+    case ETHA_F32: cvt_pair<S, TagF32>(nl, src, dst); break;
+    default: cvt_pair<S, TagF64>(nl, src, dst); break;
   }
 }
 
@@ -317,67 +345,92 @@ __device__ __forceinline__ int64_t trunc_i64(double f) { return (f >= -922337203
 
 __device__ __forceinline__ bool is_int_code(uint32_t dt) { return dt >= ETHA_I8 && dt <= ETHA_BOOL; }
 
-__device__ __forceinline__ int64_t load_int_elem(uint32_t dt, uint64_t addr) {
+// ---- one element as raw bits (zero-extended into 64) --------------------------------------------
+__device__ __forceinline__ uint32_t dtype_bytes(uint32_t dt) {
   switch (dt) {
-    case ETHA_I8: return (int8_t)ld_stream<uint8_t>(addr);
-    case ETHA_U8: return ld_stream<uint8_t>(addr);
-    case ETHA_BOOL: return ld_stream<uint8_t>(addr) != 0;
-    case ETHA_I16: return (int16_t)ld_stream<uint16_t>(addr);
-    case ETHA_I32: return (int32_t)ld_stream<uint32_t>(addr);
-    default: return (int64_t)ld_stream<uint64_t>(addr);
+    case ETHA_F16: case ETHA_BF16: case ETHA_B16: case ETHA_I16: return 2;
+    case ETHA_F32: case ETHA_B32: case ETHA_I32: return 4;
+    case ETHA_F64: case ETHA_B64: case ETHA_I64: return 8;
+    default: return 1;
   }
 }
-__device__ __forceinline__ void store_int_elem(uint32_t dt, uint64_t addr, int64_t v) {
-  switch (dt) {
-    case ETHA_I8: case ETHA_U8: st_stream<uint8_t>(addr, (uint8_t)v); break;
-    case ETHA_BOOL: st_stream<uint8_t>(addr, v != 0 ? 1 : 0); break;
-    case ETHA_I16: st_stream<uint16_t>(addr, (uint16_t)v); break;
-    case ETHA_I32: st_stream<uint32_t>(addr, (uint32_t)v); break;
-    default: st_stream<uint64_t>(addr, (uint64_t)v); break;
+__device__ __forceinline__ uint64_t load_bits(uint32_t bytes, uint64_t addr) {
+  switch (bytes) {
+    case 1: return ld_stream<uint8_t>(addr);
+    case 2: return ld_stream<uint16_t>(addr);
+    case 4: return ld_stream<uint32_t>(addr);
+    default: return ld_stream<uint64_t>(addr);
   }
 }
-__device__ __forceinline__ float load_float_elem(uint32_t dt, uint64_t addr) {  // every float type but f64 -> exact; f64 rounds
-  switch (dt) {
-    case ETHA_F16: return to_f32(TagF16(), ld_stream<uint16_t>(addr));
-    case ETHA_BF16: return to_f32(TagBF16(), ld_stream<uint16_t>(addr));
-    case ETHA_F32: return to_f32(TagF32(), ld_stream<uint32_t>(addr));
-    case ETHA_F8E4M3: return e4m3_to_f32(ld_stream<uint8_t>(addr));
-    case ETHA_F8E5M2: return e5m2_to_f32(ld_stream<uint8_t>(addr));
-    default: return to_f32(TagF64(), ld_stream<uint64_t>(addr));
+__device__ __forceinline__ void store_bits(uint32_t bytes, uint64_t addr, uint64_t v) {
+  switch (bytes) {
+    case 1: st_stream<uint8_t>(addr, (uint8_t)v); break;
+    case 2: st_stream<uint16_t>(addr, (uint16_t)v); break;
+    case 4: st_stream<uint32_t>(addr, (uint32_t)v); break;
+    default: st_stream<uint64_t>(addr, v); break;
   }
 }
-__device__ __forceinline__ void store_float_elem(uint32_t dt, uint64_t addr, float f) {
+__device__ __forceinline__ int64_t int_value(uint32_t dt, uint64_t bits) {
   switch (dt) {
-    case ETHA_F16: st_stream<uint16_t>(addr, from_f32(TagF16(), f)); break;
-    case ETHA_BF16: st_stream<uint16_t>(addr, from_f32(TagBF16(), f)); break;
-    case ETHA_F32: st_stream<uint32_t>(addr, from_f32(TagF32(), f)); break;
-    case ETHA_F8E4M3: st_stream<uint8_t>(addr, f32_to_e4m3(f)); break;
-    case ETHA_F8E5M2: st_stream<uint8_t>(addr, f32_to_e5m2(f)); break;
-    default: st_stream<uint64_t>(addr, from_f32(TagF64(), f)); break;
+    case ETHA_I8: return (int8_t)(uint8_t)bits;
+    case ETHA_U8: return (uint8_t)bits;
+    case ETHA_BOOL: return (uint8_t)bits != 0;
+    case ETHA_I16: return (int16_t)(uint16_t)bits;
+    case ETHA_I32: return (int32_t)(uint32_t)bits;
+    default: return (int64_t)bits;
+  }
+}
+__device__ __forceinline__ uint64_t int_bits(uint32_t dt, int64_t v) {
+  switch (dt) {
+    case ETHA_I8: case ETHA_U8: return (uint8_t)v;
+    case ETHA_BOOL: return v != 0 ? 1u : 0u;
+    case ETHA_I16: return (uint16_t)v;
+    case ETHA_I32: return (uint32_t)v;
+    default: return (uint64_t)v;
+  }
+}
+__device__ __forceinline__ float float_value(uint32_t dt, uint64_t bits) {  // every float type but f64 -> exact; f64 rounds
+  switch (dt) {
+    case ETHA_F16: return to_f32(TagF16(), (uint16_t)bits);
+    case ETHA_BF16: return to_f32(TagBF16(), (uint16_t)bits);
+    case ETHA_F32: return to_f32(TagF32(), (uint32_t)bits);
+    case ETHA_F8E4M3: return e4m3_to_f32((uint8_t)bits);
+    case ETHA_F8E5M2: return e5m2_to_f32((uint8_t)bits);
+    default: return to_f32(TagF64(), bits);
+  }
+}
+__device__ __forceinline__ uint64_t float_bits(uint32_t dt, float f) {
+  switch (dt) {
+    case ETHA_F16: return from_f32(TagF16(), f);
+    case ETHA_BF16: return from_f32(TagBF16(), f);
+    case ETHA_F32: return from_f32(TagF32(), f);
+    case ETHA_F8E4M3: return f32_to_e4m3(f);
+    case ETHA_F8E5M2: return f32_to_e5m2(f);
+    default: return from_f32(TagF64(), f);
   }
 }
 
-__device__ __forceinline__ void convert_generic(uint32_t sd, uint32_t dd, uint64_t src, uint64_t dst) {
+// Tensor.to(dtype) on one element, for every pair of value types: the element-by-element moves of the tile kernels
+// and the typed transposing blocks both go through this.
+__device__ __forceinline__ uint64_t convert_bits(uint32_t sd, uint32_t dd, uint64_t bits) {
   if (is_int_code(sd)) {
-    const int64_t v = load_int_elem(sd, src);
-    if (is_int_code(dd))
-      store_int_elem(dd, dst, v);
-    else if (dd == ETHA_F64)
-      st_stream<uint64_t>(dst, __builtin_bit_cast(uint64_t, (double)v));
-    else
-      store_float_elem(dd, dst, (float)v);  // narrower floats are built from float(value)
-    return;
+    const int64_t v = int_value(sd, bits);
+    if (is_int_code(dd)) return int_bits(dd, v);
+    if (dd == ETHA_F64) return __builtin_bit_cast(uint64_t, (double)v);
+    return float_bits(dd, (float)v);  // narrower floats are built from float(value)
   }
   if (sd == ETHA_F64 && is_int_code(dd)) {
-    const double d = __builtin_bit_cast(double, ld_stream<uint64_t>(src));
-    store_int_elem(dd, dst, dd == ETHA_BOOL ? (int64_t)(d != 0.0) : (dd == ETHA_I64 || dd == ETHA_U8) ? trunc_i64(d) : trunc_i32(d));
-    return;
+    const double d = __builtin_bit_cast(double, bits);
+    return int_bits(dd, dd == ETHA_BOOL ? (int64_t)(d != 0.0) : (dd == ETHA_I64 || dd == ETHA_U8) ? trunc_i64(d) : trunc_i32(d));
   }
-  const float f = load_float_elem(sd, src);
+  const float f = float_value(sd, bits);
   if (is_int_code(dd))
-    store_int_elem(dd, dst, dd == ETHA_BOOL ? (int64_t)(f != 0.0f) : (dd == ETHA_I64 || dd == ETHA_U8) ? trunc_i64(f) : trunc_i32(f));
-  else
-    store_float_elem(dd, dst, f);
+    return int_bits(dd, dd == ETHA_BOOL ? (int64_t)(f != 0.0f) : (dd == ETHA_I64 || dd == ETHA_U8) ? trunc_i64(f) : trunc_i32(f));
+  return float_bits(dd, f);
+}
+
+__device__ __forceinline__ void convert_generic(uint32_t sd, uint32_t dd, uint64_t src, uint64_t dst) {
+  store_bits(dtype_bytes(dd), dst, convert_bits(sd, dd, load_bits(dtype_bytes(sd), src)));
 }
 
 template <bool REV>
@@ -416,12 +469,12 @@ __device__ __forceinline__ void move_unit(uint32_t meta, uint64_t a, uint64_t b)
     convert_generic(sd, dd, src, dst);
     return;
   }
-  const bool vec = (meta & kMetaVec) != 0;
+  const uint32_t nl = (meta >> kMetaElemsShift) & 3u;
   switch (sd) {
-    case ETHA_F16: cvt_from<TagF16>(dd, vec, src, dst); break;
-    case ETHA_BF16: cvt_from<TagBF16>(dd, vec, src, dst); break;
-    case ETHA_F32: cvt_from<TagF32>(dd, vec, src, dst); break;
-    default: cvt_from<TagF64>(dd, vec, src, dst); break;
+    case ETHA_F16: cvt_from<TagF16>(dd, nl, src, dst); break;
+    case ETHA_BF16: cvt_from<TagBF16>(dd, nl, src, dst); break;
+    case ETHA_F32: cvt_from<TagF32>(dd, nl, src, dst); break;
+    default: cvt_from<TagF64>(dd, nl, src, dst); break;
   }
 }
 
@@ -839,6 +892,7 @@ __device__ __forceinline__ void transpose_block(const TransTile& t, uint8_t* __r
 
 template <bool REV>
 __device__ __forceinline__ void transpose_tile(const TransTile& t, uint8_t* __restrict__ lds) {
+  if (t.cvt & kTransTyped) return;  // a block of the typed kernel (uniform over the workgroup: no barrier is skipped)
   if (t.cvt) {  // f32 on the a side, f16 or bf16 on the b side
     if ((t.cvt & 15u) == ETHA_F16)
       transpose_block_cvt<TagF16, REV>(t, lds);
@@ -1040,33 +1094,42 @@ __device__ __forceinline__ void reduce_f64(const uint64_t* __restrict__ peers, u
   out.store(dst);
 }
 
+template <typename S, typename D, int N>
+__device__ __forceinline__ void reduce_n(const uint64_t* peers, uint32_t np, uint32_t op, uint32_t via, uint64_t a_off,
+                                         uint64_t dst) {
+  if constexpr (sizeof(typename S::bits) == 8)
+    reduce_f64<D, N>(peers, np, op, via, a_off, dst);
+  else
+    reduce_f32<S, D, N>(peers, np, op, via, a_off, dst);
+}
+
+// nl = log2 of the elements in this unit (at most 16 bytes on the wider side)
 template <typename S, typename D>
-__device__ __forceinline__ void reduce_pair(bool vec, const uint64_t* peers, uint32_t np, uint32_t op, uint32_t via,
+__device__ __forceinline__ void reduce_pair(uint32_t nl, const uint64_t* peers, uint32_t np, uint32_t op, uint32_t via,
                                             uint64_t a_off, uint64_t dst) {
   constexpr int kMaxBytes = sizeof(typename S::bits) > sizeof(typename D::bits) ? sizeof(typename S::bits)
                                                                                   : sizeof(typename D::bits);
   constexpr int kN = 16 / kMaxBytes;
-  if (sizeof(typename S::bits) == 8) {
-    if (vec)
-      reduce_f64<D, kN>(peers, np, op, via, a_off, dst);
-    else
-      reduce_f64<D, 1>(peers, np, op, via, a_off, dst);
-  } else {
-    if (vec)
-      reduce_f32<S, D, kN>(peers, np, op, via, a_off, dst);
-    else
-      reduce_f32<S, D, 1>(peers, np, op, via, a_off, dst);
+  if constexpr (kN >= 8) {
+    if (nl == 3) return reduce_n<S, D, 8>(peers, np, op, via, a_off, dst);
   }
+  if constexpr (kN >= 4) {
+    if (nl == 2) return reduce_n<S, D, 4>(peers, np, op, via, a_off, dst);
+  }
+  if constexpr (kN >= 2) {
+    if (nl == 1) return reduce_n<S, D, 2>(peers, np, op, via, a_off, dst);
+  }
+  reduce_n<S, D, 1>(peers, np, op, via, a_off, dst);
 }
 
 template <typename S>
-__device__ __forceinline__ void reduce_from(uint32_t dd, bool vec, const uint64_t* peers, uint32_t np, uint32_t op,
+__device__ __forceinline__ void reduce_from(uint32_t dd, uint32_t nl, const uint64_t* peers, uint32_t np, uint32_t op,
                                             uint32_t via, uint64_t a_off, uint64_t dst) {
   switch (dd) {
-    case ETHA_F16: reduce_pair<S, TagF16>(vec, peers, np, op, via, a_off, dst); break;
-    case ETHA_BF16: reduce_pair<S, TagBF16>(vec, peers, np, op, via, a_off, dst); break;
-    case ETHA_F32: reduce_pair<S, TagF32>(vec, peers, np, op, via, a_off, dst); break;
-    default: reduce_pair<S, TagF64>(vec, peers, np, op, via, a_off, dst); break;
+    case ETHA_F16: reduce_pair<S, TagF16>(nl, peers, np, op, via, a_off, dst); break;
+    case ETHA_BF16: reduce_pair<S, TagBF16>(nl, peers, np, op, via, a_off, dst); break;
+    case ETHA_F32: reduce_pair<S, TagF32>(nl, peers, np, op, via, a_off, dst); break;
+    default: reduce_pair<S, TagF64>(nl, peers, np, op, via, a_off, dst); break;
   }
 }
 
@@ -1081,13 +1144,247 @@ __global__ __launch_bounds__(ETHA_BLOCK_THREADS) void etha_reduce_kernel(const R
   const uint64_t a_off = t.a + (uint64_t)((int64_t)r * t.a_pitch) + ((uint64_t)c << ((meta >> kMetaUaShift) & 15u));
   const uint64_t dst = t.b + (uint64_t)((int64_t)r * t.b_pitch) + ((uint64_t)c << ((meta >> kMetaUbShift) & 15u));
   const uint64_t* peers = peer_bases + t.peer_first;
-  const bool vec = (meta & kMetaVec) != 0;
+  const uint32_t nl = (meta >> kMetaElemsShift) & 3u;
   const uint32_t dd = (meta >> kMetaDtbShift) & 15u;
   switch ((meta >> kMetaDtaShift) & 15u) {
-    case ETHA_F16: reduce_from<TagF16>(dd, vec, peers, t.n_peers, t.reduce_op, t.via, a_off, dst); break;
-    case ETHA_BF16: reduce_from<TagBF16>(dd, vec, peers, t.n_peers, t.reduce_op, t.via, a_off, dst); break;
-    case ETHA_F32: reduce_from<TagF32>(dd, vec, peers, t.n_peers, t.reduce_op, t.via, a_off, dst); break;
-    default: reduce_from<TagF64>(dd, vec, peers, t.n_peers, t.reduce_op, t.via, a_off, dst); break;
+    case ETHA_F16: reduce_from<TagF16>(dd, nl, peers, t.n_peers, t.reduce_op, t.via, a_off, dst); break;
+    case ETHA_BF16: reduce_from<TagBF16>(dd, nl, peers, t.n_peers, t.reduce_op, t.via, a_off, dst); break;
+    case ETHA_F32: reduce_from<TagF32>(dd, nl, peers, t.n_peers, t.reduce_op, t.via, a_off, dst); break;
+    default: reduce_from<TagF64>(dd, nl, peers, t.n_peers, t.reduce_op, t.via, a_off, dst); break;
+  }
+}
+
+// ---- typed transposing blocks -------------------------------------------------------------------
+// Transposing chunks that the plain transposing kernel does not take: any pair of value types, and Partial sources
+// (the N members' blocks are combined in registers, strictly in list order, as the reduce kernel combines rows).
+// The source side is read with 16-byte vectors along its contiguous dim, every element is converted to the
+// destination's type (reduced first, for a Partial source) and parked in LDS, and the destination side is written
+// by the same gather-from-LDS step the plain blocks use.  Edge blocks move element by element.
+template <typename ES, int N, bool RED>
+__device__ __forceinline__ void typed_values(uint32_t sd, uint32_t dd, uint64_t src, const uint64_t* __restrict__ peers,
+                                             uint32_t np, uint32_t op, uint32_t via, uint64_t (&out)[N]) {
+  Pack<ES, N> in;
+  if constexpr (!RED) {
+    in.load(src);
+#pragma unroll
+    for (int e = 0; e < N; e++) out[e] = convert_bits(sd, dd, (uint64_t)in.get(e));
+    return;
+  }
+  // Partial source: src is an offset from each member's base; f16/bf16/f32 accumulate in fp32, f64 in f64
+  if (sd == ETHA_F64) {
+    double acc[N];
+    in.load(peers[0] + src);
+#pragma unroll
+    for (int e = 0; e < N; e++) acc[e] = __builtin_bit_cast(double, (uint64_t)in.get(e));
+    for (uint32_t p = 1; p < np; p++) {
+      in.load(peers[p] + src);
+#pragma unroll
+      for (int e = 0; e < N; e++) acc[e] = combine(op, acc[e], __builtin_bit_cast(double, (uint64_t)in.get(e)));
+    }
+#pragma unroll
+    for (int e = 0; e < N; e++) {
+      double r = acc[e];
+      if (op == ETHA_AVG) r = r / (double)np;
+      if (dd == ETHA_F64 && via == 0) {
+        out[e] = __builtin_bit_cast(uint64_t, r);
+      } else {
+        float rf = (float)r;
+        asm volatile("" : "+v"(rf));  // two roundings, as in the plain f64 -> narrower move
+        out[e] = float_bits(dd, round_via(via, rf));
+      }
+    }
+    return;
+  }
+  float acc[N];
+  in.load(peers[0] + src);
+#pragma unroll
+  for (int e = 0; e < N; e++) acc[e] = float_value(sd, (uint64_t)in.get(e));
+  for (uint32_t p = 1; p < np; p++) {
+    in.load(peers[p] + src);
+#pragma unroll
+    for (int e = 0; e < N; e++) acc[e] = combine(op, acc[e], float_value(sd, (uint64_t)in.get(e)));
+  }
+  const float cnt = (float)np;
+#pragma unroll
+  for (int e = 0; e < N; e++) {
+    float r = acc[e];
+    if (op == ETHA_AVG) r = r / cnt;
+    out[e] = float_bits(dd, round_via(via, r));
+  }
+}
+
+// Full block of a Partial source whose members hold f16, bf16 or f32: the loads of up to four members are in flight
+// together (a member's vectors only meet the accumulators once all of the batch have been requested), members are
+// still combined strictly in list order, and all conversions are straight-line code.
+template <typename S, typename D, uint32_t DX, uint32_t DY>
+__device__ __forceinline__ void reduce_block_full(const TransTile& t, const uint64_t* __restrict__ peers, uint8_t* __restrict__ lds) {
+  typedef typename S::bits ES;
+  typedef typename D::bits ED;
+  constexpr uint32_t kVs = 16 / sizeof(ES), kVecPerRow = DX / kVs, kVecs = DY * kVecPerRow, kPer = kVecs / kTransThreads;
+  static_assert(kVecs % kTransThreads == 0 && kPer >= 1, "a whole number of vectors per work-item");
+  constexpr uint32_t kPitchBytes = trans_pitch(DX, sizeof(ED)) * sizeof(ED);
+  constexpr uint32_t kBatch = 2;  // members whose loads are in flight together
+  const uint32_t tid = threadIdx.x, np = t.n_peers, op = t.reduce_op, via = t.via;
+  uint64_t off[kPer];
+#pragma unroll
+  for (uint32_t i = 0; i < kPer; i++) {
+    const uint32_t q = tid + i * kTransThreads, y = q / kVecPerRow, xv = q % kVecPerRow;
+    off[i] = t.a + (uint64_t)((int64_t)y * t.a_pitch) + xv * 16u;
+  }
+  float acc[kPer][kVs];
+  for (uint32_t p = 0; p < np; p += kBatch) {
+    Pack<ES, kVs> raw[kBatch][kPer];
+#pragma unroll
+    for (uint32_t j = 0; j < kBatch; j++)
+      if (p + j < np) {
+        const uint64_t base = peers[p + j];
+#pragma unroll
+        for (uint32_t i = 0; i < kPer; i++) raw[j][i].load(base + off[i]);
+      }
+#pragma unroll
+    for (uint32_t j = 0; j < kBatch; j++)
+      if (p + j < np) {
+#pragma unroll
+        for (uint32_t i = 0; i < kPer; i++)
+#pragma unroll
+          for (uint32_t e = 0; e < kVs; e++) {
+            const float v = to_f32(S(), raw[j][i].get(e));
+            acc[i][e] = (p + j == 0) ? v : combine(op, acc[i][e], v);
+          }
+      }
+  }
+  const float cnt = (float)np;
+#pragma unroll
+  for (uint32_t i = 0; i < kPer; i++) {
+    const uint32_t q = tid + i * kTransThreads, y = q / kVecPerRow, xv = q % kVecPerRow;
+    ED* row = reinterpret_cast<ED*>(lds + y * kPitchBytes) + xv * kVs;
+#pragma unroll
+    for (uint32_t e = 0; e < kVs; e++) {
+      float r = acc[i][e];
+      if (op == ETHA_AVG) r = r / cnt;
+      row[e] = from_f32(D(), round_via(via, r));
+    }
+  }
+  __syncthreads();
+  TransBlock<ED, DX, DY>::emit(lds, t.b, t.b_pitch);
+}
+
+template <typename S, typename ED, uint32_t DX, uint32_t DY>
+__device__ __forceinline__ bool reduce_block_to(uint32_t dd, const TransTile& t, const uint64_t* __restrict__ peers, uint8_t* __restrict__ lds) {
+  if constexpr (sizeof(ED) == 2) {
+    if (dd == ETHA_F16) {
+      reduce_block_full<S, TagF16, DX, DY>(t, peers, lds);
+      return true;
+    }
+    if (dd == ETHA_BF16) {
+      reduce_block_full<S, TagBF16, DX, DY>(t, peers, lds);
+      return true;
+    }
+  }
+  if constexpr (sizeof(ED) == 4) {
+    if (dd == ETHA_F32) {
+      reduce_block_full<S, TagF32, DX, DY>(t, peers, lds);
+      return true;
+    }
+  }
+  return false;
+}
+
+template <typename ES, typename ED, bool RED>
+__device__ __forceinline__ void typed_block(const TransTile& t, bool rev, const uint64_t* __restrict__ peer_bases, uint8_t* __restrict__ lds) {
+  constexpr uint32_t kD = trans_typed_dim(sizeof(ES), sizeof(ED));
+  constexpr uint32_t kPitchBytes = trans_pitch(kD, sizeof(ED)) * sizeof(ED);
+  const uint32_t dta = (t.cvt >> 4) & 15u, dtb = t.cvt & 15u;
+  const uint32_t sd = rev ? dtb : dta, dd = rev ? dta : dtb;
+  const uint64_t src = rev ? t.b : t.a, dst = rev ? t.a : t.b;
+  const int64_t src_pitch = rev ? t.b_pitch : t.a_pitch, dst_pitch = rev ? t.a_pitch : t.b_pitch;
+  const uint32_t nx = rev ? t.nk : t.nj, ny = rev ? t.nj : t.nk;  // elements per source row, source rows
+  const uint64_t* peers = peer_bases + t.peer_first;
+  const uint32_t np = t.n_peers, op = t.reduce_op, via = t.via, tid = threadIdx.x;
+  if constexpr (RED && sizeof(ES) == 2 && sizeof(ED) <= 4) {  // f16 / bf16 members: the straight-line path, its own block shape
+    if (nx == kRedDimJ2 && ny == kRedDimK2) {
+      bool done = false;
+      if (sd == ETHA_F16) done = reduce_block_to<TagF16, ED, kRedDimJ2, kRedDimK2>(dd, t, peers, lds);
+      if (sd == ETHA_BF16) done = reduce_block_to<TagBF16, ED, kRedDimJ2, kRedDimK2>(dd, t, peers, lds);
+      if (done) return;
+    }
+  }
+  if (nx == kD && ny == kD) {
+    if constexpr (RED && sizeof(ES) == 4 && sizeof(ED) <= 4) {  // f32 members
+      if (sd == ETHA_F32 && reduce_block_to<TagF32, ED, kD, kD>(dd, t, peers, lds)) return;
+    }
+    constexpr uint32_t kVs = 16 / sizeof(ES), kVecPerRow = kD / kVs, kVecs = kD * kVecPerRow;
+    constexpr uint32_t kPerThread = (kVecs + kTransThreads - 1) / kTransThreads;
+#pragma unroll
+    for (uint32_t i = 0; i < kPerThread; i++) {
+      const uint32_t q = tid + i * kTransThreads, y = q / kVecPerRow, xv = q % kVecPerRow;
+      if (kVecs % kTransThreads == 0 || q < kVecs) {
+        uint64_t v[kVs];
+        typed_values<ES, (int)kVs, RED>(sd, dd, src + (uint64_t)((int64_t)y * src_pitch) + xv * 16u, peers, np, op, via, v);
+        ED* row = reinterpret_cast<ED*>(lds + y * kPitchBytes) + xv * kVs;
+#pragma unroll
+        for (uint32_t e = 0; e < kVs; e++) row[e] = (ED)v[e];
+      }
+    }
+    __syncthreads();
+    TransBlock<ED, kD, kD>::emit(lds, dst, dst_pitch);
+    return;
+  }
+  const uint32_t n = nx * ny;
+  for (uint32_t q = tid; q < n; q += kTransThreads) {
+    const uint32_t y = q / nx, x = q - y * nx;
+    uint64_t v[1];
+    typed_values<ES, 1, RED>(sd, dd, src + (uint64_t)((int64_t)y * src_pitch) + (uint64_t)x * sizeof(ES), peers, np, op, via, v);
+    *reinterpret_cast<ED*>(lds + y * kPitchBytes + x * sizeof(ED)) = (ED)v[0];
+  }
+  __syncthreads();
+  for (uint32_t q = tid; q < n; q += kTransThreads) {
+    const uint32_t x = q / ny, y = q - x * ny;
+    st_stream<ED>(dst + (uint64_t)((int64_t)x * dst_pitch) + (uint64_t)y * sizeof(ED),
+                  *reinterpret_cast<const ED*>(lds + y * kPitchBytes + x * sizeof(ED)));
+  }
+}
+
+template <typename ES, bool RED>
+__device__ __forceinline__ void typed_block_to(uint32_t dst_bytes, const TransTile& t, bool rev, const uint64_t* __restrict__ peers,
+                                               uint8_t* __restrict__ lds) {
+  switch (dst_bytes) {
+    case 1:
+      if constexpr (!RED) typed_block<ES, uint8_t, RED>(t, rev, peers, lds);  // no 1-byte float takes part in a reduction
+      break;
+    case 2: typed_block<ES, uint16_t, RED>(t, rev, peers, lds); break;
+    case 4: typed_block<ES, uint32_t, RED>(t, rev, peers, lds); break;
+    default: typed_block<ES, uint64_t, RED>(t, rev, peers, lds); break;
+  }
+}
+
+// blocks that convert between two value types (no Partial source); rev = unpack direction
+__global__ __launch_bounds__(ETHA_TRANS_THREADS) void etha_transpose_typed_kernel(const TransTile* __restrict__ tiles, uint32_t rev) {
+  extern __shared__ __attribute__((aligned(16))) uint8_t lds_bytes[];
+  const TransTile t = tiles[blockIdx.x];
+  if (!(t.cvt & kTransTyped) || t.n_peers) return;  // another kernel's block (the whole workgroup leaves)
+  const uint32_t dta = (t.cvt >> 4) & 15u, dtb = t.cvt & 15u;
+  const uint32_t src_bytes = dtype_bytes(rev ? dtb : dta), dst_bytes = dtype_bytes(rev ? dta : dtb);
+  switch (src_bytes) {
+    case 1: typed_block_to<uint8_t, false>(dst_bytes, t, rev != 0, nullptr, lds_bytes); break;
+    case 2: typed_block_to<uint16_t, false>(dst_bytes, t, rev != 0, nullptr, lds_bytes); break;
+    case 4: typed_block_to<uint32_t, false>(dst_bytes, t, rev != 0, nullptr, lds_bytes); break;
+    default: typed_block_to<uint64_t, false>(dst_bytes, t, rev != 0, nullptr, lds_bytes); break;
+  }
+}
+
+// blocks of a Partial source whose members are stored transposed (pack direction only)
+// (eight waves per SIMD, i.e. two workgroups per CU: with 64 registers the two-member batches fit without spills)
+__global__ __launch_bounds__(ETHA_TRANS_THREADS, 8) void etha_transpose_reduce_kernel(const TransTile* __restrict__ tiles,
+                                                                                    const uint64_t* __restrict__ peer_bases) {
+  extern __shared__ __attribute__((aligned(16))) uint8_t lds_bytes[];
+  const TransTile t = tiles[blockIdx.x];
+  if (!(t.cvt & kTransTyped) || !t.n_peers) return;
+  const uint32_t dta = (t.cvt >> 4) & 15u, dtb = t.cvt & 15u;
+  switch (dtype_bytes(dta)) {
+    case 2: typed_block_to<uint16_t, true>(dtype_bytes(dtb), t, false, peer_bases, lds_bytes); break;
+    case 4: typed_block_to<uint32_t, true>(dtype_bytes(dtb), t, false, peer_bases, lds_bytes); break;
+    default: typed_block_to<uint64_t, true>(dtype_bytes(dtb), t, false, peer_bases, lds_bytes); break;
   }
 }
 
@@ -1330,23 +1627,37 @@ class PairCompiler {
   // kernel in blocks of trans_dim_a x trans_dim_b elements; all other dims are unrolled here.
   int try_transposing(bool* done) {
     *done = false;
-    // same element type on both sides, or f32 on the a side with f16 / bf16 in the bucket (converted on the way)
+    // same element type on both sides, or f32 on the a side with f16 / bf16 in the bucket (converted on the way):
+    // blocks of the plain transposing kernel.  Every other pair of value types, and Partial sources reduced with one
+    // op, take the blocks of the typed kernel (a Partial source with nested levels keeps its row tiles).
     const bool converting = cvt_ && red_.n_peers == 0 && dta_ == ETHA_F32 && (dtb_ == ETHA_F16 || dtb_ == ETHA_BF16);
-    if (!(run_elems_ == 1 && (plain_ || converting) && k_ >= 2 && sb_[k_ - 1] == esb_ && sa_[k_ - 1] != esa_)) return ETHA_OK;
+    const bool typed = !plain_ && !converting && is_typed(dta_) && is_typed(dtb_) && (red_.op >> 16) == 0;
+    if (!(run_elems_ == 1 && (plain_ || converting || typed) && k_ >= 2 && sb_[k_ - 1] == esb_ && sa_[k_ - 1] != esa_)) return ETHA_OK;
     int j = -1;
     for (int i = 0; i < k_ - 1; i++)
       if (sa_[i] == esa_ && n_[i] >= 8) j = i;
     const int kk = k_ - 1;
     if (j < 0 || n_[kk] < 8 || (A_.base % (uint64_t)esa_) != 0 || (B_.base % (uint64_t)esb_) != 0) return ETHA_OK;
+    for (uint64_t p : align_bases_)
+      if (p % (uint64_t)esa_) return ETHA_OK;  // the row tiles report the misaligned member
+    for (int i = 0; i < k_; i++)
+      if (sa_[i] % esa_ || sb_[i] % esb_) return ETHA_OK;
     int64_t pos[ETHA_MAX_NDIM] = {0};
     uint64_t off_a = 0, off_b = 0;
-    // blocks are sized by the element that goes through LDS: the b side's
-    const int64_t kDimJ = (int64_t)trans_dim_a((uint32_t)esb_), kDimK = (int64_t)trans_dim_b((uint32_t)esb_);
+    // blocks are sized by the element that goes through LDS: the b side's (typed blocks: by the wider side)
+    const int64_t kDimJ = typed ? (int64_t)trans_typed_dim((uint32_t)esa_, (uint32_t)esb_) : (int64_t)trans_dim_a((uint32_t)esb_);
+    const int64_t kDimK = typed ? kDimJ : (int64_t)trans_dim_b((uint32_t)esb_);
     // the part of the chunk that whole wide blocks cover; blocks of the plain extent (and edge blocks) cover the rest
-    const int64_t kP = (int64_t)trans_wide((uint32_t)esb_);
-    const int64_t wide_dim_j = converting ? (int64_t)kTransCvtWideJ : kDimJ * kP, wide_dim_k = converting ? (int64_t)kTransCvtWideK : kDimK * kP;
-    const bool has_wide = wide_dim_j > kDimJ || wide_dim_k > kDimK;
-    const int64_t wide_j = has_wide ? n_[j] / wide_dim_j * wide_dim_j : 0, wide_k = has_wide ? n_[kk] / wide_dim_k * wide_dim_k : 0;
+    const int64_t kP = typed ? 1 : (int64_t)trans_wide((uint32_t)esb_);
+    // Partial members of 2-byte elements have a block shape of their own
+    const bool red_shape = typed && red_.n_peers && esa_ == 2 && esb_ <= 4 && (dta_ == ETHA_F16 || dta_ == ETHA_BF16) && dtb_ <= ETHA_F32;
+    const int64_t wide_dim_j = red_shape ? (int64_t)kRedDimJ2 : converting ? (int64_t)kTransCvtWideJ : kDimJ * kP;
+    const int64_t wide_dim_k = red_shape ? (int64_t)kRedDimK2 : converting ? (int64_t)kTransCvtWideK : kDimK * kP;
+    const bool has_wide = wide_dim_j != kDimJ || wide_dim_k != kDimK;
+    // the region the wide blocks cover ends where blocks of the plain extent can take over
+    const auto lcm = [](int64_t x, int64_t y) { int64_t a = x, b = y; while (b) { const int64_t r = a % b; a = b; b = r; } return x / a * y; };
+    const int64_t step_j = lcm(wide_dim_j, kDimJ), step_k = lcm(wide_dim_k, kDimK);
+    const int64_t wide_j = has_wide ? n_[j] / step_j * step_j : 0, wide_k = has_wide ? n_[kk] / step_k * step_k : 0;
     const bool wide = wide_j > 0 && wide_k > 0;
     do {
       // Launch order.  Blocks are grouped into super-blocks of S x S blocks that are emitted together: blocks
@@ -1379,7 +1690,11 @@ class PairCompiler {
                 t.nj = (uint32_t)(j_end - j0 < dim_j ? j_end - j0 : dim_j);
                 t.nk = (uint32_t)(k_end - k0 < dim_k ? k_end - k0 : dim_k);
                 t.es_log2 = (uint32_t)log2u((uint64_t)esb_);
-                t.cvt = converting ? (dta_ << 4) | dtb_ : 0u;
+                t.cvt = converting ? (dta_ << 4) | dtb_ : typed ? ((dta_ << 4) | dtb_ | kTransTyped) : 0u;
+                t.peer_first = red_.peer_first;
+                t.n_peers = red_.n_peers;
+                t.reduce_op = red_.op;
+                t.via = red_.via;
                 bld_.trans.push_back(t);
               }
         return ETHA_OK;
@@ -1476,30 +1791,33 @@ class PairCompiler {
     return ETHA_OK;
   }
 
-  // Converting and reducing moves: whole vectors of `epv` elements (the narrow side moves up to 16 bytes;
-  // converting moves may use two accesses on the wide side, reductions one) when the run is a multiple of
-  // that; else a body of whole vectors plus a remainder of single elements; runs shorter than one vector
-  // single elements.
+  // Converting and reducing moves: a row is cut into whole vectors of `epv` elements (the narrow side moves up to 16
+  // bytes; converting moves may use two accesses on the wide side, reductions one) and a remainder, which moves in
+  // narrower vectors of 4 or 2 elements before single elements are used: each width is an ordinary, densely
+  // packed tile set over the same rows.
   int compile_typed_move() {
     if (!(is_float(dta_) && is_float(dtb_)))  // an integer, bool or 8-bit float side: element by element
       return emit(A_.base, B_.base, run_elems_, (uint64_t)esa_, (uint64_t)esb_,
                   dt_bits_ | kMetaCvt | kMetaGeneric | unit_bits(log2u((uint64_t)esa_), log2u((uint64_t)esb_)));
     const int epv = red_.n_peers ? 16 / (esa_ > esb_ ? esa_ : esb_) : cvt_elems_per_unit(esa_, esb_);
-    const int ea = log2u((uint64_t)esa_), eb = log2u((uint64_t)esb_);
-    const int va = log2u((uint64_t)(epv * esa_)), vb = log2u((uint64_t)(epv * esb_));
-    const uint32_t vec_meta = dt_bits_ | kMetaCvt | kMetaVec | unit_bits(va, vb) | skew_bits(va, vb);
-    // element units are always aligned (checked by the caller), so they carry no skew flags
-    const uint32_t elem_meta = dt_bits_ | kMetaCvt | unit_bits(ea, eb);
-    if (epv > 1 && run_elems_ % (uint64_t)epv == 0)
-      return emit(A_.base, B_.base, run_elems_ / (uint64_t)epv, 1ull << va, 1ull << vb, vec_meta);
-    if (epv > 1 && run_elems_ > (uint64_t)epv) {
-      const uint64_t body_units = run_elems_ / (uint64_t)epv, rem_elems = run_elems_ % (uint64_t)epv;
-      const int rc = emit(A_.base, B_.base, body_units, 1ull << va, 1ull << vb, vec_meta);
+    uint64_t done = 0, left = run_elems_;
+    int v = epv;  // elements per unit: a power of two
+    while (left) {
+      while ((uint64_t)v > left) v >>= 1;
+      const uint64_t units = left / (uint64_t)v, off_a = done * (uint64_t)esa_, off_b = done * (uint64_t)esb_;
+      const int va = log2u((uint64_t)(v * esa_)), vb = log2u((uint64_t)(v * esb_));
+      // single elements are always aligned (checked by the caller); wider units may sit at any element boundary
+      const uint32_t skew = v == 1 ? 0u
+                                   : ((((mask_a_ | off_a) & ((1ull << va) - 1)) ? kMetaSkew : 0u) |
+                                      (((mask_b_ | off_b) & ((1ull << vb) - 1)) ? kMetaSkewB : 0u));
+      const uint32_t meta = dt_bits_ | kMetaCvt | (v == epv && epv > 1 ? kMetaVec : 0u) |
+                            ((uint32_t)log2u((uint64_t)v) << kMetaElemsShift) | unit_bits(va, vb) | skew;
+      const int rc = emit(A_.base + off_a, B_.base + off_b, units, 1ull << va, 1ull << vb, meta);
       if (rc != ETHA_OK) return rc;
-      return emit(A_.base + body_units * (uint64_t)(epv * esa_), B_.base + body_units * (uint64_t)(epv * esb_), rem_elems,
-                  (uint64_t)esa_, (uint64_t)esb_, elem_meta);
+      done += units * (uint64_t)v;
+      left -= units * (uint64_t)v;
     }
-    return emit(A_.base, B_.base, run_elems_, (uint64_t)esa_, (uint64_t)esb_, elem_meta);
+    return ETHA_OK;
   }
 
   // Tiles for rows of `run_units` units starting at base_a / base_b.  Long or tile-multiple rows (and
@@ -1592,6 +1910,7 @@ struct EthaTable {
   std::vector<RowTile> h_row;
   std::vector<TransTile> h_trans;
   std::vector<uint32_t> run_begin, row_begin, trans_begin;
+  std::vector<uint32_t> typed_begin;    // number of typed transposing tiles before chunk i's
   std::vector<uint32_t> reduce_prefix;  // number of reduce chunks before chunk i
   std::vector<uint64_t> h_peers;
   RunTile* d_run = nullptr;
@@ -1621,6 +1940,12 @@ struct EthaTable {
 };
 
 namespace {
+
+// LDS bytes a transposing tile needs
+uint32_t trans_tile_lds(const TransTile& tt) {
+  if (tt.cvt & kTransTyped) return trans_typed_lds_bytes((uint32_t)dtype_size((tt.cvt >> 4) & 15u), (uint32_t)dtype_size(tt.cvt & 15u));
+  return trans_lds_bytes(1u << tt.es_log2);
+}
 
 // tables that exist, by address -> serial; a schedule checks its tables against this before it launches
 std::mutex g_tables_mutex;
@@ -1685,7 +2010,13 @@ int finish_table(Builder& bld, EthaTable* t, const uint64_t* partial_ptrs, uint3
     t->row_begin.swap(bld.row_begin);
     t->trans_begin.swap(bld.trans_begin);
     for (const TransTile& tt : t->h_trans)
-      if (trans_lds_bytes(1u << tt.es_log2) > t->trans_lds) t->trans_lds = trans_lds_bytes(1u << tt.es_log2);
+      if (trans_tile_lds(tt) > t->trans_lds) t->trans_lds = trans_tile_lds(tt);
+    t->typed_begin.assign(t->n_chunks + 1, 0);
+    for (uint32_t i = 0; i < t->n_chunks; i++) {
+      uint32_t typed = 0;
+      for (uint32_t k = t->trans_begin[i]; k < t->trans_begin[i + 1]; k++) typed += (t->h_trans[k].cvt & kTransTyped) ? 1u : 0u;
+      t->typed_begin[i + 1] = t->typed_begin[i] + typed;
+    }
     t->reduce_prefix.assign(t->n_chunks + 1, 0);
     for (uint32_t i = 0; i < t->n_chunks; i++) t->reduce_prefix[i + 1] = t->reduce_prefix[i] + bld.is_reduce[i];
     t->payload_bytes = bld.payload_bytes;
@@ -1736,9 +2067,11 @@ void launch_kernel(F kernel, dim3 grid, dim3 block, size_t lds, void* stream, ui
 // One kernel launch with everything resolved: which kernel, its grid and its arguments.  Every entry point
 // first plans its launches into a list of these and then issues the list; a schedule (etha_schedule_create)
 // keeps such lists, so that re-issuing a whole transfer is a loop over ready-made launches.
-enum : uint32_t { kKernelTile = 0, kKernelTile2D, kKernelGather, kKernelMixed, kKernelTrans, kKernelTrans2D, kKernelReduce };
+enum : uint32_t { kKernelTile = 0, kKernelTile2D, kKernelGather, kKernelMixed, kKernelTrans, kKernelTrans2D, kKernelReduce,
+                  kKernelTransTyped, kKernelTransReduce };
 const char* const kKernelNames[] = {"etha_tile_kernel", "etha_tile_kernel_2d", "etha_gather_kernel", "etha_unpack_mixed_kernel",
-                                    "etha_transpose_kernel", "etha_transpose_kernel_2d", "etha_reduce_kernel"};
+                                    "etha_transpose_kernel", "etha_transpose_kernel_2d", "etha_reduce_kernel",
+                                    "etha_transpose_typed_kernel", "etha_transpose_reduce_kernel"};
 
 struct PreparedLaunch {
   uint32_t kernel;  // kKernel*
@@ -1752,8 +2085,9 @@ struct PreparedLaunch {
       const uint64_t* gather;
       uint32_t n_run, n_plain, n_gather;
     } tile;
-    struct {
+    struct {  // kKernelTrans, kKernelTransTyped
       const TransTile* tiles;
+      const uint64_t* peers;
     } trans;
     struct {
       const RowTile* row;
@@ -1810,6 +2144,12 @@ void issue_one(const PreparedLaunch& p, void* stream, uint32_t flags) {
         launch_kernel(etha_transpose_kernel_2d<true>, grid, block, p.lds, stream, flags, p.u.t2d);
       else
         launch_kernel(etha_transpose_kernel_2d<false>, grid, block, p.lds, stream, flags, p.u.t2d);
+      break;
+    case kKernelTransTyped:
+      launch_kernel(etha_transpose_typed_kernel, grid, block, p.lds, stream, flags, p.u.trans.tiles, p.rev);
+      break;
+    case kKernelTransReduce:
+      launch_kernel(etha_transpose_reduce_kernel, grid, block, p.lds, stream, flags, p.u.trans.tiles, p.u.trans.peers);
       break;
     default:
       launch_kernel(etha_reduce_kernel, grid, block, 0, stream, flags, p.u.reduce.row, p.u.reduce.peers);
@@ -1895,12 +2235,31 @@ void plan_trans(const TransTile* tiles, uint32_t n, bool rev, uint32_t lds, uint
 
 // One chunk range as the single-range entry points run it: the transposing tiles in their kernel, then the
 // plain tiles - and, for an unpack range with a write-ordered copy, its gather tiles in the same launch.
-void plan_tiles(const EthaTable* t, uint32_t first, uint32_t count, bool rev, uint32_t flags, LaunchList& out) {
+// The typed transposing tiles of a chunk range.  Plain and typed tiles share one list in chunk order; a range that
+// holds both is walked by both kernels, each leaving the other's blocks alone.
+bool plan_typed(const EthaTable* t, uint32_t first, uint32_t count, bool rev, uint32_t flags, LaunchList& out) {
   const uint32_t x0 = t->trans_begin[first], n_trans = t->trans_begin[first + count] - x0;
+  if (t->typed_begin[first + count] == t->typed_begin[first]) return false;
+  // a chunk range is all Partial chunks or none (the entry points check): its typed tiles are all of one kind
+  const bool reduce = t->reduce_prefix[first + count] != t->reduce_prefix[first];
+  PreparedLaunch p = new_launch(reduce ? kKernelTransReduce : kKernelTransTyped, rev, flags, n_trans, 1, kTransThreads, t->trans_lds);
+  p.u.trans.tiles = t->d_trans + x0;
+  p.u.trans.peers = t->d_peers;
+  out.push_back(p);
+  return true;
+}
+uint32_t plain_trans_tiles(const EthaTable* t, uint32_t first, uint32_t count) {  // 0: none of the range's tiles is a plain one
+  const uint32_t n_trans = t->trans_begin[first + count] - t->trans_begin[first];
+  return n_trans - (t->typed_begin[first + count] - t->typed_begin[first]) ? n_trans : 0u;
+}
+
+void plan_tiles(const EthaTable* t, uint32_t first, uint32_t count, bool rev, uint32_t flags, LaunchList& out) {
+  const uint32_t x0 = t->trans_begin[first], n_trans = plain_trans_tiles(t, first, count);
   if (n_trans) {
     plan_trans(t->d_trans + x0, n_trans, rev, t->trans_lds, flags, out);
-    flags |= ETHA_LAUNCH_UNORDERED;  // the two kernels of one call touch different chunks
+    flags |= ETHA_LAUNCH_UNORDERED;  // the kernels of one call touch different chunks
   }
+  if (plan_typed(t, first, count, rev, flags, out)) flags |= ETHA_LAUNCH_UNORDERED;
   const Seg2D g = tile_range(t, first, count, rev);
   const Seg2D gathered = gather_range(t, first, count, rev);
   if (g.n_tiles && gathered.n_tiles) {  // the gather tiles follow the plain row tiles in the ordered copy
@@ -1921,6 +2280,7 @@ void plan_tiles(const EthaTable* t, uint32_t first, uint32_t count, bool rev, ui
 }
 
 void plan_reduce(const EthaTable* t, uint32_t first, uint32_t count, uint32_t flags, LaunchList& out) {
+  if (plan_typed(t, first, count, false, flags, out)) flags |= ETHA_LAUNCH_UNORDERED;  // members stored transposed
   const uint32_t w0 = t->row_begin[first], w1 = t->row_begin[first + count];
   if (w1 == w0) return;
   PreparedLaunch p = new_launch(kKernelReduce, false, flags, (w1 - w0) * kBlocksPerTile, 1, kBlockThreads, 0);
@@ -2123,11 +2483,12 @@ void plan_segments(const EthaSegment* segs, uint32_t n_segments, uint32_t flags,
       continue;
     }
     const bool rev = g.kind == ETHA_SEG_UNPACK;
-    const uint32_t x0 = t->trans_begin[g.first], n_trans = t->trans_begin[g.first + g.count] - x0;
+    const uint32_t x0 = t->trans_begin[g.first], n_trans = plain_trans_tiles(t, g.first, g.count);
     if (n_trans) {
       (rev ? trans_reverse : trans_forward).push_back(TransSeg{t->d_trans + x0, n_trans, 0});
       if (t->trans_lds > trans_lds) trans_lds = t->trans_lds;
     }
+    if (plan_typed(t, g.first, g.count, rev, flags, out)) flags |= ETHA_LAUNCH_UNORDERED;
     const Seg2D r = tile_range(t, g.first, g.count, rev);
     if (r.n_tiles) (rev ? reverse : forward).push_back(r);
     const Seg2D gr = gather_range(t, g.first, g.count, rev);
@@ -2678,12 +3039,19 @@ int etha_copy_regions_noalloc(const EthaChunkDesc* src, const EthaChunkDesc* dst
     HIP_TRY(hipEventRecord(st.copied, (hipStream_t)stream));
     st.copy_pending = true;
     uint32_t lds = 0;
-    for (const TransTile& tt : bld.trans)
-      if (trans_lds_bytes(1u << tt.es_log2) > lds) lds = trans_lds_bytes(1u << tt.es_log2);
-    PreparedLaunch launches[2];
+    bool typed_tiles = false, plain_tiles = false;
+    for (const TransTile& tt : bld.trans) {
+      if (trans_tile_lds(tt) > lds) lds = trans_tile_lds(tt);
+      ((tt.cvt & kTransTyped) ? typed_tiles : plain_tiles) = true;
+    }
+    PreparedLaunch launches[3];
     size_t n_launches = 0;
-    if (!bld.trans.empty()) {
+    if (plain_tiles) {
       launches[n_launches] = new_launch(kKernelTrans, false, 0, (uint32_t)bld.trans.size(), 1, kTransThreads, lds);
+      launches[n_launches++].u.trans.tiles = (const TransTile*)(base + trans_off);
+    }
+    if (typed_tiles) {  // both kernels walk the whole list; each leaves the other's blocks alone
+      launches[n_launches] = new_launch(kKernelTransTyped, false, 0, (uint32_t)bld.trans.size(), 1, kTransThreads, lds);
       launches[n_launches++].u.trans.tiles = (const TransTile*)(base + trans_off);
     }
     const uint32_t n_run = (uint32_t)bld.run.size(), n_row = (uint32_t)bld.row.size();

@@ -84,6 +84,19 @@ def scatter_32_byte_pieces(piece_bytes: int = 32, total_bytes: int = 1 << 29, dt
     return [TensorSpec("t", (rows, cols), src, (Replicate(), Shard(1)), tgt, (Replicate(),), dtype, seed=1)], [4], 64 * MIB
 
 
+def scatter_96_byte_pieces():
+    return scatter_32_byte_pieces(piece_bytes=96)
+
+
+def scatter_480_byte_pieces():
+    return scatter_32_byte_pieces(piece_bytes=480)
+
+
+def scatter_2048_byte_pieces():
+    """Whole 128-byte lines per piece: the same scatter without partial lines, for comparison."""
+    return scatter_32_byte_pieces(piece_bytes=2048)
+
+
 def partial4_to_shard2(n_tensors: int = 16, n: int = 8192, dtype=torch.bfloat16):
     """16 bf16 [8192,8192], mesh (4,) Partial(sum) -> mesh (2,) Shard(0); one target rank.
     Partial of source rank r of tensor i: normal(0, 0.02) with seed 4*i + r."""
@@ -93,6 +106,16 @@ def partial4_to_shard2(n_tensors: int = 16, n: int = 8192, dtype=torch.bfloat16)
         for i in range(n_tensors)
     ]
     return specs, [4], 64 * MIB
+
+
+def partial4_transposed_to_shard2(n_tensors: int = 16, n: int = 8192, dtype=torch.bfloat16):
+    """``partial4_to_shard2`` with every member's partial stored as a ``.t()`` view (kept [in, out], handed over as
+    [out, in]): the Partial collapse runs in the typed transposing kernel, which combines the four members' blocks
+    in registers before they are parked in LDS."""
+    specs, targets, bucket = partial4_to_shard2(n_tensors, n, dtype)
+    for s in specs:
+        s.source_layout = "transposed"
+    return specs, targets, bucket
 
 
 def moe_experts_and_uneven_vocab(n_experts: int = 8, hidden: int = 4096, inter: int = 14336, vocab: int = 151936,
@@ -136,6 +159,11 @@ def transposed_parents(n_tensors: int = 16, n: int = 8192, dtype=torch.bfloat16,
     return specs, [4], 64 * MIB
 
 
+def transposed_parents_4096():
+    """The same layout with 4096 x 4096 weights (64 tensors, same bytes): bucket rows at an 8 KiB pitch."""
+    return transposed_parents(n_tensors=64, n=4096)
+
+
 def transposed_parents_fp32_to_bf16():
     """The same with fp32 ``.t()`` sources and bf16 targets (master weights kept [in, out] -> serving weights): the
     transposing pack converts."""
@@ -154,9 +182,14 @@ WORKLOADS = {
     "llama3_8b_fsdp8_to_tp2_fp32_to_bf16": llama3_8b_fsdp8_to_tp2_fp32_to_bf16,
     "many_small_2d_to_replicate": many_small_2d_to_replicate,
     "partial4_to_shard2": partial4_to_shard2,
+    "partial4_transposed_to_shard2": partial4_transposed_to_shard2,
     "scatter_32_byte_pieces": scatter_32_byte_pieces,
+    "scatter_96_byte_pieces": scatter_96_byte_pieces,
+    "scatter_480_byte_pieces": scatter_480_byte_pieces,
+    "scatter_2048_byte_pieces": scatter_2048_byte_pieces,
     "moe_experts_and_uneven_vocab": moe_experts_and_uneven_vocab,
     "moe_experts_row_parallel_w2": moe_experts_row_parallel_w2,
     "transposed_parents": transposed_parents,
+    "transposed_parents_4096": transposed_parents_4096,
     "transposed_parents_fp32_to_bf16": transposed_parents_fp32_to_bf16,
 }

@@ -78,11 +78,39 @@ def clone_specs(specs):
     return [copy.copy(s) for s in specs]
 
 
+def next_values(gpu_job: ReshardJob, cpu_job: ReshardJob, k: int) -> None:
+    """New source values on both jobs (a transfer that moved stale bytes would show); targets are poisoned."""
+    targets = [x for d in gpu_job.target_locals for x in d.values()]
+    for g_src, c_src in zip(gpu_job.source_locals, cpu_job.source_locals):
+        for r, t in g_src.items():
+            if any(t is x for x in targets) or t.numel() == 0:
+                continue
+            if t.dtype in (torch.float8_e4m3fn, torch.float8_e5m2):
+                t.copy_((t.float() * -0.5).to(t.dtype))
+            elif t.dtype.is_floating_point:
+                t.copy_((t.double() * -0.75 + 0.125 * k).to(t.dtype))
+            elif t.dtype == torch.bool:
+                t.copy_(~t)
+            else:
+                t.copy_(t.flip(-1) if t.dim() else t)
+            c_src[r].copy_(t.cpu())
+    sources = [x for d in gpu_job.source_locals for x in d.values()]
+    for job in (gpu_job, cpu_job):
+        srcs = [x for d in job.source_locals for x in d.values()]
+        for d in job.target_locals:
+            for t in d.values():
+                if not any(t is x for x in srcs) and t.numel():
+                    t.copy_(torch.ones_like(t))
+    del sources
+
+
 def gpu_vs_oracle(specs, device, bucket_size, target_ranks=None, merge_launches=False, check_closed_form=True,
-                  pool="ring", max_in_flight=2):
-    """Run the same job on the GPU (HIP path) and on the CPU (oracle); compare every target shard."""
+                  pool="ring", max_in_flight=2, repeat=0, replay=True):
+    """Run the same job on the GPU (HIP path) and on the CPU (oracle); compare every target shard.  ``repeat`` more
+    transfers follow on new source values (with ``replay`` they are served from the wire's recording of the first)."""
     gpu_job = ReshardJob(clone_specs(specs), device=device, bucket_size=bucket_size, target_ranks=target_ranks,
                          keep_globals=True, fill=cpu_fill, pool=pool, max_in_flight=max_in_flight)
+    gpu_job.wire.replay_schedules = replay
     cpu_job = ReshardJob(clone_specs(specs), device="cpu", bucket_size=bucket_size, target_ranks=target_ranks,
                          keep_globals=True, fill=cpu_fill)
     mirror_partials(gpu_job, cpu_job)
@@ -98,6 +126,16 @@ def gpu_vs_oracle(specs, device, bucket_size, target_ranks=None, merge_launches=
             same_obj = any(t is x for x in gpu_job.target_locals[i].values())
             if not same_obj:
                 assert_bit_equal(t, src_before[i][r], f"{spec.name} source rank {r} mutated")
+    for k in range(repeat):
+        next_values(gpu_job, cpu_job, k + 1)
+        before = gpu_job.wire.replays
+        gpu_job.run(merge_launches=merge_launches)
+        run_oracle(cpu_job)
+        for i, spec in enumerate(specs):
+            for r, t in gpu_job.target_locals[i].items():
+                assert_bit_equal(t, cpu_job.target_locals[i][r], f"transfer {k + 2}: {spec.name} target rank {r} vs oracle")
+        if pool == "ring":
+            assert (gpu_job.wire.replays > before) == bool(replay), "served from the recording exactly when that is switched on"
     return gpu_job, cpu_job
 
 

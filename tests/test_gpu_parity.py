@@ -10,12 +10,12 @@ import pytest
 import torch
 from torch.distributed.tensor.placement_types import Partial, Replicate, Shard
 
-from etha_amd import workloads
+from etha_amd import _native, workloads
 from etha_amd.comm import Chunk, LoopbackWire, Transport, bucket_comm, chunk_to_bucket_ops
 from etha_amd.world import ReshardJob, TensorSpec
 
 from helpers import (DTYPES, assert_bit_equal, bits, clone_specs, cpu_fill, expected_target, gpu_vs_oracle, load_cases, mesh_of,
-                     mirror_partials, parse_placements, run_oracle)
+                     mirror_partials, next_values, parse_placements, run_oracle)
 
 pytestmark = pytest.mark.gpu
 CASES = load_cases()
@@ -336,6 +336,30 @@ def test_recv_before_send_is_an_error(gpu_device):
 
 # ---- scaled-down versions of the headline configs, against the oracle ---------------------------------
 
+@pytest.mark.parametrize("replay", [True, False], ids=["recorded", "pipelines"])
+@pytest.mark.parametrize("workload", ["llama", "short_rows", "partial", "moe_self_copy", "transposed", "fp32_to_bf16"])
+def test_repeated_transfers_with_and_without_the_recording(gpu_device, workload, replay):
+    """Three transfers of one registration on new values each time, scaled-down forms of the configurations: with the
+    wire's recording of the first transfer switched on (the second and third are re-issued by etha_schedule_launch)
+    and off (the pipelines are stepped every time), against the oracle every time."""
+    if workload == "llama":
+        specs, targets, _ = workloads.llama3_8b_fsdp8_to_tp2(n_layers=2, hidden=256, inter=896, kv=64, vocab=2056)
+    elif workload == "fp32_to_bf16":
+        specs, targets, _ = workloads.llama3_8b_fsdp8_to_tp2(n_layers=2, hidden=256, inter=896, kv=64, vocab=2056,
+                                                             dtype=torch.float32, target_dtype=torch.bfloat16)
+    elif workload == "short_rows":
+        specs, targets, _ = workloads.many_small_2d_to_replicate(n_tensors=12, rows=64)
+    elif workload == "partial":
+        specs, targets, _ = workloads.partial4_to_shard2(n_tensors=3, n=256)
+    elif workload == "moe_self_copy":
+        specs, targets, _ = workloads.moe_experts_and_uneven_vocab(n_experts=8, hidden=64, inter=224, vocab=1030)
+    else:
+        specs, targets, _ = workloads.transposed_parents(n_tensors=3, n=520)
+    for s in specs:
+        s.std = 1.0
+    gpu_vs_oracle(specs, gpu_device, 64 * 1024, target_ranks=targets, merge_launches=True, repeat=2, replay=replay)
+
+
 @pytest.mark.parametrize("pool", ["ring", "resident"])
 @pytest.mark.parametrize("merge", [False, True])
 def test_llama_like_fsdp_to_tp_small(gpu_device, merge, pool):
@@ -566,6 +590,142 @@ def test_transposed_f32_parents_convert_in_the_transposing_kernel(gpu_device, na
     wide = (tiles["nj"] == 128) & (tiles["nk"] == 256)
     full = (tiles["nj"] == 128) & (tiles["nk"] == 128)
     assert np.all(tiles["cvt"] != 0) and wide.any() and full.any() and (~wide & ~full).any()
+
+
+_TYPED_PAIRS = [
+    # (source dtype, target dtype, which side is the .t() view)
+    (torch.float64, torch.float32, "source"), (torch.float64, torch.bfloat16, "source"), (torch.float32, torch.int8, "source"),
+    (torch.int32, torch.int16, "source"), (torch.float32, torch.float8_e4m3fn, "source"), (torch.int64, torch.float32, "source"),
+    (torch.float16, torch.bfloat16, "target"), (torch.bfloat16, torch.float64, "target"), (torch.int8, torch.int32, "target"),
+    (torch.float32, torch.float64, "target"), (torch.bool, torch.float16, "target"), (torch.uint8, torch.int64, "target"),
+]
+
+
+@pytest.mark.parametrize("src_dt,tgt_dt,side", _TYPED_PAIRS,
+                         ids=lambda v: str(v).replace("torch.", "") if not isinstance(v, str) else v)
+def test_transposed_parents_of_any_value_type_convert_in_lds_blocks(gpu_device, src_dt, tgt_dt, side):
+    """``.t()`` shards whose element type differs from the wire's, beyond f32 <-> 16-bit: the typed transposing kernel
+    converts every element while the block is parked in LDS (full blocks of 128 x 128, or 64 x 64 with an 8-byte
+    side, and edge blocks), against the oracle's restatement of the reference path."""
+    src, tgt = mesh_of(0, [4]), mesh_of(4, [2])
+    specs = [TensorSpec(f"w{i}", (904, 652), src, (Shard(0),), tgt, (Shard(0),), src_dt, tgt_dt, seed=i, std=1.0,
+                        source_layout="transposed" if side == "source" else "contiguous",
+                        target_layout="transposed" if side == "target" else "contiguous") for i in range(2)]
+    job, _ = gpu_vs_oracle(specs, gpu_device, 256 * 1024, target_ranks=[4], check_closed_form=False)
+    if side == "source":
+        tables = [job.wire.plan(b).send_table for b in job.send_buckets.values()]
+    else:
+        tables = [job.wire.plan(job.recv_buckets[4]).recv_table]
+    dim = 64 if 8 in (src_dt.itemsize, tgt_dt.itemsize) else 128
+    for table in tables:
+        info, tiles = table.info(), table.trans_tiles()
+        assert info.n_trans_tiles > 0 and info.n_row_tiles == 0 and info.n_run_tiles == 0
+        assert np.all(tiles["cvt"] & _native.TRANS_TYPED) and np.all(tiles["n_peers"] == 0)
+        full = (tiles["nj"] == dim) & (tiles["nk"] == dim)
+        assert full.any() and (~full).any() and tiles["nj"].max() <= dim and tiles["nk"].max() <= dim
+
+
+def test_direct_wire_converts_transposed_sources_in_lds_blocks(gpu_device):
+    """The direct wire writes the target straight from a ``.t()`` source of another type (bf16 -> f32: the narrow side
+    is the tensor, which no bucket table ever sees): typed blocks in the region-to-region table."""
+    src, tgt = mesh_of(0, [4]), mesh_of(4, [2])
+    specs = [TensorSpec("w", (776, 520), src, (Shard(0),), tgt, (Shard(0),), torch.bfloat16, torch.float32, seed=3, std=1.0,
+                        source_layout="transposed")]
+    jobs = []
+    for direct in (True, False):
+        job = ReshardJob(clone_specs(specs), device=gpu_device, bucket_size=256 * 1024, target_ranks=[4], fill=cpu_fill, direct=direct)
+        job.run()
+        jobs.append(job)
+    assert_bit_equal(jobs[0].target_locals[0][4], jobs[1].target_locals[0][4], "direct wire vs buckets")
+    tiles = jobs[0].wire.plan(jobs[0].recv_buckets[4]).local_table.trans_tiles()
+    assert len(tiles) and np.all(tiles["cvt"] & _native.TRANS_TYPED)
+
+
+@pytest.mark.parametrize("dtype,wire", [(torch.bfloat16, None), (torch.float32, torch.bfloat16), (torch.float16, None),
+                                        (torch.float64, torch.float32)],
+                         ids=["bf16", "f32_to_bf16", "f16", "f64_to_f32"])
+@pytest.mark.parametrize("op", ["sum", "avg", "max"])
+def test_partial_members_stored_transposed_are_reduced_in_lds_blocks(gpu_device, dtype, wire, op):
+    """A Partial source whose members are ``.t()`` views: the typed transposing kernel combines the members' blocks in
+    registers (fp32, list order; f64 for f64 members), rounds once and writes the bucket through LDS - full and
+    edge blocks, against the oracle (bit for bit: the oracle's reduce is the same rank-order sum)."""
+    src, tgt = mesh_of(0, [4]), mesh_of(4, [2])
+    specs = [TensorSpec(f"p{i}", (1320, 776), src, (Partial(op),), tgt, (Shard(0),), dtype, wire, seed=10 * i, std=1.0,
+                        source_layout="transposed") for i in range(2)]
+    job, _ = gpu_vs_oracle(specs, gpu_device, 256 * 1024, target_ranks=[4])
+    seen = 0
+    for b in job.send_buckets.values():
+        table = job.wire.plan(b).send_table
+        if table is None or not table.info().n_chunks:
+            continue
+        tiles = table.trans_tiles()
+        if len(tiles):
+            assert table.info().n_row_tiles == 0
+            assert np.all(tiles["n_peers"] == 4) and np.all(tiles["cvt"] & _native.TRANS_TYPED)
+            dim = 64 if dtype == torch.float64 else 128
+            full = (tiles["nj"] == dim) & (tiles["nk"] == dim)
+            assert full.any() and (~full).any() and tiles["nj"].max() <= dim and tiles["nk"].max() <= dim
+            seen += 1
+    assert seen > 0
+
+
+def test_partial_transposed_full_size_properties(gpu_device):
+    """16 bf16 [8192, 8192] Partial tensors whose four members are ``.t()`` views: the target shard equals the fp32
+    rank-order sum of the members, recomputed with torch device ops, rounded once (0 ulp); members unchanged."""
+    specs, targets, bucket = workloads.partial4_transposed_to_shard2()
+    job = ReshardJob(specs, device=gpu_device, bucket_size=bucket, target_ranks=targets)
+    sums = [{r: t.view(torch.int16).sum(dtype=torch.int64).item() for r, t in d.items()} for d in job.source_locals[:2]]
+    job.run(merge_launches=True)
+    for i in range(len(specs)):
+        acc = job.source_locals[i][0].float()
+        for r in (1, 2, 3):
+            acc = acc + job.source_locals[i][r].float()
+        want = acc.to(torch.bfloat16)[:4096]
+        assert torch.equal(job.target_locals[i][4].view(torch.int16), want.contiguous().view(torch.int16)), f"tensor {i}"
+    for i, d in enumerate(job.source_locals[:2]):
+        for r, t in d.items():
+            assert not t.is_contiguous() and t.view(torch.int16).sum(dtype=torch.int64).item() == sums[i][r], "member mutated"
+    info = job.wire.plan(job.send_buckets[0]).send_table.info()
+    assert info.n_trans_tiles > 0 and info.n_row_tiles == 0
+
+
+@pytest.mark.parametrize("src_dt,tgt_dt", [(torch.float32, torch.bfloat16), (torch.bfloat16, torch.float32),
+                                           (torch.float16, torch.float64), (torch.float64, torch.float16),
+                                           (torch.float16, torch.bfloat16)],
+                         ids=lambda d: str(d).replace("torch.", ""))
+def test_short_and_ragged_converting_rows_use_narrow_vectors(gpu_device, src_dt, tgt_dt):
+    """Converting rows that are not whole vectors: the remainder of a row (and rows shorter than one vector) move in
+    vectors of 4 and 2 elements before single elements are used.  Every row length from 1 to 23 elements, rows at
+    element-aligned pitches, against torch's cast of the same slice."""
+    from etha_amd.comm.device_plan import fill_region
+
+    dev = gpu_device
+    g = torch.Generator(device=dev).manual_seed(3)
+    pairs, keep = [], []
+    for run in range(1, 24):
+        s = (torch.randn(301, run + 3, generator=g, device=dev, dtype=torch.float32) * 50).to(src_dt)
+        d = torch.full((301, run + 5), 7.0, device=dev, dtype=tgt_dt)
+        pairs.append((s, (slice(0, 301), slice(1, 1 + run)), d, (slice(0, 301), slice(2, 2 + run))))
+    src = np.zeros(len(pairs), dtype=_native.CHUNK_DESC)
+    dst = np.zeros(len(pairs), dtype=_native.CHUNK_DESC)
+    for i, (s, ss, d, ds) in enumerate(pairs):
+        a, b = np.zeros((), dtype=_native.CHUNK_DESC), np.zeros((), dtype=_native.CHUNK_DESC)
+        fill_region(a, s, ss, tuple(s[ss].shape))
+        fill_region(b, d, ds, tuple(s[ss].shape))
+        a["wire_dtype"], b["wire_dtype"] = a["tensor_dtype"], b["tensor_dtype"]
+        src[i], dst[i] = a, b
+    table = _native.Table.create_selfcopy(src, dst)
+    _, rows = table.tiles()
+    elems = (rows["meta"] >> 22) & 3
+    full = 16 // max(src_dt.itemsize, tgt_dt.itemsize) if min(src_dt.itemsize, tgt_dt.itemsize) * 2 < max(src_dt.itemsize, tgt_dt.itemsize) else None
+    assert set(np.unique(elems)) >= {0, 1}  # single elements and pairs at least; wider ones where the pair allows
+    table.selfcopy(0, len(pairs), torch.cuda.current_stream(dev).cuda_stream)
+    torch.cuda.synchronize()
+    for s, ss, d, ds in pairs:
+        assert torch.equal(bits(d[ds]), bits(s[ss].to(tgt_dt))), f"row length {s[ss].shape[1]}"
+        outside = torch.ones_like(d, dtype=torch.bool)
+        outside[ds] = False
+        assert bool((d[outside] == 7.0).all())
 
 
 def test_transposed_parents_full_size_properties(gpu_device):
@@ -811,11 +971,15 @@ def test_random_batches_gpu(gpu_device, seed):
                          zero_copy=mode == "zero_copy", direct=mode == "direct", pool=pool, max_in_flight=depth)
     cpu_job = ReshardJob(specs, device="cpu", bucket_size=bucket_size, keep_globals=True, fill=cpu_fill, local_view=view)
     mirror_partials(gpu_job, cpu_job)
-    gpu_job.run(merge_launches=merge, fanout=fanout)
-    run_oracle(cpu_job)
-    for i, spec in enumerate(specs):
-        for r, t in gpu_job.target_locals[i].items():
-            assert_bit_equal(t, cpu_job.target_locals[i][r], f"seed {seed} ({mode}, {pool} pool, fanout {fanout}) {spec.name} rank {r}")
+    for transfer in range(2):  # the second transfer, on new values, is served from the wire's recording of the first (ring pool)
+        if transfer:
+            next_values(gpu_job, cpu_job, transfer)
+        gpu_job.run(merge_launches=merge, fanout=fanout)
+        run_oracle(cpu_job)
+        for i, spec in enumerate(specs):
+            for r, t in gpu_job.target_locals[i].items():
+                assert_bit_equal(t, cpu_job.target_locals[i][r],
+                                 f"seed {seed} ({mode}, {pool} pool, fanout {fanout}) transfer {transfer} {spec.name} rank {r}")
 
 
 @pytest.mark.parametrize("dtype", [torch.int8, torch.bfloat16, torch.float32, torch.float64])

@@ -149,7 +149,7 @@ def _execute(table, arena, direction, first, count, peers, ordered) -> None:
     trans_begin = table.trans_ranges()
     trans = table.trans_tiles()[trans_begin[first] : trans_begin[first + count]]
     if len(trans):
-        _transpose_blocks(arena, trans, direction == "unpack")
+        _transpose_blocks(arena, trans, direction == "unpack", peers)
     assert np.all(run_tiles["n"] <= THREADS) and np.all(row_tiles["n"] <= THREADS)
     assert np.all(run_tiles["n"] > 0) and np.all(row_tiles["n"] > 0)
     rev = direction == "unpack"
@@ -171,6 +171,9 @@ def _execute(table, arena, direction, first, count, peers, ordered) -> None:
                 assert generic == (dta > 3 or dtb > 3)
                 if generic:
                     assert (ua, ub) == (_CODE_SIZE[dta], _CODE_SIZE[dtb]) and not vec
+                else:  # the unit's element count is stated in the meta word and agrees with both unit sizes
+                    n_el = 1 << ((int(m) >> 22) & 3)
+                    assert ua == n_el * _CODE_SIZE[dta] and ub == n_el * _CODE_SIZE[dtb], "unit sizes and element count disagree"
             if reduce:
                 _reduce_units(arena, mem, row_tiles, row_idx[sel], a[sel], b[sel], ua, ub, dta, dtb, peers, skew_a)
                 continue
@@ -192,28 +195,56 @@ def _execute(table, arena, direction, first, count, peers, ordered) -> None:
             mem[do] = data
 
 
-def _transpose_blocks(arena, trans, rev: bool) -> None:
+def _transpose_blocks(arena, trans, rev: bool, peers=None) -> None:
     mem = arena.buf[arena.pad : arena.pad + arena.nbytes]
     for t in trans:
         es = 1 << int(t["es_log2"])
         nj, nk = int(t["nj"]), int(t["nk"])
         assert 0 < nj <= 512 and 0 < nk <= 512  # block side: a fixed number of bytes per row
         cvt = int(t["cvt"])
-        dta, dtb = cvt >> 4, cvt & 15
-        if cvt:  # a converting block: f32 on the a side, f16 or bf16 in the bucket; blocks are sized by the b side
-            assert dta == 2 and dtb in (0, 1) and es == 2 and nj <= 128 and nk <= 256
+        typed = bool(cvt & 256)
+        dta, dtb = (cvt >> 4) & 15, cvt & 15
+        n_peers = int(t["n_peers"])
+        if typed:  # a block of the typed kernel: any pair of value types, or a Partial source reduced with one op
+            dim = 64 if 8 in (_CODE_SIZE[dta], _CODE_SIZE[dtb]) else 128
+            assert nj <= dim and nk <= dim and (dta != dtb or n_peers)
+            assert not n_peers or (not rev and dta <= 3 and dtb <= 3 and int(t["reduce_op"]) <= 4)
+        else:
+            assert n_peers == 0
+            if cvt:  # a converting block: f32 on the a side, f16 or bf16 in the bucket; blocks are sized by the b side
+                assert dta == 2 and dtb in (0, 1) and es == 2 and nj <= 128 and nk <= 256
         esa, esb = (_CODE_SIZE[dta], _CODE_SIZE[dtb]) if cvt else (es, es)
         j, k = np.meshgrid(np.arange(nj), np.arange(nk), indexing="ij")
         a = int(t["a"]) + j * esa + k * int(t["a_pitch"])
         b = int(t["b"]) + j * int(t["b_pitch"]) + k * esb
         assert np.all(a % esa == 0) and np.all(b % esb == 0)
         src, dst, ess, esd, ds_, dd = (b, a, esb, esa, dtb, dta) if rev else (a, b, esa, esb, dta, dtb)
-        so = arena.offsets(src.reshape(-1), ess)[:, None] + np.arange(ess)
         do = arena.offsets(dst.reshape(-1), esd)[:, None] + np.arange(esd)
         if arena.writes is not None:
             np.add.at(arena.writes, do.reshape(-1), 1)
-        _note("r", so)
         _note("w", do)
+        if n_peers:  # src holds offsets from each member's base
+            bases = peers[int(t["peer_first"]) : int(t["peer_first"]) + n_peers].astype(np.int64)
+            staged = []
+            for base in bases:
+                assert base % esa == 0, "misaligned member"
+                so = arena.offsets(base + src.reshape(-1), ess)[:, None] + np.arange(ess)
+                _note("r", so)
+                staged.append(np.ascontiguousarray(mem[so]).reshape(-1).copy())
+            via = int(t["via"])
+            out_dt = via - 1 if via else dd
+            n_el = src.size
+            out = np.zeros(n_el, dtype=_CODE_RAW[out_dt])
+            scratch = np.zeros(n_el, dtype=np.float64)
+            op = {0: "sum", 1: "avg", 2: "max", 3: "min", 4: "product"}[int(t["reduce_op"])]
+            ch = co.make_chunk(0, (0,), (n_el,), (1,), ds_, out_dt, peers=[s.ctypes.data for s in staged], op=op)
+            assert co.lib().oracle_reduce(ch, out.ctypes.data, scratch.ctypes.data) == 0
+            if via:
+                out = co.cast(out, out_dt, dd, _CODE_RAW[dd])
+            mem[do] = out.view(np.uint8).reshape(n_el, esd)
+            continue
+        so = arena.offsets(src.reshape(-1), ess)[:, None] + np.arange(ess)
+        _note("r", so)
         data = mem[so]
         if cvt:
             elems = np.ascontiguousarray(data).view(_CODE_RAW[ds_]).reshape(-1)
