@@ -282,7 +282,8 @@ def launches_per_step(job, run):
 
 
 OTHER_WORKLOADS = ("single_fp32_shard0_to_shard1", "many_small_2d_to_replicate", "partial4_to_shard2",
-                   "moe_experts_and_uneven_vocab", "llama3_8b_fsdp8_to_tp2_fp32_to_bf16", "transposed_parents")
+                   "moe_experts_and_uneven_vocab", "llama3_8b_fsdp8_to_tp2_fp32_to_bf16", "transposed_parents",
+                   "partial4_transposed_to_shard2")
 
 
 def measure_workload(name: str, dev, steps: int, warmup: int):
@@ -497,6 +498,7 @@ def main():
             "launches_per_step": n_launch,
         },
         "setup_s": round(setup_s, 1),
+        "library_digest": _native.lib().etha_source_hash().decode(),
     }
 
     def leg(j, reps=None, **kw):

@@ -60,6 +60,22 @@ def reduce_levels(slices: list[torch.Tensor], levels) -> torch.Tensor:
     return values[0]
 
 
+def reduce_levels_in_tensor_dtype(slices: list[torch.Tensor], levels) -> torch.Tensor:
+    """The same nested reduction with the reference's intermediate roundings: each of its all-reduces runs in place on a
+    buffer of the *tensor's* dtype (``ir.py:123-124``), so for f16 / bf16 members the value is rounded to that dtype
+    after every level.  ``reduce_levels`` above - which the kernels follow - keeps the accumulator in fp32 across levels
+    and rounds once: for f32 / f64 members the two are the same function; for 16-bit members they can differ in the
+    last place of a level's result.  Kept to quantify that difference (``tests/test_partial_levels.py``); what an
+    all-reduce does inside one level is the backend's business and is not restated here."""
+    dtype = slices[0].dtype
+    values = list(slices)
+    for op, size in levels:
+        assert len(values) % size == 0
+        values = [reduce_rank_order(values[i:i + size], op).to(dtype) for i in range(0, len(values), size)]
+    assert len(values) == 1
+    return values[0]
+
+
 def _peers(chunk):
     groups = getattr(chunk, "source_partial_groups", None)
     if not groups:

@@ -58,7 +58,8 @@ def test_default_line_carries_every_configuration(gpu_device):
     assert "extra_legs_error" not in d
     wl = d["workloads"]
     assert set(wl) == {"single_fp32_shard0_to_shard1", "many_small_2d_to_replicate", "partial4_to_shard2",
-                       "moe_experts_and_uneven_vocab", "llama3_8b_fsdp8_to_tp2_fp32_to_bf16", "transposed_parents"}
+                       "moe_experts_and_uneven_vocab", "llama3_8b_fsdp8_to_tp2_fp32_to_bf16", "transposed_parents",
+                       "partial4_transposed_to_shard2"}
     for name, w in wl.items():
         assert "error" not in w, (name, w)
         assert w["steps"] >= 20 and w["warmup"] >= 3

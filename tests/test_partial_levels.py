@@ -156,3 +156,33 @@ def test_partial_source_delivered_to_its_own_rank_on_the_gpu(gpu_device, ops):
     kinds = {s[0] for b in job.send_buckets.values() for s in job.wire.plan(b).steps}
     assert "selfcopy_reduce" in kinds
     gpu_vs_oracle(specs, gpu_device, 2048, check_closed_form=False, merge_launches=True, pool="resident")
+
+
+def test_rounding_between_levels_is_the_only_difference_from_the_reference():
+    """The reference all-reduces a buffer of the tensor's dtype once per Partial mesh dim (ir.py:123-124): 16-bit
+    members are rounded after every level.  The kernels keep fp32 across levels and round once.  For f32 members the
+    two forms are the same function; for bf16 members they agree wherever no intermediate rounding happens (small
+    integers, max/min levels) and otherwise stay within one rounding step of the inner level's result."""
+    from oracle.reference_path import reduce_levels, reduce_levels_in_tensor_dtype
+
+    g = torch.Generator().manual_seed(4)
+    levels = (("sum", 2), ("max", 3))
+    f32 = [torch.randn(257, generator=g) for _ in range(6)]
+    assert torch.equal(reduce_levels(f32, levels), reduce_levels_in_tensor_dtype(f32, levels))
+    small = [torch.randint(-8, 9, (257,), generator=g).to(torch.bfloat16) for _ in range(6)]
+    assert torch.equal(reduce_levels(small, levels).to(torch.bfloat16), reduce_levels_in_tensor_dtype(small, levels))
+    only_order = (("max", 2), ("min", 3))  # no arithmetic: nothing to round
+    bf = [torch.randn(257, generator=g).to(torch.bfloat16) for _ in range(6)]
+    assert torch.equal(reduce_levels(bf, only_order).to(torch.bfloat16), reduce_levels_in_tensor_dtype(bf, only_order))
+    # sums of random bf16 values, then a second sum: the inner sums are rounded (reference) or not (kernels)
+    two_sums = (("sum", 2), ("avg", 3))
+    once = reduce_levels(bf, two_sums).to(torch.bfloat16).float()
+    each = reduce_levels_in_tensor_dtype(bf, two_sums).float()
+    inner = torch.stack([b.double() for b in bf]).reshape(3, 2, -1).sum(1)
+    exact = inner.mean(0)
+    eps = torch.finfo(torch.bfloat16).eps
+    # each inner sum is off by at most half a step of its own magnitude, the results by one step of theirs
+    bound = eps * (inner.abs().max(0).values + exact.abs()).float()
+    assert bool(((once - each).abs() <= bound).all())  # they differ, by roundings only ...
+    assert not torch.equal(once, each)
+    assert float((once.double() - exact).abs().mean()) <= float((each.double() - exact).abs().mean())  # ... and once is no worse
