@@ -1216,7 +1216,9 @@ __device__ __forceinline__ void typed_values(uint32_t sd, uint32_t dd, uint64_t 
 // Full block of a Partial source whose members hold f16, bf16 or f32: the loads of up to four members are in flight
 // together (a member's vectors only meet the accumulators once all of the batch have been requested), members are
 // still combined strictly in list order, and all conversions are straight-line code.
-template <typename S, typename D, uint32_t DX, uint32_t DY>
+// SUM: true when the op is a sum or an average - the usual case, for which the combine step is straight-line code;
+// with a run-time op every element of the unrolled loops would go through the op's switch.
+template <typename S, typename D, uint32_t DX, uint32_t DY, bool SUM>
 __device__ __forceinline__ void reduce_block_full(const TransTile& t, const uint64_t* __restrict__ peers, uint8_t* __restrict__ lds) {
   typedef typename S::bits ES;
   typedef typename D::bits ED;
@@ -1241,15 +1243,21 @@ __device__ __forceinline__ void reduce_block_full(const TransTile& t, const uint
 #pragma unroll
         for (uint32_t i = 0; i < kPer; i++) raw[j][i].load(base + off[i]);
       }
+    if (p == 0) {  // the first member starts the accumulators
+#pragma unroll
+      for (uint32_t i = 0; i < kPer; i++)
+#pragma unroll
+        for (uint32_t e = 0; e < kVs; e++) acc[i][e] = to_f32(S(), raw[0][i].get(e));
+    }
 #pragma unroll
     for (uint32_t j = 0; j < kBatch; j++)
-      if (p + j < np) {
+      if (p + j < np && (j || p)) {
 #pragma unroll
         for (uint32_t i = 0; i < kPer; i++)
 #pragma unroll
           for (uint32_t e = 0; e < kVs; e++) {
             const float v = to_f32(S(), raw[j][i].get(e));
-            acc[i][e] = (p + j == 0) ? v : combine(op, acc[i][e], v);
+            acc[i][e] = SUM ? acc[i][e] + v : combine(op, acc[i][e], v);
           }
       }
   }
@@ -1262,28 +1270,36 @@ __device__ __forceinline__ void reduce_block_full(const TransTile& t, const uint
     for (uint32_t e = 0; e < kVs; e++) {
       float r = acc[i][e];
       if (op == ETHA_AVG) r = r / cnt;
-      row[e] = from_f32(D(), round_via(via, r));
+      row[e] = from_f32(D(), via ? round_via(via, r) : r);
     }
   }
   __syncthreads();
   TransBlock<ED, DX, DY>::emit(lds, t.b, t.b_pitch);
 }
 
+template <typename S, typename D, uint32_t DX, uint32_t DY>
+__device__ __forceinline__ void reduce_block_any_op(const TransTile& t, const uint64_t* __restrict__ peers, uint8_t* __restrict__ lds) {
+  if (t.reduce_op == ETHA_SUM || t.reduce_op == ETHA_AVG)
+    reduce_block_full<S, D, DX, DY, true>(t, peers, lds);
+  else
+    reduce_block_full<S, D, DX, DY, false>(t, peers, lds);
+}
+
 template <typename S, typename ED, uint32_t DX, uint32_t DY>
 __device__ __forceinline__ bool reduce_block_to(uint32_t dd, const TransTile& t, const uint64_t* __restrict__ peers, uint8_t* __restrict__ lds) {
   if constexpr (sizeof(ED) == 2) {
     if (dd == ETHA_F16) {
-      reduce_block_full<S, TagF16, DX, DY>(t, peers, lds);
+      reduce_block_any_op<S, TagF16, DX, DY>(t, peers, lds);
       return true;
     }
     if (dd == ETHA_BF16) {
-      reduce_block_full<S, TagBF16, DX, DY>(t, peers, lds);
+      reduce_block_any_op<S, TagBF16, DX, DY>(t, peers, lds);
       return true;
     }
   }
   if constexpr (sizeof(ED) == 4) {
     if (dd == ETHA_F32) {
-      reduce_block_full<S, TagF32, DX, DY>(t, peers, lds);
+      reduce_block_any_op<S, TagF32, DX, DY>(t, peers, lds);
       return true;
     }
   }
