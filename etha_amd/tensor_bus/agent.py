@@ -75,6 +75,7 @@ class BatchState:
     send_buckets: dict = field(default_factory=dict)
     recv_buckets: dict = field(default_factory=dict)
     send_count: dict = field(default_factory=dict)
+    siblings: dict = field(default_factory=dict)  # (kind, rank) -> (senders, receivers) of that rank's transfer
     recv_count: dict = field(default_factory=dict)
     owed: dict = field(default_factory=dict)  # destination rank -> number of receives its sources have asked of it
     send_arrived: dict = field(default_factory=dict)  # rank -> number of send commands it has issued so far
@@ -129,6 +130,9 @@ class TensorBusAgent:
         self._unsynced: list[tuple[dict, float, str]] = []  # (result, start time, label) of transfers enqueued, not yet synchronised
         self._queued = False  # pipelines were queued on the wire in this pass and have not been stepped yet
         self.stats = {"ipc_tensors": 0, "in_process_tensors": 0, "transfers": 0}
+        # host time of the passes that launched transfers, in ms: waiting for the other ranks' commands, walking the
+        # commands and issuing launches, waiting for the device, publishing state and replying
+        self.timing = {"passes": 0, "gather_ms": 0.0, "issue_ms": 0.0, "device_ms": 0.0, "reply_ms": 0.0}
         for rank in range(world_size):
             cmd_path, state_path = self.path_naming_fn(rank)
             self._queues[rank] = CommandQueue(cmd_path, serve=True)
@@ -196,13 +200,17 @@ class TensorBusAgent:
                 self._pending.append(self._inbox.get_nowait())
             except queue.Empty:
                 break
-        deadline = time.perf_counter() + self.gather_window
+        # ranks of one batch issue their commands from threads that take turns: wait while commands keep coming
+        # (the window restarts at every arrival), but never longer than eight windows in all
+        start = time.perf_counter()
+        deadline, limit = start + self.gather_window, start + 8 * self.gather_window
         while self._siblings_missing():
-            left = deadline - time.perf_counter()
+            left = min(deadline, limit) - time.perf_counter()
             if left <= 0:
                 break
             try:
                 self._pending.append(self._inbox.get(timeout=left))
+                deadline = time.perf_counter() + self.gather_window
             except queue.Empty:
                 break
         # Sweep until nothing moves.  Commands that complete are answered only after the sweep: the device
@@ -210,6 +218,7 @@ class TensorBusAgent:
         # and the state files are written once, instead of once per rank.
         finished: list[tuple[_Entry, tuple]] = []
         progressed = True
+        t_gathered = time.perf_counter()
         while progressed:
             progressed, self._moved = False, False
             for entry in self._in_rank_order(self._pending):
@@ -232,6 +241,8 @@ class TensorBusAgent:
             # a command that changed shared state without completing (a send that lends its tensors and now
             # waits for its receivers) may have unblocked commands examined earlier in this pass
             progressed = progressed or self._moved
+        timed = bool(self._unsynced)
+        t_issued = time.perf_counter()
         if self._unsynced:
             # a worker may overwrite its tensors as soon as its send returns, and read them as soon as its
             # recv returns: both replies wait for the device
@@ -247,6 +258,13 @@ class TensorBusAgent:
             self._write_state(force=True)
             for entry, message in finished:
                 self._reply(entry, message)
+        if timed:
+            t_end = time.perf_counter()
+            self.timing["passes"] += 1
+            self.timing["gather_ms"] += (t_gathered - start) * 1e3
+            self.timing["issue_ms"] += (t_issued - t_gathered) * 1e3
+            self.timing["device_ms"] += (now - t_issued) * 1e3
+            self.timing["reply_ms"] += (t_end - now) * 1e3
 
     @staticmethod
     def _in_rank_order(pending: list) -> list:
@@ -256,22 +274,46 @@ class TensorBusAgent:
                            key=lambda e: (e.command.batch_id, e.command.transfer_type != "send", e.rank))
         return [e for e in pending if not isinstance(e.command, Transfer)] + transfers
 
+    def _ranks_of_transfer(self, batch: BatchState, kind: str, rank: int) -> tuple[frozenset, frozenset]:
+        """(senders, receivers) of the transfer that ``rank``'s command of ``kind`` belongs to: the ranks its buckets
+        go to or come from, their other sources, the members of Partial sources, and so on until nothing is added.
+        A batch plans both directions of its pairs; the opposite direction is a different transfer."""
+        key = (kind, rank)
+        if key not in batch.siblings:
+            senders, receivers = ({rank}, set()) if kind == "send" else (set(), {rank})
+            grown = True
+            while grown:
+                before = len(senders) + len(receivers)
+                for s in list(senders):
+                    receivers |= self._peers(batch.send_buckets.get(s) or (), "dst")
+                    senders |= self._partial_members(batch, s)
+                for d in list(receivers):
+                    senders |= self._peers(batch.recv_buckets.get(d) or (), "src")
+                grown = len(senders) + len(receivers) != before
+            batch.siblings[key] = (frozenset(senders), frozenset(receivers))
+        return batch.siblings[key]
+
     def _siblings_missing(self) -> bool:
-        """True while some rank of a batch has issued a transfer command that is not under way yet and another rank
-        with buckets in the same direction has not issued its command of that generation."""
+        """True while some rank has issued a transfer command that is not under way yet and another rank of the same
+        transfer has not issued its command of that generation (a rank that both sends and receives counts as
+        present with either command: it issues them one after the other)."""
         waiting: dict = {}
         for e in self._pending:
             if isinstance(e.command, Transfer) and not e.started:
-                waiting.setdefault((e.command.batch_id, e.command.transfer_type), set()).add(e.rank)
-        for (batch_id, kind), ranks in waiting.items():
+                waiting.setdefault(e.command.batch_id, []).append((e.command.transfer_type, e.rank))
+        for batch_id, entries in waiting.items():
             batch = self.batches.get(batch_id)
             if batch is None:
                 continue
-            table = batch.send_buckets if kind == "send" else batch.recv_buckets
-            counts = batch.send_count if kind == "send" else batch.recv_count
-            gen = min((counts.get(r, 0) for r in ranks), default=0)
-            for r, buckets in table.items():
-                if buckets and r not in ranks and counts.get(r, 0) <= gen:
+            present = {r for _, r in entries}
+            for kind, rank in entries:
+                if rank not in batch.planned_ranks:
+                    continue
+                gen = (batch.send_count if kind == "send" else batch.recv_count).get(rank, 0)
+                senders, receivers = self._ranks_of_transfer(batch, kind, rank)
+                if any(r not in present and batch.send_count.get(r, 0) <= gen for r in senders):
+                    return True
+                if any(r not in present and batch.recv_count.get(r, 0) <= gen for r in receivers):
                     return True
         return False
 
@@ -413,6 +455,7 @@ class TensorBusAgent:
             if all(self._pair_complete(batch, p) for p in mine):
                 self._plan_rank(batch, rank, mine)
                 batch.planned_ranks.add(rank)
+                batch.siblings.clear()
         # tile programs: a receive list pairs with send lists, so it is compiled once all its sources' lists are
         for rank in sorted(batch.planned_ranks - batch.send_compiled):
             self._plan_if_device(batch.send_buckets.get(rank), batch.batch_id)
@@ -567,6 +610,7 @@ class TensorBusAgent:
                 except Exception:
                     logger.exception("closing an IPC mapping failed")
         batch.planned_ranks.discard(rank)
+        batch.siblings.clear()
 
     def _release_batch(self, batch: BatchState) -> None:
         # receivers first: their plans only reference slots, the senders' plans own them

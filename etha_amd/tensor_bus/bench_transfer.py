@@ -182,7 +182,8 @@ def main() -> None:
         for p in procs:
             if p.is_alive():
                 p.kill()
-        agent_stats = dict(agent.stats, drives_served_from_a_recording=agent.wire.replays)
+        agent_stats = dict(agent.stats, drives_served_from_a_recording=agent.wire.replays,
+                           host_ms_of_transfer_passes={k: round(v, 3) for k, v in agent.timing.items()})
         agent.close()
     # checksum of checksums: a same-dtype tensor's bits, summed over all target ranks, equal the sum over all
     # source ranks times the number of copies the target layout holds of each element (per copy the source holds)
@@ -202,18 +203,22 @@ def main() -> None:
             raise RuntimeError(f"{s.name}: checksum over the target ranks differs from the source ranks' ({got} vs {want})")
         verified += 1
     send, recv = results["trainer"]["stamps"], results["inference"]["stamps"]
-    lat = []
+    lat, spread = [], []
     for k in range(args.warmup, args.warmup + args.steps):
         start = min(v[k][0] for v in send.values())
         end = max(v[k][1] for v in recv.values())
         lat.append(end - start)
+        # from the first rank's command to the last rank's, either direction
+        spread.append(max(v[k][0] for side in (send, recv) for v in side.values()) - start)
     lat.sort()
+    spread.sort()
     med = lat[len(lat) // 2]
     payload = results["inference"]["bytes"]
     print(json.dumps({
         "metric": "end-to-end handler.transfer through the tensor bus, three processes on one GPU",
         "value": payload / med / 1e9, "unit": "GB/s", "ms_per_transfer": med * 1e3, "min_ms": lat[0] * 1e3,
         "steps": args.steps, "warmup": args.warmup, "payload_bytes": payload,
+        "ms_between_first_and_last_rank_command": spread[len(spread) // 2] * 1e3,
         "config": {"workload": args.workload, "source_ranks": len(results["trainer"]["ranks"]),
                    "target_ranks": len(results["inference"]["ranks"]), "zero_copy_single_chunk": args.zero_copy,
                    "direct_same_device": args.direct},

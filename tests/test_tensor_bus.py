@@ -92,6 +92,56 @@ def test_init_pair_register_and_errors_on_cpu(agent_factory):
         c.close()
 
 
+def test_the_agent_waits_for_the_ranks_of_one_direction_only(agent_factory):
+    """A batch plans both directions of its pair.  The agent gathers the commands of one transfer - its senders and
+    their receivers - before it queues them, and must not wait for commands of the opposite direction."""
+    from etha_amd.tensor_bus.agent import _Entry
+    from etha_amd.tensor_bus.commands import Transfer
+
+    agent, naming = agent_factory(6)
+    clients = {r: _client(naming, r, connection_timeout=5) for r in range(6)}
+    src = {r: torch.zeros(8, 16) for r in range(2)}
+    tgt = {r: torch.zeros(16, 4) for r in range(2, 6)}
+
+    def body(r):
+        c = clients[r]
+        if r < 2:
+            c.init_pair("w", "trainer", "inference", 2, device_mesh=torch.arange(2), placements=(Shard(0),), timeout=10)
+            return c.register_tensors("b0", [(src[r], "w")], timeout=10)
+        c.init_pair("w", "inference", "trainer", 4, device_mesh=torch.arange(4), placements=(Shard(1),), timeout=10)
+        return c.register_tensors("b0", [(tgt[r], "w")], timeout=10)
+
+    handlers = run_ranks(body, range(6))  # kept: a handler that goes away cleans its batch up
+    agent._stop.set()
+    agent._serve_thread.join()
+    batch = agent.batches["b0"]
+    assert all(batch.send_buckets[r] and batch.recv_buckets[r] for r in range(6))  # both directions are planned
+    forward = [_Entry(rank=r, conn=None, command=Transfer(batch_id="b0", transfer_type="send" if r < 2 else "recv"))
+               for r in range(6)]
+    for n in range(1, 6):
+        agent._pending = forward[:n]
+        assert agent._siblings_missing(), n
+    agent._pending = forward
+    assert not agent._siblings_missing()
+    backward = [_Entry(rank=r, conn=None, command=Transfer(batch_id="b0", transfer_type="recv" if r < 2 else "send"))
+                for r in range(6)]
+    agent._pending = backward[2:]
+    assert agent._siblings_missing()
+    agent._pending = backward
+    assert not agent._siblings_missing()
+    # a rank that is a generation ahead is not waited for
+    batch.recv_count[5] = 1
+    agent._pending = forward[:5]
+    assert not agent._siblings_missing()
+    agent._pending = []
+    agent._stop.clear()
+    agent.start_in_thread()
+    for h in handlers.values():
+        h.close()
+    for c in clients.values():
+        c.close()
+
+
 def test_partial_target_direction_is_rejected(agent_factory):
     agent, naming = agent_factory(2)
     clients = {r: _client(naming, r, connection_timeout=5) for r in range(2)}
