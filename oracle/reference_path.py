@@ -126,8 +126,12 @@ def bucket_prepare_source(bucket) -> torch.Tensor:
     chunks = bucket.chunks
     if len(chunks) == 1:
         # (flattened before the byte view: the reference's plain .view(torch.uint8) refuses a last dim of one
-        # element that carries a stride other than 1, which torch reports for some slices; the bytes are the same)
-        return chunk_prepare(chunks[0]).contiguous().reshape(-1).view(torch.uint8)
+        # element that carries a stride other than 1, which torch reports for some slices - and for a single
+        # element cut from a .t() view even after flattening; the bytes are the same)
+        flat = chunk_prepare(chunks[0]).contiguous().reshape(-1)
+        if flat.numel() == 1 and flat.stride(0) != 1:
+            flat = flat.as_strided((1,), (1,))
+        return flat.view(torch.uint8)
     offsets = bucket_offsets(bucket)
     total = offsets[-1] + chunks[-1].nbytes
     buffer = torch.empty(total, dtype=torch.uint8)

@@ -63,7 +63,10 @@ def expected_target(spec: TensorSpec, glob: torch.Tensor, rank: int) -> torch.Te
 
 def bits(t: torch.Tensor) -> torch.Tensor:
     """Raw bytes of a tensor, for bit-exact comparison (NaNs and -0 included)."""
-    return t.detach().cpu().contiguous().reshape(-1).view(torch.uint8)  # flat first: a size-1 last dim may carry any stride
+    flat = t.detach().cpu().contiguous().reshape(-1)  # flat first: a size-1 last dim may carry any stride ...
+    if flat.numel() == 1 and flat.stride(0) != 1:  # ... and so may a single element cut from a .t() view
+        flat = flat.as_strided((1,), (1,))
+    return flat.view(torch.uint8)
 
 
 def assert_bit_equal(a: torch.Tensor, b: torch.Tensor, what: str = "") -> None:

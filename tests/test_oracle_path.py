@@ -89,6 +89,21 @@ def test_symmetric_mesh_both_directions():
             assert_bit_equal(t, expected_target(spec, job.globals_[0], r), f"rank {r}")
 
 
+def test_single_element_chunks_of_transposed_shards():
+    """A chunk of one element cut from a ``.t()`` view keeps a stride other than 1 through ``.contiguous()`` and
+    ``reshape(-1)``, which the byte view refuses; the oracle flattens such a chunk itself (found by the GPU sweeps)."""
+    from torch.distributed.tensor.placement_types import Shard
+
+    def transposed(kind, t):
+        return torch.zeros(t.shape[1], t.shape[0], dtype=t.dtype).t() if t.dim() == 2 else torch.zeros_like(t)
+
+    spec = TensorSpec("w", (4, 1), mesh_of(0, [1]), (Shard(1),), mesh_of(1, [4]), (Shard(0),), torch.float32, seed=5, std=1.0)
+    job = ReshardJob([spec], device="cpu", bucket_size=None, keep_globals=True, fill=cpu_fill, local_view=transposed)
+    run_oracle(job)
+    for r, t in job.target_locals[0].items():
+        assert_bit_equal(t, expected_target(spec, job.globals_[0], r), f"rank {r}")
+
+
 @pytest.mark.parametrize("case", [c for c in CASES["reshard"] if not c["slice_view"]],
                          ids=lambda c: f"{c['src_mesh']}{c['src']}->{c['tgt_mesh']}{c['tgt']}")
 @pytest.mark.parametrize("bucket_size", CASES["reshard_bucket_sizes"])
