@@ -30,10 +30,10 @@ from __future__ import annotations
 import json
 import logging
 import os
-import queue
 import threading
 import time
 from dataclasses import dataclass, field
+from multiprocessing.connection import wait as mp_wait
 
 import numpy as np
 import torch
@@ -118,12 +118,12 @@ class TensorBusAgent:
         self.wire.direct_same_device = direct_same_device
         self.pairs: dict[str, PairState] = {}
         self.batches: dict[str, BatchState] = {}
-        self._inbox: queue.Queue = queue.Queue()
+        self._opened: list = []  # (rank, connection) accepted, command not read yet
+        self._rank_of_queue: dict[int, int] = {}
         self._pending: list[_Entry] = []
         self._stop = threading.Event()
         self._queues: dict[int, CommandQueue] = {}
         self._state_paths: dict[int, str] = {}
-        self._threads: list[threading.Thread] = []
         self._last_heartbeat = 0.0
         self._last_core: dict | None = None
         self._moved = False  # set by a command that changed shared state without completing
@@ -136,26 +136,41 @@ class TensorBusAgent:
         for rank in range(world_size):
             cmd_path, state_path = self.path_naming_fn(rank)
             self._queues[rank] = CommandQueue(cmd_path, serve=True)
+            self._rank_of_queue[id(self._queues[rank])] = rank
             self._state_paths[rank] = state_path
-            t = threading.Thread(target=self._accept_loop, args=(rank,), daemon=True)
-            t.start()
-            self._threads.append(t)
         self._write_state(force=True)
 
     # ---- plumbing ---------------------------------------------------------------------------
-    def _accept_loop(self, rank: int) -> None:
-        q = self._queues[rank]
-        while not self._stop.is_set():
+    def _receive(self, timeout: float) -> int:
+        """Wait up to ``timeout`` for commands on any rank's socket and append what has arrived to the pending list;
+        returns how many.  One thread waits on every socket: ten ranks that issue their commands together are taken
+        in one go, without a hand-over between threads per command."""
+        opened = list(self._opened)
+        try:
+            ready = mp_wait(list(self._queues.values()) + [c for _, c in opened], timeout)
+        except OSError:  # a socket was closed under the wait (close() from another thread)
+            return 0
+        got = 0
+        for obj in ready:
+            if isinstance(obj, CommandQueue):
+                rank = self._rank_of_queue[id(obj)]
+                for conn in obj.accept_ready():
+                    self._opened.append((rank, conn))
+        # a worker sends its command right after connecting: most new connections can be read at once
+        for item in list(self._opened):
+            rank, conn = item
             try:
-                conn = q.accept()
-            except (OSError, EOFError):
-                return
-            try:
+                if not conn.poll(0):
+                    continue
                 command = conn.recv()
             except (EOFError, OSError):
+                self._opened.remove(item)
                 conn.close()
                 continue
-            self._inbox.put(_Entry(rank=rank, conn=conn, command=command))
+            self._opened.remove(item)
+            self._pending.append(_Entry(rank=rank, conn=conn, command=command))
+            got += 1
+        return got
 
     def _write_state(self, force: bool = False) -> None:
         """Publish heartbeat and pair/batch state.  ``force`` asks for the current state to be visible on
@@ -190,16 +205,7 @@ class TensorBusAgent:
 
     def step(self, timeout: float = 0.0) -> None:
         self._write_state()
-        try:
-            entry = self._inbox.get(timeout=timeout)
-            self._pending.append(entry)
-        except queue.Empty:
-            pass
-        while True:
-            try:
-                self._pending.append(self._inbox.get_nowait())
-            except queue.Empty:
-                break
+        self._receive(timeout)
         # ranks of one batch issue their commands from threads that take turns: wait while commands keep coming
         # (the window restarts at every arrival), but never longer than eight windows in all
         start = time.perf_counter()
@@ -208,11 +214,8 @@ class TensorBusAgent:
             left = min(deadline, limit) - time.perf_counter()
             if left <= 0:
                 break
-            try:
-                self._pending.append(self._inbox.get(timeout=left))
+            if self._receive(left):
                 deadline = time.perf_counter() + self.gather_window
-            except queue.Empty:
-                break
         # Sweep until nothing moves.  Commands that complete are answered only after the sweep: the device
         # work of every transfer that became ready is enqueued first, then the stream is synchronised once
         # and the state files are written once, instead of once per rank.

@@ -1,11 +1,12 @@
 """End-to-end timing of ``handler.transfer`` through the tensor bus on one GPU.
 
-    python -m etha_amd.tensor_bus.bench_transfer [--workload NAME] [--steps K] [--warmup W] [--zero-copy | --direct]
+    python -m etha_amd.tensor_bus.bench_transfer [--workload NAME] [--steps K] [--warmup W] [--zero-copy | --direct] [--thread-per-rank]
 
-Three processes share the GPU, as in a deployment on one device: this process runs the hub agent,
-a "trainer" worker process holds every source rank's shards and a "inference" worker process
-holds every target rank's shards (one thread per rank in both).  Workers register their tensors over
-hipIPC once (``register_tensors``) and then repeat ``transfer("send")`` / ``transfer("recv")``.
+This process runs the hub agent; every source rank ("trainer") and every target rank ("inference") is a worker
+process of its own on the same GPU, as the reference's workers are (``--thread-per-rank``: one worker process per
+side with a thread per rank instead - the rank threads then issue their commands one after the other).  Workers
+register their tensors over hipIPC once (``register_tensors``) and then repeat ``transfer("send")`` /
+``transfer("recv")``.
 One step is timed on the host wall clock from the moment the first source rank issues its send to
 the moment the last target rank's blocking recv returns, so it includes the command round trips,
 the agent's launches and the device work.  After the last step every same-dtype tensor is verified by a
@@ -48,8 +49,10 @@ def _pairs(specs):
     return names, {n: s for n, s in first.values()}
 
 
-def _worker(role: str, workload: str, tmpdir: str, device: str, steps: int, warmup: int, out_q) -> None:
-    """Body of a worker process: every rank of one side, one thread per rank."""
+def _worker(role: str, workload: str, tmpdir: str, device: str, steps: int, warmup: int, out_q, only_rank=None,
+            shared_barrier=None) -> None:
+    """Body of a worker process: every rank of one side, one thread per rank - or, with ``only_rank``, that rank
+    alone (one process per rank, as in a deployment; ``shared_barrier`` then lines the processes of a side up)."""
     try:
         import torch
 
@@ -64,6 +67,8 @@ def _worker(role: str, workload: str, tmpdir: str, device: str, steps: int, warm
         naming = _naming(tmpdir)
         source = role == "trainer"
         my_ranks = sorted({int(r) for s in specs for r in np.asarray(s.source_mesh if source else s.target_mesh).reshape(-1)})
+        if only_rank is not None:
+            my_ranks = [r for r in my_ranks if r == only_rank]
         shards: dict[int, list] = {r: [] for r in my_ranks}
         gen = torch.Generator(device=device)
         for i, s in enumerate(specs):
@@ -71,6 +76,8 @@ def _worker(role: str, workload: str, tmpdir: str, device: str, steps: int, warm
             placements = s.source_placements if source else s.target_placements
             dtype = s.source_dtype if source else (s.target_dtype or s.source_dtype)
             for pos, r in enumerate(int(x) for x in mesh.reshape(-1)):
+                if r not in shards:
+                    continue
                 shape = local_shape(s.shape, mesh.shape, placements, mesh_coord(mesh.shape, pos))
                 if source:  # values are irrelevant to timing; seeded so that runs repeat
                     gen.manual_seed(1000 * i + r)
@@ -79,7 +86,7 @@ def _worker(role: str, workload: str, tmpdir: str, device: str, steps: int, warm
                     t = torch.zeros(shape, dtype=dtype, device=device)
                 shards[r].append((t, pair_names[i]))
         torch.cuda.synchronize()
-        barrier = threading.Barrier(len(my_ranks))
+        barrier = shared_barrier if shared_barrier is not None else threading.Barrier(len(my_ranks))
         stamps = {r: [] for r in my_ranks}
         errors = []
 
@@ -124,6 +131,8 @@ def _worker(role: str, workload: str, tmpdir: str, device: str, steps: int, warm
                     sums[i] += int(t.contiguous().view(raw[t.element_size()]).sum(dtype=torch.int64).item())
         out_q.put((role, "ok", {"stamps": stamps, "bytes": nbytes, "ranks": my_ranks, "checksums": sums}))
     except BaseException:
+        if shared_barrier is not None:
+            shared_barrier.abort()
         out_q.put((role, "error", traceback.format_exc()))
 
 
@@ -134,6 +143,9 @@ def main() -> None:
     ap.add_argument("--warmup", type=int, default=2)
     ap.add_argument("--zero-copy", action="store_true", help="lend contiguous single-chunk buckets (agent option)")
     ap.add_argument("--direct", action="store_true", help="no bucket buffers: receivers copy from the senders' tensors")
+    ap.add_argument("--thread-per-rank", action="store_true",
+                    help="one worker process per side with a thread per rank, instead of a process per rank "
+                         "(taken anyway when the workload has more than 12 ranks)")
     ap.add_argument("--device", default="cuda:0")
     args = ap.parse_args()
 
@@ -160,13 +172,21 @@ def main() -> None:
     agent.start_in_thread()
     ctx = mp.get_context("spawn")
     out_q = ctx.Queue()
-    procs = [ctx.Process(target=_worker, args=(role, args.workload, tmpdir, args.device, args.steps, args.warmup, out_q))
-             for role in ("trainer", "inference")]
+    if not args.thread_per_rank and len(src_ranks) + len(tgt_ranks) <= 12:
+        # the ranks of a side start a step together: one barrier per side, shared by its processes
+        barriers = {"trainer": ctx.Barrier(len(src_ranks)), "inference": ctx.Barrier(len(tgt_ranks))}
+        procs = [ctx.Process(target=_worker, args=(role, args.workload, tmpdir, args.device, args.steps, args.warmup, out_q, r,
+                                                   barriers[role]))
+                 for role, ranks in (("trainer", src_ranks), ("inference", tgt_ranks)) for r in sorted(ranks)]
+    else:
+        procs = [ctx.Process(target=_worker, args=(role, args.workload, tmpdir, args.device, args.steps, args.warmup, out_q))
+                 for role in ("trainer", "inference")]
     for p in procs:
         p.start()
     results = {}
     try:
-        while len(results) < 2:
+        answered = 0
+        while answered < len(procs):
             try:
                 role, status, payload = out_q.get(timeout=1.0)
             except Exception:
@@ -175,7 +195,15 @@ def main() -> None:
                 continue
             if status != "ok":
                 raise RuntimeError(f"{role} failed:\n{payload}")
-            results[role] = payload
+            answered += 1
+            if role not in results:
+                results[role] = payload
+            else:  # another rank of the same side
+                mine = results[role]
+                mine["stamps"].update(payload["stamps"])
+                mine["bytes"] += payload["bytes"]
+                mine["ranks"] = sorted(mine["ranks"] + payload["ranks"])
+                mine["checksums"] = [a + b for a, b in zip(mine["checksums"], payload["checksums"])]
     finally:
         for p in procs:
             p.join(timeout=30)
@@ -215,13 +243,13 @@ def main() -> None:
     med = lat[len(lat) // 2]
     payload = results["inference"]["bytes"]
     print(json.dumps({
-        "metric": "end-to-end handler.transfer through the tensor bus, three processes on one GPU",
+        "metric": "end-to-end handler.transfer through the tensor bus, agent and worker processes on one GPU",
         "value": payload / med / 1e9, "unit": "GB/s", "ms_per_transfer": med * 1e3, "min_ms": lat[0] * 1e3,
         "steps": args.steps, "warmup": args.warmup, "payload_bytes": payload,
         "ms_between_first_and_last_rank_command": spread[len(spread) // 2] * 1e3,
         "config": {"workload": args.workload, "source_ranks": len(results["trainer"]["ranks"]),
                    "target_ranks": len(results["inference"]["ranks"]), "zero_copy_single_chunk": args.zero_copy,
-                   "direct_same_device": args.direct},
+                   "direct_same_device": args.direct, "worker_processes": len(procs)},
         "agent": agent_stats, "tensors_verified_by_checksum": verified,
     }))
 

@@ -12,10 +12,11 @@ from __future__ import annotations
 
 import os
 import pickle
+import socket
 import sqlite3
 import threading
 import time
-from multiprocessing.connection import Client, Connection, Listener
+from multiprocessing.connection import Client, Connection
 
 
 class BusyError(Exception):
@@ -64,17 +65,21 @@ class Completion:
 
 class CommandQueue:
     """``CommandQueue(path)`` on the worker side enqueues; ``CommandQueue(path, serve=True)`` on the
-    agent side accepts connections."""
+    agent side accepts connections.  The serving side is a plain non-blocking listening socket: the agent waits on
+    the sockets of all its ranks at once (``fileno``) and takes what has arrived (``accept_ready``)."""
 
     def __init__(self, path: str, serve: bool = False):
         if path is None:
             raise ValueError("command queue path is required")
         self.path = path
-        self._listener: Listener | None = None
+        self._socket: socket.socket | None = None
         if serve:
             if os.path.exists(path):
                 os.unlink(path)
-            self._listener = Listener(address=path, family="AF_UNIX")
+            self._socket = socket.socket(socket.AF_UNIX, socket.SOCK_STREAM)
+            self._socket.bind(path)
+            self._socket.listen(128)
+            self._socket.setblocking(False)
 
     # worker side
     def enqueue(self, command) -> Completion:
@@ -91,17 +96,27 @@ class CommandQueue:
         return Completion(conn, getattr(command, "semaphore_name", None) or "command")
 
     # agent side
-    @property
-    def listener(self) -> Listener:
-        return self._listener
+    def fileno(self) -> int:
+        return self._socket.fileno()
 
-    def accept(self) -> Connection:
-        return self._listener.accept()
+    def accept_ready(self) -> list[Connection]:
+        """The connections that are waiting to be accepted, without blocking (possibly none)."""
+        out = []
+        while self._socket is not None:
+            try:
+                s, _ = self._socket.accept()
+            except (BlockingIOError, InterruptedError):
+                break
+            except OSError:
+                break
+            s.setblocking(True)
+            out.append(Connection(s.detach()))
+        return out
 
     def close(self) -> None:
-        if self._listener is not None:
-            self._listener.close()
-            self._listener = None
+        if self._socket is not None:
+            self._socket.close()
+            self._socket = None
             if os.path.exists(self.path):
                 try:
                     os.unlink(self.path)
