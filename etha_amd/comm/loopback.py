@@ -16,8 +16,9 @@ its previous bucket has unpacked, so senders and receivers advance together: the
 pipelines (:class:`etha_amd.comm.comm_methods.Program`) of every rank that has called ``bucket_comm``
 and steps them in turn, the single-process form of the ranks' concurrent ``bucket_comm`` loops.
 ``pool="resident"`` gives every bucket a slot of its own for the life of its plan (pool = payload);
-that form allows one launch over many buckets, side streams, graph capture and exporting the pool to
-another process.
+that form allows one launch over many buckets, side streams and graph capture.  Either form can be exported to a
+consumer in another process (``export_manifest`` / ``from_manifest``); a ring's slots then change hands through
+"packed" / "unpacked" notifications (``exchange``).
 
 Matching follows the point-to-point rule of the reference's transports: the k-th bucket a rank
 sends on a wire key ``(src_rank, dst_ranks, transport)`` is the k-th bucket each of its peers
@@ -374,8 +375,8 @@ class LoopbackWire:
         """Describe every planned send slot so that another process on the same GPU can consume it.
 
         Pool segments are exported with ``hipIpcGetMemHandle`` (allocation base + offset); a slot is
-        ``(segment, offset)``.  The producer sends this once, after planning; afterwards only
-        "generation n is packed" notifications are needed per transfer.
+        ``(segment, offset)``.  The producer sends this once, after planning.  Per transfer a resident pool needs
+        one "packed" notification; a ring's two ends trade notifications while the transfer runs (``exchange``).
         """
         from .. import _native as nat
 
