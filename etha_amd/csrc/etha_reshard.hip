@@ -532,12 +532,50 @@ __device__ __forceinline__ void tile_body(const RunTile* __restrict__ run_tiles,
   move_unit<REV>(meta, a, b);
 }
 
+// A wave fetches its tile entry before it can do anything else, and an entry that has to come from HBM doubles the
+// wave's life.  The entries are read once, in order, so a few waves fetch ahead for all the others: of every 4096
+// workgroups (256 tiles) the first eight - one per XCD, as workgroups are dealt to the XCDs in turn - touch, after
+// their own work, the lines that hold the entries of the 256 tiles kPrefetchGroups groups further on, each lane one
+// line per step, so that those are in the XCD's L2 when their workgroups start (more than the 512 tiles in flight at
+// a time lie between).  The eight of the first group also touch what lies before that.  Only these eight waves wait
+// for what they fetch.
+// Measured: converting packs, whose workgroups are issued faster than a copy's, gain 3 points of the HBM peak
+// (fp32 -> bf16 of the Llama shapes: 79.2 -> 82.3 %), plain copies half a point.  The plain tile kernels only: in the
+// gather and mixed kernels the same step cost 1.5 points, in the reduce kernel it changed nothing.
+#ifndef ETHA_PREFETCH_GROUPS
+#define ETHA_PREFETCH_GROUPS 4
+#endif
+constexpr uint32_t kPrefetchGroups = ETHA_PREFETCH_GROUPS, kPrefetchTiles = 4096u / kBlocksPerTile;
+// every 128-byte line that holds bytes of [lo, hi), one line per lane and step.  Ordinary loads, so that the compiler
+// knows which registers they write and when (a load issued from inline asm returns into a register the compiler
+// already considers free); the values are folded into `seen`, which the caller keeps alive to the end.
+__device__ __forceinline__ void touch_lines(uint64_t lo, uint64_t hi, uint32_t& seen) {
+  for (uint64_t line = (lo & ~(uint64_t)127) + (uint64_t)threadIdx.x * 128u; line < hi; line += kBlockThreads * 128u)
+    seen ^= *reinterpret_cast<const ETHA_GLOBAL uint32_t*>(line);
+}
+// tiles are counted run tiles first, then row tiles, as tile_body takes them
+__device__ __forceinline__ void prefetch_entries(const RunTile* run_tiles, uint32_t n_run, const RowTile* row_tiles,
+                                                 uint32_t n_tiles) {
+  if (kPrefetchGroups == 0 || (blockIdx.x & 4095u) >= 8u) return;
+  const uint32_t group = blockIdx.x >> 12;
+  uint32_t first = group == 0 ? kPrefetchTiles : (group + kPrefetchGroups) * kPrefetchTiles;
+  uint32_t last = (group + kPrefetchGroups + 1) * kPrefetchTiles;
+  first = first < n_tiles ? first : n_tiles;
+  last = last < n_tiles ? last : n_tiles;
+  uint32_t seen = 0;
+  if (first < n_run) touch_lines((uint64_t)(run_tiles + first), (uint64_t)(run_tiles + (last < n_run ? last : n_run)), seen);
+  if (last > n_run)
+    touch_lines((uint64_t)(row_tiles + ((first > n_run ? first : n_run) - n_run)), (uint64_t)(row_tiles + (last - n_run)), seen);
+  asm volatile("" ::"v"(seen));  // the loads are performed although nothing uses what they return
+}
+
 template <bool REV>
 __global__ __launch_bounds__(ETHA_BLOCK_THREADS) void etha_tile_kernel(const RunTile* __restrict__ run_tiles, uint32_t n_run,
                                                                         const RowTile* __restrict__ row_tiles,
                                                                         const uint64_t* __restrict__ gather) {
   tile_body<REV>(run_tiles, n_run, row_tiles, gather, blockIdx.x / kBlocksPerTile,
                  (blockIdx.x % kBlocksPerTile) * kBlockThreads + threadIdx.x);
+  prefetch_entries(run_tiles, n_run, row_tiles, gridDim.x / kBlocksPerTile);
 }
 
 // Several chunk ranges of one direction in one launch: blockIdx.y picks the range, blockIdx.x walks its tiles
@@ -569,6 +607,7 @@ __global__ __launch_bounds__(ETHA_BLOCK_THREADS) void etha_tile_kernel_2d(const 
   const RowTile* row = (const RowTile*)(GlobalRow)(((uint64_t)raw[3] << 32) | raw[2]);
   const uint64_t* gather = (const uint64_t*)(GlobalU64)(((uint64_t)raw[5] << 32) | raw[4]);
   tile_body<REV>(run, raw[6], row, gather, bid, (blockIdx.x % kBlocksPerTile) * kBlockThreads + threadIdx.x);
+  prefetch_entries(run, raw[6], row, raw[7]);
 }
 
 // The gather tiles of write-ordered unpack ranges (see kMetaGather).  Consecutive 1 KiB pieces of such a tile read
