@@ -14,6 +14,7 @@ import os
 import pickle
 import socket
 import sqlite3
+import struct
 import threading
 import time
 from multiprocessing.connection import Client, Connection
@@ -110,6 +111,9 @@ class CommandQueue:
             except OSError:
                 break
             s.setblocking(True)
+            # the agent reads a command only once part of it has arrived; a sender that stalls in mid-message holds
+            # the agent's one serving thread for at most this long (the read then fails and the connection is dropped)
+            s.setsockopt(socket.SOL_SOCKET, socket.SO_RCVTIMEO, struct.pack("ll", 1, 0))
             out.append(Connection(s.detach()))
         return out
 

@@ -92,6 +92,36 @@ def test_init_pair_register_and_errors_on_cpu(agent_factory):
         c.close()
 
 
+def test_idle_and_broken_connections_do_not_stall_the_agent(agent_factory):
+    """One thread of the agent serves every rank's socket: a connection that never sends its command, or goes away
+    before it has, must not keep the others waiting."""
+    import socket
+
+    agent, naming = agent_factory(2)
+    idle = socket.socket(socket.AF_UNIX, socket.SOCK_STREAM)
+    idle.connect(naming(0)[0])  # connected, silent
+    gone = socket.socket(socket.AF_UNIX, socket.SOCK_STREAM)
+    gone.connect(naming(1)[0])
+    gone.close()  # connected, closed without a command
+    half = socket.socket(socket.AF_UNIX, socket.SOCK_STREAM)
+    half.connect(naming(1)[0])
+    half.sendall(b"\x00\x00")  # two of the four bytes of a message header, then nothing
+    half.close()
+    stalled = socket.socket(socket.AF_UNIX, socket.SOCK_STREAM)
+    stalled.connect(naming(1)[0])
+    stalled.sendall(b"\x00\x00")  # the same, but the sender stays: the agent gives such a read one second
+    client = _client(naming, 0, connection_timeout=5)
+    t0 = time.time()
+    with pytest.raises(ValueError, match="unknown batch"):
+        client.transfer("never_registered", "send", blocking=True, timeout=5)
+    assert time.time() - t0 < 3.0
+    idle.close()
+    stalled.close()
+    with pytest.raises(ValueError, match="unknown batch"):
+        client.transfer("never_registered", "recv", blocking=True, timeout=5)
+    client.close()
+
+
 def test_the_agent_waits_for_the_ranks_of_one_direction_only(agent_factory):
     """A batch plans both directions of its pair.  The agent gathers the commands of one transfer - its senders and
     their receivers - before it queues them, and must not wait for commands of the opposite direction."""
