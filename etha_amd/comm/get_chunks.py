@@ -68,8 +68,11 @@ def _side_slicers(tensor, num_slicers, this_mesh, this_pl, other_mesh, other_pl,
 
 
 def _partial_signature(m2m: M2MMap, src_rank: int) -> tuple:
-    """``((member ranks), op)`` of the Partial reduction ``src_rank`` takes part in, as one group over the
-    whole connected component - the form ``etha_amd.world.create_partial_groups`` builds on the sending side."""
+    """``((member ranks), op, levels)`` of the Partial reduction ``src_rank`` takes part in, as one group over the
+    whole connected component - what ``Chunk.partial_signature`` gives for the group that
+    ``etha_amd.world.create_partial_groups`` builds on the sending side.  Two reductions over the same ranks with the
+    same ops are still different groups when their mesh dims nest differently (sum over 2 then avg over 3, against
+    sum over 3 then avg over 2): the sender keeps their chunks in separate buckets, so the receiver must too."""
     if not m2m.source_partial_reductions or m2m.source_mesh is None:
         return ()
     import numpy as np
@@ -81,10 +84,14 @@ def _partial_signature(m2m: M2MMap, src_rank: int) -> tuple:
     index: list = [int(c) for c in where[0]]
     for mesh_dim, _ in m2m.source_partial_reductions:
         index[mesh_dim] = slice(None)
-    ranks = tuple(sorted(int(r) for r in np.asarray(mesh[tuple(index)]).reshape(-1)))
+    members = np.asarray(mesh[tuple(index)])  # one axis per Partial mesh dim, in mesh-dim order
     ops = [op for _, op in sorted(m2m.source_partial_reductions)]
-    # one op, or one per Partial mesh dim: either way chunks of this reduction only bundle with each other
-    return ((ranks, ops[0] if len(set(ops)) == 1 else "+".join(ops)),)
+    if len(set(ops)) == 1:
+        return ((tuple(sorted(int(r) for r in members.reshape(-1))), ops[0], ()),)
+    # one op per Partial mesh dim: members in level order (first Partial mesh dim fastest), and the levels themselves
+    ranks = tuple(int(r) for r in members.transpose().reshape(-1))
+    levels = tuple((str(op), int(n)) for op, n in zip(ops, members.shape))
+    return ((ranks, "+".join(ops), levels),)
 
 
 def _shape_of(slices: tuple[slice, ...]) -> tuple[int, ...]:

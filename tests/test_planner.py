@@ -158,7 +158,37 @@ def test_partial_and_plain_tensors_bucket_alike_on_both_ends():
     send_b = [b for b in chunk_to_bucket_ops(send, 1 << 30) if b.dst_ranks]
     recv_b = [b for b in chunk_to_bucket_ops(recv, 1 << 30) if b.src_rank == 0]
     assert [[c.nbytes for c in b.chunks] for b in send_b] == [[c.nbytes for c in b.chunks] for b in recv_b]
-    assert len(send_b) == 2 and recv_b[1].chunks[0].source_partial_signature == (((0, 1), "sum"),)
+    assert len(send_b) == 2 and recv_b[1].chunks[0].source_partial_signature == (((0, 1), "sum", ()),)
+    # the receive chunks name the group exactly as the send chunks do
+    assert recv_b[1].chunks[0].partial_signature == send_b[1].chunks[0].partial_signature
+
+
+def test_partial_reductions_that_nest_differently_bucket_alike_on_both_ends():
+    """Two Partial tensors over the same six ranks with the same two ops, but sum over 2 then avg over 3 in one and sum
+    over 3 then avg over 2 in the other: different groups, so the sender keeps their chunks in separate buckets, and
+    the receiver has to split the channel the same way (found by a sweep of random batches on the GPU)."""
+    from etha_amd.world import create_partial_groups
+
+    mesh_a, mesh_b = np.arange(6).reshape(2, 3), np.arange(6).reshape(3, 2)
+    pl = (Partial("sum"), Partial("avg"))
+    maps = [get_m2m_map(mesh_a, pl, [6], (Replicate(),)), get_m2m_map(mesh_b, pl, [6], (Replicate(),))]
+    src = [{r: torch.empty(4, 8, device="meta") for r in range(6)} for _ in maps]
+    tgt = torch.empty(4, 8, device="meta")
+    send_keys, recv_keys = [], []
+    for r in range(6):
+        send = []
+        for m, mesh, tensors in zip(maps, (mesh_a, mesh_b), src):
+            groups = create_partial_groups(mesh, m.source_partial_reductions, r, tensors)
+            send += m2m_to_chunks(m, r, source_tensor=tensors[r], source_partial_groups=groups)
+        send_b = [b for b in chunk_to_bucket_ops(send, 1 << 30) if b.dst_ranks]
+        recv = [c for m in maps for c in m2m_to_chunks(m, 6, target_tensor=tgt)]
+        recv_b = [b for b in chunk_to_bucket_ops(recv, 1 << 30) if b.src_rank == r]
+        assert [[c.nbytes for c in b.chunks] for b in send_b] == [[c.nbytes for c in b.chunks] for b in recv_b], r
+        for sb, rb in zip(send_b, recv_b):
+            assert sb.chunks[0].partial_signature == rb.chunks[0].partial_signature
+        send_keys += [b.chunks[0].partial_signature for b in send_b]
+        recv_keys += [b.chunks[0].partial_signature for b in recv_b]
+    assert len(set(send_keys)) == 2 and send_keys == recv_keys  # the rank that ships the reduced chunks has one bucket per group
 
 
 def test_strided_shard_grids():
